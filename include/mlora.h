@@ -1,0 +1,222 @@
+/*
+ * mlora.h — C-ABI of the MI355X (gfx950) multi-LoRA batched apply library.
+ *
+ * One shared library, plain pointers and sizes, no torch types.  Every entry
+ * point enqueues work on the HIP stream it is given and returns without
+ * synchronising, so all of them are legal under HIP graph capture.  Device
+ * pointers are borrowed for the duration of the enqueued work only.
+ *
+ * Return value of every int-returning entry point: 0 on success, a negative
+ * MLORA_E_* code for an argument the library rejects before launching
+ * anything, or a positive hipError_t when a launch failed.  The text of the
+ * last failure on the calling thread is available from mlora_last_error().
+ *
+ * Weight layout is the reference's: A_i is [slots, r, K] contiguous (K
+ * fastest), B_i is [slots, N_i, r] contiguous (r fastest)
+ * (reference: nanovllm_voxcpm/layers/lora.py:289-297,507-511,703-705,828-829).
+ */
+#ifndef MLORA_H_
+#define MLORA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLORA_ABI_VERSION 1
+
+/* element types of x / y / A / B */
+#define MLORA_DTYPE_F32 0
+#define MLORA_DTYPE_F16 1
+#define MLORA_DTYPE_BF16 2
+
+/* which kernel family mlora_add_lora uses */
+#define MLORA_FORM_AUTO 0  /* library chooses from shapes and the plan */
+#define MLORA_FORM_TOKEN 1 /* one workgroup per token, any shape or dtype; needs no plan */
+#define MLORA_FORM_BGMV 2  /* segment tiles of <= 8 tokens, wave64 dot-product reductions */
+#define MLORA_FORM_SGMV 3  /* MFMA tiles for segments >= threshold, BGMV tiles for the rest */
+#define MLORA_FORM_MFMA 4  /* MFMA tiles for every segment */
+
+/* error codes (negative) */
+#define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
+#define MLORA_E_UNSUPPORTED (-2) /* well-formed but outside what the selected form handles */
+#define MLORA_E_TOO_LARGE (-3)   /* exceeds a compile-time capacity (slices, slots, rank) */
+
+#define MLORA_MAX_SLICES 8
+#define MLORA_MAX_SLOTS 1024 /* valid slot ids are [0, max_slots), max_slots <= this */
+#define MLORA_MAX_RANK 256
+
+/* One LoRA-wrapped slice of a stacked projection (q / k / v, gate / up, or
+ * the only slice of o / down).  Replaces the per-slice pointer, stride and
+ * column-start tables the reference uploads to the device
+ * (reference: nanovllm_voxcpm/lora_ops/triton_ops/utils.py:15-116). */
+typedef struct MloraSlice {
+  const void* a;      /* A_i: [slots, r, K] contiguous */
+  const void* b;      /* B_i: [slots, n, r] contiguous */
+  int32_t n;          /* output columns of this slice */
+  int32_t y_col;      /* first column of this slice inside y */
+} MloraSlice;
+
+/* Arguments of the fused apply:  for every token t with s = token_to_slot[t] >= 0
+ * and every slice i:  y[t, y_col_i : y_col_i + n_i] += scaling * (x[t] . A_i[s]^T) . B_i[s]^T
+ * with fp32 accumulation and a single rounding to the element type.  Rows with
+ * s < 0 are not touched.
+ * Replaces LoRABackend.add_lora (reference: nanovllm_voxcpm/lora.py:43-54, body
+ * :241-381) including its shrink/expand grouping (:195-239, :299-381). */
+typedef struct MloraAddArgs {
+  void* stream;           /* hipStream_t */
+  const void* x;          /* [T, K], row stride x_stride elements, unit column stride */
+  void* y;                /* [T, >= max(y_col_i + n_i)], row stride y_stride elements */
+  int64_t x_stride;
+  int64_t y_stride;
+  const int32_t* token_to_slot; /* [T] on device */
+  const int32_t* plan;    /* workspace filled by mlora_plan_build for this token_to_slot, or NULL
+                             (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it) */
+  int32_t num_tokens;     /* T */
+  int32_t k;              /* K, input features */
+  int32_t r;              /* rank dimension of the A/B buffers (max_lora_rank) */
+  int32_t num_slots;      /* first dimension of A_i / B_i */
+  int32_t num_slices;     /* <= MLORA_MAX_SLICES */
+  int32_t dtype;          /* MLORA_DTYPE_* of x, y, A and B */
+  int32_t form;           /* MLORA_FORM_* */
+  float scaling;
+  MloraSlice slices[MLORA_MAX_SLICES];
+} MloraAddArgs;
+
+int mlora_add_lora(const MloraAddArgs* args);
+
+/* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0
+ * for rows with s_t < 0 (the reference zero-fills the buffer first).
+ * Replaces lora_shrink (reference:
+ * nanovllm_voxcpm/lora_ops/triton_ops/lora_shrink_op.py:257-341). */
+typedef struct MloraShrinkArgs {
+  void* stream;
+  const void* x;          /* [T, K] */
+  void* out;              /* [S, T, r] contiguous, element type out_dtype */
+  int64_t x_stride;
+  const int32_t* token_to_slot;
+  int32_t num_tokens, k, r, num_slots, num_slices;
+  int32_t dtype;          /* of x and A */
+  int32_t out_dtype;      /* of out */
+  float scaling;
+  const void* a[MLORA_MAX_SLICES];
+} MloraShrinkArgs;
+
+int mlora_shrink(const MloraShrinkArgs* args);
+
+/* Unfused expand:  y[t, c_i : c_i + n_i] (+)= h[i, t] . B_i[s_t]^T for s_t >= 0 where
+ * c_i = offset_start + n_0 + ... + n_{i-1}.  The product is rounded to B's element type
+ * before it is added (add_inputs != 0) or stored (add_inputs == 0), as the reference does.
+ * Replaces lora_expand (reference:
+ * nanovllm_voxcpm/lora_ops/triton_ops/lora_expand_op.py:94-170). */
+typedef struct MloraExpandArgs {
+  void* stream;
+  const void* h;          /* [S, T, r] contiguous, element type h_dtype */
+  void* y;                /* [T, *], row stride y_stride elements, element type dtype */
+  int64_t y_stride;
+  const int32_t* token_to_slot;
+  int32_t num_tokens, r, num_slots, num_slices;
+  int32_t dtype;          /* of B and y */
+  int32_t h_dtype;
+  int32_t offset_start;
+  int32_t add_inputs;
+  const void* b[MLORA_MAX_SLICES];
+  int32_t n[MLORA_MAX_SLICES];
+} MloraExpandArgs;
+
+int mlora_expand(const MloraExpandArgs* args);
+
+/* ---- segment metadata built on the device from the slot-id vector ------------------ */
+
+/* Bytes of plan workspace needed for num_tokens tokens and max_slots slots. */
+size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
+
+/* Header words of a plan workspace (int32 index). */
+#define MLORA_PLAN_MAGIC 0
+#define MLORA_PLAN_NUM_TOKENS 1
+#define MLORA_PLAN_MAX_SLOTS 2
+#define MLORA_PLAN_NUM_LORA_TOKENS 3 /* tokens with a valid slot */
+#define MLORA_PLAN_NUM_ACTIVE 4      /* distinct valid slots in use */
+#define MLORA_PLAN_NO_LORA 5         /* 1 iff no token has a valid slot */
+#define MLORA_PLAN_BAD_SLOT 6        /* 1 iff some slot id was >= max_slots (treated as -1) */
+#define MLORA_PLAN_TILES_SHORT 7     /* small tiles of segments below the threshold */
+#define MLORA_PLAN_TILES_LONG_SMALL 8 /* small tiles of segments at or above the threshold */
+#define MLORA_PLAN_TILES_LONG_BIG 9  /* big tiles of segments at or above the threshold */
+#define MLORA_PLAN_MAX_SEGMENT 10    /* longest segment */
+#define MLORA_PLAN_HEADER_WORDS 16
+#define MLORA_PLAN_MAGIC_VALUE 0x4d4c5031 /* "MLP1" */
+
+/* Segment length from which a segment gets MFMA tiles, and the two tile heights. */
+#define MLORA_SEGMENT_THRESHOLD 16
+#define MLORA_TILE_SMALL 8
+#define MLORA_TILE_BIG 64
+
+/* Arguments of the on-device metadata build: a stable counting sort of the tokens by
+ * slot id.  The plan workspace (always written when non-NULL) feeds mlora_add_lora; the
+ * optional outputs reproduce, bit for bit, the three index layouts the reference builds
+ * on the host:
+ *   compact, -1 left out   — engine path (reference: nanovllm_voxcpm/engine/lora_manager.py:77-91)
+ *                            and torch builder (nanovllm_voxcpm/utils/context.py:77-116)
+ *   compact, -1 as a bucket — LoRAKernelMeta.prepare_tensors
+ *                            (nanovllm_voxcpm/lora_ops/triton_ops/lora_kernel_metadata.py:46-68)
+ *   dense by slot id        — graph buffers (nanovllm_voxcpm/engine/model_runner.py:743-797)
+ * Any output pointer may be NULL. */
+typedef struct MloraMetaArgs {
+  void* stream;
+  const int32_t* token_to_slot; /* [T] on device */
+  int32_t num_tokens;           /* T */
+  int32_t max_slots;            /* L <= MLORA_MAX_SLOTS */
+  int32_t no_lora_bucket;       /* 0: tokens with slot -1 are left out of every output;
+                                   1: they form the first bucket (id -1) of sorted_idx and the
+                                      compact arrays (not of the plan) */
+  int32_t* plan;                /* mlora_plan_workspace_bytes(T, L) bytes, or NULL */
+  int32_t* sorted_idx;          /* token indices grouped by slot, ascending inside a slot */
+  int32_t* compact_ids;         /* [compact_capacity], unused tail filled with -1 */
+  int32_t* compact_counts;      /* [compact_capacity], unused tail filled with 0 */
+  int32_t* compact_offsets;     /* [compact_capacity + 1]: 0, running totals, unused tail 0 */
+  int32_t compact_capacity;
+  int32_t* dense_counts;        /* [L + 1], index slot + 1; entry 0 (slot -1) is always 0 */
+  int32_t* dense_offsets;       /* [L + 2]: 0 followed by the running totals of dense_counts */
+  int32_t* padded_token_to_slot; /* [padded_len]: copy of token_to_slot, tail filled with -1 */
+  int32_t padded_len;
+  int32_t* scalars;             /* [4]: number of buckets written to the compact arrays, number
+                                   of entries written to sorted_idx, no_lora flag, bad_slot flag */
+} MloraMetaArgs;
+
+int mlora_meta_build(const MloraMetaArgs* args);
+
+/* Fused slot install:  A[slot, :, :] = 0; A[slot, 0:rank, :] = a_src[0:rank, :];
+ * B[slot, :, :] = 0; B[slot, :, 0:rank] = b_src[:, 0:rank] * scaling  in one launch.
+ * Replaces the zero / copy / scale sequence of set_slot_lora
+ * (reference: nanovllm_voxcpm/layers/lora.py:395-417, 599-621, 744-762, 851-869). */
+typedef struct MloraInstallArgs {
+  void* stream;
+  void* a_dst;            /* [slots, r, K] */
+  void* b_dst;            /* [slots, n, r] */
+  const void* a_src;      /* [>= rank, K], row stride a_src_stride elements */
+  const void* b_src;      /* [n, >= rank], row stride b_src_stride elements */
+  int64_t a_src_stride, b_src_stride;
+  int32_t slot, k, n, r, rank;
+  int32_t dtype;          /* of the destination buffers */
+  int32_t src_dtype;      /* of a_src and b_src */
+  float scaling;
+} MloraInstallArgs;
+
+int mlora_install_slot(const MloraInstallArgs* args);
+
+/* Identifier of the graph capture in progress on `stream`, 0 when the stream is not
+ * capturing.  No counterpart in the reference: lets a host-side cache tell work recorded
+ * into one capture from work run eagerly or recorded into another capture. */
+uint64_t mlora_stream_capture_id(void* stream);
+
+/* Library identification and diagnostics. */
+int mlora_abi_version(void);
+const char* mlora_last_error(void);
+const char* mlora_build_info(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLORA_H_ */

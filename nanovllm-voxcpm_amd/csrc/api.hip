@@ -1,0 +1,132 @@
+// C-ABI front door: argument checks, form selection, error text.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "common.h"
+#include "launch.h"
+
+namespace mlora {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return static_cast<int>(e);
+  }
+  return 0;
+}
+
+int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  if (!v || !*v) return fallback;
+  return atoi(v);
+}
+
+}  // namespace mlora
+
+using namespace mlora;
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// The vectorised kernels move eight 16-bit elements per lane: every row they touch has to
+// start on a 16-byte boundary.
+bool vector_ok(const MloraAddArgs* a) {
+  if (a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) return false;
+  if (!a->plan) return false;
+  if (a->r != 8 && a->r != 16 && a->r != 32 && a->r != 64) return false;
+  if (a->k % 8 || a->x_stride % 8 || a->y_stride % 8) return false;
+  if (!aligned16(a->x) || !aligned16(a->y)) return false;
+  for (int i = 0; i < a->num_slices; ++i) {
+    const MloraSlice& s = a->slices[i];
+    if (s.n % 8 || s.y_col % 8 || !aligned16(s.a) || !aligned16(s.b)) return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+extern "C" int mlora_add_lora(const MloraAddArgs* a) {
+  if (!a) { set_error("mlora_add_lora: NULL args"); return MLORA_E_INVALID; }
+  if (a->num_tokens < 0 || a->k < 0 || a->r < 0 || a->num_slots < 0 || a->num_slices < 0) {
+    set_error("mlora_add_lora: negative size"); return MLORA_E_INVALID;
+  }
+  if (a->dtype != MLORA_DTYPE_F32 && a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) {
+    set_error("mlora_add_lora: unknown dtype %d", a->dtype); return MLORA_E_INVALID;
+  }
+  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_MFMA) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
+  if (a->num_slices > MLORA_MAX_SLICES) { set_error("mlora_add_lora: %d slices exceed %d", a->num_slices, MLORA_MAX_SLICES); return MLORA_E_TOO_LARGE; }
+  if (a->r > MLORA_MAX_RANK) { set_error("mlora_add_lora: rank %d exceeds %d", a->r, MLORA_MAX_RANK); return MLORA_E_TOO_LARGE; }
+  if (a->num_slots > MLORA_MAX_SLOTS) { set_error("mlora_add_lora: %d slots exceed %d", a->num_slots, MLORA_MAX_SLOTS); return MLORA_E_TOO_LARGE; }
+  if (a->num_tokens == 0 || a->num_slices == 0 || a->num_slots == 0 || a->r == 0) return 0;
+  if (!a->x || !a->y || !a->token_to_slot) { set_error("mlora_add_lora: NULL tensor pointer"); return MLORA_E_INVALID; }
+  bool any = false;
+  for (int i = 0; i < a->num_slices; ++i) {
+    const MloraSlice& s = a->slices[i];
+    if (s.n < 0 || s.y_col < 0) { set_error("mlora_add_lora: slice %d has negative extent", i); return MLORA_E_INVALID; }
+    if (s.n > 0 && (!s.a || !s.b)) { set_error("mlora_add_lora: slice %d has NULL weights", i); return MLORA_E_INVALID; }
+    any |= s.n > 0;
+  }
+  if (!any) return 0;
+  if (reinterpret_cast<uintptr_t>(a->plan) & 15) { set_error("mlora_add_lora: plan must be 16-byte aligned"); return MLORA_E_INVALID; }
+
+  int form = a->form;
+  const bool vec = vector_ok(a);
+  if (form == MLORA_FORM_AUTO) {
+    const int forced = env_int("MLORA_FORCE_FORM", 0);
+    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_MFMA && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
+  }
+  if (form == MLORA_FORM_AUTO) {
+    if (!vec) form = MLORA_FORM_TOKEN;
+    else if (!sgmv_supported(a)) form = MLORA_FORM_BGMV;
+    else form = a->num_tokens <= env_int("MLORA_BGMV_MAX_TOKENS", 1024) ? MLORA_FORM_BGMV : MLORA_FORM_SGMV;
+  }
+  switch (form) {
+    case MLORA_FORM_TOKEN:
+      return launch_token_add(a);
+    case MLORA_FORM_BGMV:
+      if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
+      return launch_bgmv(a, /*include_long=*/true);
+    case MLORA_FORM_SGMV:
+    case MLORA_FORM_MFMA: {
+      if (!vec || !sgmv_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
+      if (form == MLORA_FORM_MFMA) return launch_sgmv(a, /*all_segments=*/true);
+      int rc = launch_bgmv(a, /*include_long=*/false);
+      if (rc) return rc;
+      return launch_sgmv(a, /*all_segments=*/false);
+    }
+  }
+  set_error("mlora_add_lora: unreachable form %d", form);
+  return MLORA_E_INVALID;
+}
+
+extern "C" uint64_t mlora_stream_capture_id(void* stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long id = 0;
+  if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &status, &id) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return status == hipStreamCaptureStatusActive ? static_cast<uint64_t>(id) : 0;
+}
+
+extern "C" int mlora_abi_version(void) { return MLORA_ABI_VERSION; }
+
+extern "C" const char* mlora_last_error(void) { return g_error; }
+
+extern "C" const char* mlora_build_info(void) {
+  return "mlora gfx950 (wave64; bgmv: dot2 + wave reductions; sgmv: bf16/f16 MFMA 16x16x32) built " __DATE__ " " __TIME__;
+}

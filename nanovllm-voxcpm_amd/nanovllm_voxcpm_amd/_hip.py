@@ -1,0 +1,429 @@
+"""ctypes binding of the gfx950 multi-LoRA library (C-ABI declared in include/mlora.h).
+
+The library is built in-tree next to this file.  Nothing here computes: every function
+marshals pointers and sizes of torch tensors into the C structs and enqueues HIP work on
+torch's current stream.  A missing library is an error, never a silent fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+from pathlib import Path
+
+import torch
+
+LIB_NAME = "libmlora_gfx950.so"
+LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
+
+MAX_SLICES = 8
+MAX_SLOTS = 1024
+MAX_RANK = 256
+
+DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA = 0, 1, 2, 3, 4
+FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA}
+
+PLAN_HEADER_WORDS = 16
+(
+    PLAN_MAGIC,
+    PLAN_NUM_TOKENS,
+    PLAN_MAX_SLOTS,
+    PLAN_NUM_LORA_TOKENS,
+    PLAN_NUM_ACTIVE,
+    PLAN_NO_LORA,
+    PLAN_BAD_SLOT,
+    PLAN_TILES_SHORT,
+    PLAN_TILES_LONG_SMALL,
+    PLAN_TILES_LONG_BIG,
+    PLAN_MAX_SEGMENT,
+) = range(11)
+PLAN_MAGIC_VALUE = 0x4D4C5031
+SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 8, 64
+
+_DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
+
+EXPORTS = (
+    "mlora_add_lora",
+    "mlora_shrink",
+    "mlora_expand",
+    "mlora_plan_workspace_bytes",
+    "mlora_meta_build",
+    "mlora_install_slot",
+    "mlora_stream_capture_id",
+    "mlora_abi_version",
+    "mlora_last_error",
+    "mlora_build_info",
+)
+
+
+class MloraSlice(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("n", C.c_int32), ("y_col", C.c_int32)]
+
+
+class MloraAddArgs(C.Structure):
+    _fields_ = [
+        ("stream", C.c_void_p),
+        ("x", C.c_void_p),
+        ("y", C.c_void_p),
+        ("x_stride", C.c_int64),
+        ("y_stride", C.c_int64),
+        ("token_to_slot", C.c_void_p),
+        ("plan", C.c_void_p),
+        ("num_tokens", C.c_int32),
+        ("k", C.c_int32),
+        ("r", C.c_int32),
+        ("num_slots", C.c_int32),
+        ("num_slices", C.c_int32),
+        ("dtype", C.c_int32),
+        ("form", C.c_int32),
+        ("scaling", C.c_float),
+        ("slices", MloraSlice * MAX_SLICES),
+    ]
+
+
+class MloraShrinkArgs(C.Structure):
+    _fields_ = [
+        ("stream", C.c_void_p),
+        ("x", C.c_void_p),
+        ("out", C.c_void_p),
+        ("x_stride", C.c_int64),
+        ("token_to_slot", C.c_void_p),
+        ("num_tokens", C.c_int32),
+        ("k", C.c_int32),
+        ("r", C.c_int32),
+        ("num_slots", C.c_int32),
+        ("num_slices", C.c_int32),
+        ("dtype", C.c_int32),
+        ("out_dtype", C.c_int32),
+        ("scaling", C.c_float),
+        ("a", C.c_void_p * MAX_SLICES),
+    ]
+
+
+class MloraExpandArgs(C.Structure):
+    _fields_ = [
+        ("stream", C.c_void_p),
+        ("h", C.c_void_p),
+        ("y", C.c_void_p),
+        ("y_stride", C.c_int64),
+        ("token_to_slot", C.c_void_p),
+        ("num_tokens", C.c_int32),
+        ("r", C.c_int32),
+        ("num_slots", C.c_int32),
+        ("num_slices", C.c_int32),
+        ("dtype", C.c_int32),
+        ("h_dtype", C.c_int32),
+        ("offset_start", C.c_int32),
+        ("add_inputs", C.c_int32),
+        ("b", C.c_void_p * MAX_SLICES),
+        ("n", C.c_int32 * MAX_SLICES),
+    ]
+
+
+class MloraMetaArgs(C.Structure):
+    _fields_ = [
+        ("stream", C.c_void_p),
+        ("token_to_slot", C.c_void_p),
+        ("num_tokens", C.c_int32),
+        ("max_slots", C.c_int32),
+        ("no_lora_bucket", C.c_int32),
+        ("plan", C.c_void_p),
+        ("sorted_idx", C.c_void_p),
+        ("compact_ids", C.c_void_p),
+        ("compact_counts", C.c_void_p),
+        ("compact_offsets", C.c_void_p),
+        ("compact_capacity", C.c_int32),
+        ("dense_counts", C.c_void_p),
+        ("dense_offsets", C.c_void_p),
+        ("padded_token_to_slot", C.c_void_p),
+        ("padded_len", C.c_int32),
+        ("scalars", C.c_void_p),
+    ]
+
+
+class MloraInstallArgs(C.Structure):
+    _fields_ = [
+        ("stream", C.c_void_p),
+        ("a_dst", C.c_void_p),
+        ("b_dst", C.c_void_p),
+        ("a_src", C.c_void_p),
+        ("b_src", C.c_void_p),
+        ("a_src_stride", C.c_int64),
+        ("b_src_stride", C.c_int64),
+        ("slot", C.c_int32),
+        ("k", C.c_int32),
+        ("n", C.c_int32),
+        ("r", C.c_int32),
+        ("rank", C.c_int32),
+        ("dtype", C.c_int32),
+        ("src_dtype", C.c_int32),
+        ("scaling", C.c_float),
+    ]
+
+
+_LIB: C.CDLL | None = None
+_LOAD_ERROR: str | None = None
+
+
+def library_path() -> Path:
+    override = os.environ.get("MLORA_LIBRARY")
+    return Path(override) if override else LIB_PATH
+
+
+def load() -> C.CDLL:
+    """Load the shared library once; raise RuntimeError with the reason if that fails."""
+    global _LIB, _LOAD_ERROR
+    if _LIB is not None:
+        return _LIB
+    if _LOAD_ERROR is not None:
+        raise RuntimeError(_LOAD_ERROR)
+    path = library_path()
+    if not path.exists():
+        _LOAD_ERROR = (
+            f"HIP multi-LoRA library not built: {path} is missing "
+            "(run `make -C nanovllm-voxcpm_amd/csrc` or __graft_entry__.build())"
+        )
+        raise RuntimeError(_LOAD_ERROR)
+    try:
+        lib = C.CDLL(str(path))
+    except OSError as exc:
+        _LOAD_ERROR = f"HIP multi-LoRA library failed to load: {exc}"
+        raise RuntimeError(_LOAD_ERROR) from exc
+    for name, args in (
+        ("mlora_add_lora", MloraAddArgs),
+        ("mlora_shrink", MloraShrinkArgs),
+        ("mlora_expand", MloraExpandArgs),
+        ("mlora_meta_build", MloraMetaArgs),
+        ("mlora_install_slot", MloraInstallArgs),
+    ):
+        fn = getattr(lib, name)
+        fn.argtypes = [C.POINTER(args)]
+        fn.restype = C.c_int
+    lib.mlora_plan_workspace_bytes.argtypes = [C.c_int32, C.c_int32]
+    lib.mlora_plan_workspace_bytes.restype = C.c_size_t
+    lib.mlora_stream_capture_id.argtypes = [C.c_void_p]
+    lib.mlora_stream_capture_id.restype = C.c_uint64
+    lib.mlora_abi_version.argtypes = []
+    lib.mlora_abi_version.restype = C.c_int
+    lib.mlora_last_error.argtypes = []
+    lib.mlora_last_error.restype = C.c_char_p
+    lib.mlora_build_info.argtypes = []
+    lib.mlora_build_info.restype = C.c_char_p
+    _LIB = lib
+    return lib
+
+
+def load_error() -> str | None:
+    """Reason the library cannot be used, or None when it loads."""
+    try:
+        load()
+    except RuntimeError as exc:
+        return str(exc)
+    return None
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mlora_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (code {rc}): {msg}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported LoRA element type {dtype}") from None
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU; the HIP LoRA path has no host fallback")
+
+
+def plan_workspace_words(num_tokens: int, max_slots: int) -> int:
+    return (load().mlora_plan_workspace_bytes(num_tokens, max_slots) + 3) // 4
+
+
+def add_lora(
+    y: torch.Tensor,
+    x: torch.Tensor,
+    a_slices: list[torch.Tensor],
+    b_slices: list[torch.Tensor],
+    y_cols: list[int],
+    token_to_slot: torch.Tensor,
+    plan: torch.Tensor | None,
+    scaling: float,
+    form: int = FORM_AUTO,
+) -> None:
+    """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice."""
+    lib = load()
+    _require_cuda(x, "x")
+    if len(a_slices) > MAX_SLICES:
+        raise ValueError(f"at most {MAX_SLICES} slices per call, got {len(a_slices)}")
+    args = MloraAddArgs()
+    args.stream = _stream(x.device)
+    args.x = x.data_ptr()
+    args.y = y.data_ptr()
+    args.x_stride = x.stride(0)
+    args.y_stride = y.stride(0)
+    args.token_to_slot = token_to_slot.data_ptr()
+    args.plan = plan.data_ptr() if plan is not None else None
+    args.num_tokens = x.size(0)
+    args.k = x.size(1)
+    args.r = a_slices[0].size(-2)
+    args.num_slots = a_slices[0].size(0)
+    args.num_slices = len(a_slices)
+    args.dtype = dtype_code(x.dtype)
+    args.form = form
+    args.scaling = scaling
+    for i, (a, b, col) in enumerate(zip(a_slices, b_slices, y_cols)):
+        s = args.slices[i]
+        s.a = a.data_ptr()
+        s.b = b.data_ptr()
+        s.n = b.size(1)
+        s.y_col = col
+    _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
+
+
+def shrink(
+    x: torch.Tensor, a_slices: list[torch.Tensor], out: torch.Tensor, token_to_slot: torch.Tensor, scaling: float
+) -> None:
+    lib = load()
+    _require_cuda(x, "x")
+    args = MloraShrinkArgs()
+    args.stream = _stream(x.device)
+    args.x = x.data_ptr()
+    args.out = out.data_ptr()
+    args.x_stride = x.stride(0)
+    args.token_to_slot = token_to_slot.data_ptr()
+    args.num_tokens = x.size(0)
+    args.k = x.size(1)
+    args.r = a_slices[0].size(-2)
+    args.num_slots = a_slices[0].size(0)
+    args.num_slices = len(a_slices)
+    args.dtype = dtype_code(x.dtype)
+    args.out_dtype = dtype_code(out.dtype)
+    args.scaling = scaling
+    for i, a in enumerate(a_slices):
+        args.a[i] = a.data_ptr()
+    _check(lib.mlora_shrink(C.byref(args)), "mlora_shrink")
+
+
+def expand(
+    h: torch.Tensor,
+    b_slices: list[torch.Tensor],
+    y: torch.Tensor,
+    token_to_slot: torch.Tensor,
+    offset_start: int,
+    add_inputs: bool,
+) -> None:
+    lib = load()
+    _require_cuda(h, "inputs")
+    args = MloraExpandArgs()
+    args.stream = _stream(h.device)
+    args.h = h.data_ptr()
+    args.y = y.data_ptr()
+    args.y_stride = y.stride(0)
+    args.token_to_slot = token_to_slot.data_ptr()
+    args.num_tokens = h.size(1)
+    args.r = b_slices[0].size(-1)
+    args.num_slots = b_slices[0].size(0)
+    args.num_slices = len(b_slices)
+    args.dtype = dtype_code(y.dtype)
+    args.h_dtype = dtype_code(h.dtype)
+    args.offset_start = offset_start
+    args.add_inputs = 1 if add_inputs else 0
+    for i, b in enumerate(b_slices):
+        args.b[i] = b.data_ptr()
+        args.n[i] = b.size(1)
+    _check(lib.mlora_expand(C.byref(args)), "mlora_expand")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return t.data_ptr() if t is not None else None
+
+
+def meta_build(
+    token_to_slot: torch.Tensor,
+    max_slots: int,
+    *,
+    no_lora_bucket: bool = False,
+    plan: torch.Tensor | None = None,
+    sorted_idx: torch.Tensor | None = None,
+    compact_ids: torch.Tensor | None = None,
+    compact_counts: torch.Tensor | None = None,
+    compact_offsets: torch.Tensor | None = None,
+    compact_capacity: int = 0,
+    dense_counts: torch.Tensor | None = None,
+    dense_offsets: torch.Tensor | None = None,
+    padded_token_to_slot: torch.Tensor | None = None,
+    scalars: torch.Tensor | None = None,
+) -> None:
+    """One launch of the on-device counting sort; every output tensor is optional."""
+    lib = load()
+    _require_cuda(token_to_slot, "token_to_slot")
+    if token_to_slot.dtype != torch.int32 or not token_to_slot.is_contiguous():
+        raise ValueError("token_to_slot must be a contiguous int32 tensor")
+    args = MloraMetaArgs()
+    args.stream = _stream(token_to_slot.device)
+    args.token_to_slot = token_to_slot.data_ptr()
+    args.num_tokens = token_to_slot.numel()
+    args.max_slots = max_slots
+    args.no_lora_bucket = 1 if no_lora_bucket else 0
+    args.plan = _ptr(plan)
+    args.sorted_idx = _ptr(sorted_idx)
+    args.compact_ids = _ptr(compact_ids)
+    args.compact_counts = _ptr(compact_counts)
+    args.compact_offsets = _ptr(compact_offsets)
+    args.compact_capacity = compact_capacity
+    args.dense_counts = _ptr(dense_counts)
+    args.dense_offsets = _ptr(dense_offsets)
+    args.padded_token_to_slot = _ptr(padded_token_to_slot)
+    args.padded_len = padded_token_to_slot.numel() if padded_token_to_slot is not None else 0
+    args.scalars = _ptr(scalars)
+    _check(lib.mlora_meta_build(C.byref(args)), "mlora_meta_build")
+
+
+def install_slot(
+    a_dst: torch.Tensor,
+    b_dst: torch.Tensor,
+    slot: int,
+    a_src: torch.Tensor,
+    b_src: torch.Tensor,
+    rank: int,
+    scaling: float,
+) -> None:
+    """Rewrite one slot of A [slots, r, K] and B [slots, n, r] from an adapter payload."""
+    lib = load()
+    _require_cuda(a_dst, "lora_A")
+    args = MloraInstallArgs()
+    args.stream = _stream(a_dst.device)
+    args.a_dst = a_dst.data_ptr()
+    args.b_dst = b_dst.data_ptr()
+    args.a_src = a_src.data_ptr()
+    args.b_src = b_src.data_ptr()
+    args.a_src_stride = a_src.stride(0)
+    args.b_src_stride = b_src.stride(0)
+    args.slot = slot
+    args.k = a_dst.size(2)
+    args.n = b_dst.size(1)
+    args.r = a_dst.size(1)
+    args.rank = rank
+    args.dtype = dtype_code(a_dst.dtype)
+    args.src_dtype = dtype_code(a_src.dtype)
+    args.scaling = scaling
+    _check(lib.mlora_install_slot(C.byref(args)), "mlora_install_slot")
+
+
+def stream_capture_id(device: torch.device) -> int:
+    """Identifier of the graph capture in progress on torch's current stream, 0 when none."""
+    return int(load().mlora_stream_capture_id(_stream(device)))
+
+
+def build_info() -> str:
+    return load().mlora_build_info().decode()

