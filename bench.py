@@ -1,0 +1,269 @@
+"""Benchmark of the fused multi-LoRA apply on one MI355X.
+
+Workload (BASELINE.json configs[1], "decode BGMV bf16"): one decode step of a 24-layer
+decoder — 256 tokens (one per sequence), 32 resident adapters of rank 16, adapter ids uniform,
+LoRA applied to the stacked q|k|v [1024|256|256], o [1024->1024], gate|up [1024->2x4096] and
+down [4096->1024] projections of every layer.  A "step" is the LoRA work of that decode step:
+one on-device metadata build plus 24 x 4 fused shrink+expand launches, issued through the
+same backend entry (`LoRABackend.add_lora`) the LoRA linears call.  Every layer owns its
+weights and its activation buffers (about 0.75 GB in total), so a step streams from HBM and
+not from the 256 MB last-level cache.
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / time of a step, inputs
+resident in HBM, the step replayed as a captured graph (decode runs under graph replay in
+the serving engine).  `roofline` is quoted for the kernel every launch of the step uses
+(bgmv_kernel<bf16, rank 16>): algorithmic bytes of an average launch / average launch time.
+`cpu_baseline` times the reference's torch formulation (per-token F.linear loop) of one layer
+of the same workload on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "nanovllm-voxcpm_amd"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+NUM_LAYERS, NUM_TOKENS, NUM_SLOTS, RANK = 24, 256, 32, 16
+ORDER = ("qkv", "o", "gate_up", "down")
+
+
+def algorithmic_bytes(k: int, widths: list[int], t_lora: int, used_slots: int, rank: int, num_tokens: int) -> int:
+    """bf16 bytes one fused call has to move: x rows, the A and B slices of the slots in use,
+    y read and written once, plus the int32 slot ids; the rank-r intermediate counts as zero."""
+    s, n = len(widths), sum(widths)
+    return 2 * (t_lora * k + used_slots * s * rank * k + used_slots * rank * n + 2 * t_lora * n) + 4 * num_tokens
+
+
+def build_workload(device: str):
+    import torch
+
+    from nanovllm_voxcpm_amd import synthetic
+
+    layers = []
+    for layer in range(NUM_LAYERS):
+        entry = {}
+        for j, name in enumerate(ORDER):
+            proj = synthetic.make_projection(name, NUM_SLOTS, RANK, torch.bfloat16, seed=1000 + 16 * layer + j, device=device)
+            x, y = synthetic.make_activations(NUM_TOKENS, proj.k, sum(proj.widths), torch.bfloat16, seed=5000 + 16 * layer + j, device=device)
+            entry[name] = (proj, x, y)
+        layers.append(entry)
+    slots = synthetic.decode_slots(NUM_TOKENS, NUM_SLOTS, seed=7).to(device)
+    return layers, slots
+
+
+def make_step(layers, slots, form: str, only: str | None = None):
+    """Returns step(): metadata build + every fused apply of one decode step, via the backend."""
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend, LoRAMetadata
+
+    backend = HipLoRABackend(form)
+    status = backend.availability()
+    if not status.available:
+        raise RuntimeError(f"HIP LoRA backend unavailable: {status.reason}")
+    names = [only] if only else list(ORDER)
+    calls = []
+    for entry in layers:
+        for name in names:
+            proj, x, y = entry[name]
+            blocks = list(y.split(proj.widths, dim=-1))
+            calls.append((blocks, x, proj.a, proj.b, y if len(blocks) > 1 else None))
+
+    def step():
+        # a new metadata object per step, as the engine installs a new context per step:
+        # the first call builds the segment plan on the device, the others reuse it
+        meta = LoRAMetadata(slots, None, None, None, None, False, 0)
+        for blocks, x, a, b, packed in calls:
+            backend.add_lora(blocks, x, a, b, indices=slots, metadata=meta, scaling=1.0, y_packed=packed)
+
+    return step, len(calls)
+
+
+def time_region(fn, iters: int) -> float:
+    """Milliseconds per call of fn, HIP events on torch's current stream (the stream every
+    kernel of fn is launched on), synchronised on both sides."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def capture(step):
+    import torch
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    return graph
+
+
+def cpu_baseline(layers, slots, budget_s: float = 20.0) -> dict:
+    """The reference's torch LoRA computation on the host: per-token F.linear(F.linear(x_t, A[s]),
+    B[s]) accumulate (oracle.per_token_add_lora), fp32, one layer of the same workload, all host
+    threads.  Reported in the metric's unit: algorithmic bytes of what was run / time."""
+    import torch
+
+    from oracle import lora_apply as oracle
+
+    threads = torch.get_num_threads()
+    entry = layers[0]
+    slots_cpu = slots.cpu()
+    work = []
+    for name in ORDER:
+        proj, x, y = entry[name]
+        work.append((proj, x.cpu().float(), y.cpu().float(), [a.cpu().float() for a in proj.a], [b.cpu().float() for b in proj.b]))
+    used = int(torch.unique(slots_cpu[slots_cpu >= 0]).numel())
+    t_lora = int((slots_cpu >= 0).sum())
+    layer_bytes = sum(algorithmic_bytes(p.k, p.widths, t_lora, used, RANK, NUM_TOKENS) for p, *_ in work)
+
+    def one_layer():
+        for proj, x, y, a, b in work:
+            views = list(y.split(proj.widths, dim=-1))
+            oracle.per_token_add_lora(views, x, a, b, indices=slots_cpu, scaling=1.0, y_packed=y)
+
+    one_layer()  # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        one_layer()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    model = ""
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {
+        "value": round(layer_bytes / med / 1e9, 4),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"1 of {NUM_LAYERS} layers of the same decode step (4 projections, 256 tokens, 32 adapters, rank 16), fp32, "
+                  f"per-token torch loop, median of {len(times)} runs",
+        "us_per_layer": round(med * 1e6, 1),
+        "us_per_step_extrapolated": round(med * 1e6 * NUM_LAYERS, 1),
+        "cpu_model": model,
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | sgmv | token")
+    ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
+    ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; every box in this pool has one (use --gpus 1)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+    layers, slots = build_workload(device)
+    step, launches = make_step(layers, slots, args.form, args.only)
+
+    used = int(torch.unique(slots[slots >= 0]).numel())
+    t_lora = int((slots >= 0).sum())
+    names = [args.only] if args.only else list(ORDER)
+    per_proj = {n: algorithmic_bytes(layers[0][n][0].k, layers[0][n][0].widths, t_lora, used, RANK, NUM_TOKENS) for n in names}
+    step_bytes = NUM_LAYERS * sum(per_proj.values())
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    eager_ms = time_region(step, max(5, min(args.steps, 50)))
+    if args.eager:
+        runner = step
+    else:
+        graph = capture(step)
+        runner = graph.replay
+    for _ in range(args.warmup):
+        runner()
+    ms = time_region(runner, args.steps)
+
+    # per-projection time: the same step restricted to one projection (24 launches)
+    per_proj_us = {}
+    if not args.only and not args.eager:
+        for n in ORDER:
+            sub, cnt = make_step(layers, slots, args.form, n)
+            g = capture(sub)
+            for _ in range(5):
+                g.replay()
+            per_proj_us[n] = round(time_region(g.replay, max(20, args.steps // 4)) * 1e3 / cnt, 3)
+
+    value = step_bytes / (ms * 1e-3) / 1e9
+    launch_bytes = step_bytes / launches
+    launch_us = ms * 1e3 / launches
+    achieved = launch_bytes / (launch_us * 1e-6) / 1e9
+    out = {
+        "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "decode BGMV bf16 (BASELINE configs[1]): 256 tokens, 32 adapters, rank 16, "
+                        "qkv/o/gate_up/down x 24 layers, per-layer weights and activations",
+            "tokens": NUM_TOKENS, "adapters": NUM_SLOTS, "rank": RANK, "layers": NUM_LAYERS,
+            "projections": names, "form": args.form, "launch": "eager" if args.eager else "graph replay",
+        },
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "us_per_decode_step": round(ms * 1e3, 2),
+        "us_per_decode_step_eager": round(eager_ms * 1e3, 2),
+        "algorithmic_bytes_per_step": step_bytes,
+        "launches_per_step": launches + 1,
+        "us_per_launch_by_projection": per_proj_us,
+        "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
+        "roofline": {
+            "kernel": "bgmv_kernel<bf16, rank 16>" if args.form in ("auto", "bgmv") else args.form,
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "bytes_per_launch": round(launch_bytes),
+            "us_per_launch": round(launch_us, 3),
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(layers, slots)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -3,7 +3,9 @@
 //   shrink  — H[tokens x r] = X_tile . A[slot]^T.  The four wavefronts split K; every lane
 //             feeds the MFMA straight from 128-bit global loads of x rows and A rows, so
 //             neither operand is read twice by a workgroup.  The four partial tiles are
-//             summed through LDS and the rank-r intermediate is kept there at operand precision.
+//             summed through LDS and the rank-r intermediate is kept there as a hi + lo pair of
+//             operand-precision values (about 16 significant bits), so the expand loses nothing
+//             that would show after the final rounding of y.
 //   expand  — OUT^T[cols x tokens] = B[slot] . H^T.  The B rows fed to the four MFMAs of a
 //             64-column span are interleaved (row rho of MFMA j is column 16*(rho/4) + 4j + rho%4)
 //             so that a lane ends up with 16 consecutive output columns of one token: y is
@@ -57,7 +59,8 @@ __global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
   constexpr int HSTRIDE = R + 8;                // padded LDS row of the intermediate
 
   __shared__ __attribute__((aligned(16))) float s_red[kWaves * RB * 64 * 4];
-  __shared__ __attribute__((aligned(16))) T s_hb[MTB * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) T s_hb[MTB * HSTRIDE];  // leading part of H
+  __shared__ __attribute__((aligned(16))) T s_hl[MTB * HSTRIDE];  // remainder H - hi
 
   const int b = blockIdx.x;
   const int q = b >> 3;
@@ -137,21 +140,31 @@ __global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
         const int tok = tb * 16 + 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-        if (r < R) s_hb[tok * HSTRIDE + r] = from_f32<T>(sum * p.scaling);
+        if (r < R) {
+          const float v = sum * p.scaling;
+          const T hi = from_f32<T>(v);
+          s_hb[tok * HSTRIDE + r] = hi;
+          s_hl[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+        }
       }
       __syncthreads();
     }
   }
 
   // ---- expand ---------------------------------------------------------------------------
-  Pack8 hop[TB][KSTEPS];
+  Pack8 hop[TB][KSTEPS], hlo[TB][KSTEPS];
 #pragma unroll
   for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const int kc = lg + 4 * ks;
-      if (kc * 8 < R) hop[tb][ks].raw = load128(&s_hb[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-      else hop[tb][ks].raw = i32x4{0, 0, 0, 0};
+      if (kc * 8 < R) {
+        hop[tb][ks].raw = load128(&s_hb[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+        hlo[tb][ks].raw = load128(&s_hl[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+      } else {
+        hop[tb][ks].raw = i32x4{0, 0, 0, 0};
+        hlo[tb][ks].raw = i32x4{0, 0, 0, 0};
+      }
     }
 
   const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
@@ -177,7 +190,10 @@ __global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
       for (int j = 0; j < 4; ++j) {
         acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) acc[j] = Mma<T>::run(bop[j][ks], hop[tb][ks], acc[j]);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          acc[j] = Mma<T>::run(bop[j][ks], hlo[tb][ks], acc[j]);
+          acc[j] = Mma<T>::run(bop[j][ks], hop[tb][ks], acc[j]);
+        }
       }
       if (tb * 16 + lr < m) {
         T* yp = y + static_cast<int64_t>(row[tb]) * p.ys + c0 + 16 * lg;

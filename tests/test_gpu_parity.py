@@ -43,18 +43,26 @@ def _apply(form, proj, x, y, slots, scaling=1.0):
 
 
 def _exact(proj, x, y0, slots, scaling=1.0):
-    """fp64 evaluation of y0 + delta and of delta, per slice concatenated."""
-    xs, ys = x.cpu(), y0.cpu()
-    outs, deltas, col = [], [], 0
+    """fp64 evaluation, per slice concatenated, of y0 + delta and of sum_j |h_j| |B_nj| (the scale
+    of the error a rounding of the rank-r intermediate to operand precision can cause)."""
+    xs, ys, idx = x.cpu().double(), y0.cpu(), slots.cpu().to(torch.int64)
+    outs, mags, col = [], [], 0
     for a, b, n in zip(proj.a, proj.b, proj.widths):
-        d = oracle.grouped_delta(xs, a.cpu(), b.cpu(), slots.cpu(), scaling, torch.float64)
+        a64, b64 = a.cpu().double(), b.cpu().double()
+        d = torch.zeros(xs.size(0), n, dtype=torch.float64)
+        mag = torch.zeros_like(d)
+        for slot in torch.unique(idx[idx >= 0]).tolist():
+            rows = torch.nonzero(idx == slot).flatten()
+            h = xs[rows] @ a64[slot].T * scaling
+            d[rows] = h @ b64[slot].T
+            mag[rows] = h.abs() @ b64[slot].abs().T
         outs.append(ys[:, col : col + n].double() + d)
-        deltas.append(d)
+        mags.append(mag)
         col += n
-    return torch.cat(outs, dim=-1), torch.cat(deltas, dim=-1)
+    return torch.cat(outs, dim=-1), torch.cat(mags, dim=-1)
 
 
-def _check(got, y0, exact, delta, slots, tag):
+def _check(got, y0, exact, mag, slots, tag):
     got_c, y0_c = got.cpu(), y0.cpu()
     live = (slots.cpu() >= 0)
     # rows without a slot keep their bits
@@ -62,11 +70,10 @@ def _check(got, y0, exact, delta, slots, tag):
     want = exact.to(got.dtype)
     ok = torch.isclose(got_c.double(), want.double(), rtol=RTOL, atol=ATOL)
     assert ok.all(), f"{tag}: {(~ok).sum().item()} elements outside rtol={RTOL}/atol={ATOL}; max abs err {(got_c.double() - want.double()).abs().max().item():.4g}"
-    # tighter: one rounding of the exact sum (half an ulp) plus the operand-precision intermediate
+    # tighter: one rounding of the exact sum (half an ulp of the output) plus, at most, a rounding of
+    # the rank-r intermediate to operand precision (MFMA forms) and fp32 accumulation noise
     eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -22}[got.dtype]
-    bound = eps * exact.abs() + 4 * eps * delta.abs() + 1e-30
-    if got.dtype != torch.float32:
-        bound = bound + 2.0 ** -24
+    bound = eps * exact.abs() + eps * mag + 2.0 ** -24
     err = (got_c.double() - exact).abs()
     bad = err > bound
     assert not bad.any(), f"{tag}: {bad.sum().item()} elements beyond one rounding; worst ratio {(err / bound).max().item():.3f}"
@@ -113,23 +120,32 @@ def test_config2_decode_bf16(name, form):
     x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=101, device="cuda")
     slots = synthetic.decode_slots(256, 32, seed=102).cuda()
     got = _apply(form, proj, x, y0.clone(), slots)
-    exact, delta = _exact(proj, x, y0, slots)
-    _check(got, y0, exact, delta, slots, f"config2/{name}/{form}")
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
-def test_config2_matches_reference_bf16_torch_loop():
-    """The same batch against the reference's formulation run in bf16 on the host (per-token
-    F.linear loop), at the stated tolerance."""
+def test_config2_matches_reference_torch_loop():
+    """The same batch against the reference's torch formulation (per-token F.linear loop) on the
+    host.  With fp32 accumulation (the loop run on fp32 copies of the bf16 values) every element
+    meets the stated tolerance.  Run in bf16 end to end, that loop rounds the intermediate, the
+    update and the sum separately, which alone can leave it two output ulps (1.6 %) from the
+    exact value, so against it only the bulk of the elements is held to the tolerance."""
     from nanovllm_voxcpm_amd import synthetic
 
     proj = _make("qkv", 32, 16, torch.bfloat16, seed=100)
     x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=101, device="cuda")
     slots = synthetic.decode_slots(256, 32, seed=102)
-    got = _apply("auto", proj, x, y0.clone(), slots.cuda())
-    y_cpu = y0.cpu().clone()
-    views = list(y_cpu.split(proj.widths, dim=-1))
-    oracle.per_token_add_lora(views, x.cpu(), [a.cpu() for a in proj.a], [b.cpu() for b in proj.b], indices=slots, scaling=1.0, y_packed=y_cpu)
-    assert torch.allclose(got.cpu().float(), y_cpu.float(), rtol=RTOL, atol=ATOL)
+    got = _apply("auto", proj, x, y0.clone(), slots.cuda()).cpu().float()
+    a_cpu, b_cpu = [a.cpu() for a in proj.a], [b.cpu() for b in proj.b]
+    y32 = y0.cpu().float()
+    oracle.per_token_add_lora(list(y32.split(proj.widths, dim=-1)), x.cpu().float(), [a.float() for a in a_cpu],
+                              [b.float() for b in b_cpu], indices=slots, scaling=1.0, y_packed=y32)
+    assert torch.allclose(got, y32, rtol=RTOL, atol=ATOL)
+    y16 = y0.cpu().clone()
+    oracle.per_token_add_lora(list(y16.split(proj.widths, dim=-1)), x.cpu(), a_cpu, b_cpu, indices=slots, scaling=1.0, y_packed=y16)
+    close = torch.isclose(got, y16.float(), rtol=RTOL, atol=ATOL)
+    assert close.float().mean().item() > 0.999
+    assert torch.allclose(got, y16.float(), rtol=2.0 ** -5, atol=ATOL)
 
 
 @pytest.mark.parametrize("form", ["bgmv", "mfma", "token"])
@@ -145,8 +161,8 @@ def test_ranks_and_dtypes_small(rank, dtype, form):
     g = torch.Generator().manual_seed(rank)
     slots = torch.randint(-1, 6, (75,), generator=g, dtype=torch.int32).cuda()
     got = _apply(form, proj, x, y0.clone(), slots, scaling=0.5)
-    exact, delta = _exact(proj, x, y0, slots, scaling=0.5)
-    _check(got, y0, exact, delta, slots, f"rank{rank}/{dtype}/{form}")
+    exact, mag = _exact(proj, x, y0, slots, scaling=0.5)
+    _check(got, y0, exact, mag, slots, f"rank{rank}/{dtype}/{form}")
 
 
 @pytest.mark.parametrize("form", ["auto", "token"])
@@ -179,16 +195,18 @@ def test_config3_prefill_bf16(name, form):
 
     print(f"config3 {name} form={form}", flush=True)
     proj = _make(name, 8, 64, torch.bfloat16, seed=300)
-    slots_cpu, lengths = synthetic.prefill_slots(16, 8, seed=301)
     if name in ("gate_up", "down") or form == "bgmv":
-        slots_cpu = slots_cpu[:1500]  # bound the host-side fp64 check
+        # same mix of sequences, shorter ones: bounds the host-side fp64 check
+        slots_cpu, lengths = synthetic.prefill_slots(16, 8, seed=301, min_len=16, max_len=160)
+    else:
+        slots_cpu, lengths = synthetic.prefill_slots(16, 8, seed=301)
     T = slots_cpu.numel()
     assert (slots_cpu < 0).any() and (slots_cpu >= 0).any()
     x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=302, device="cuda")
     slots = slots_cpu.cuda()
     got = _apply(form, proj, x, y0.clone(), slots)
-    exact, delta = _exact(proj, x, y0, slots)
-    _check(got, y0, exact, delta, slots, f"config3/{name}/{form}")
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"config3/{name}/{form}")
 
 
 # ---- config 4: mixed batch, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity ----
@@ -206,8 +224,8 @@ def test_config4_mixed_batch_rank_masking(name):
     x, y0 = synthetic.make_activations(8192, proj.k, sum(proj.widths), torch.bfloat16, seed=403, device="cuda")
     slots = slots_cpu.cuda()
     got = _apply("auto", proj, x, y0.clone(), slots)
-    exact, delta = _exact(proj, x, y0, slots)
-    _check(got, y0, exact, delta, slots, f"config4/{name}")
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"config4/{name}")
     # rank padding is inert: the same adapters stored at their true rank in rank-r buffers of a
     # narrower layer give the same result for the slots whose rank fits
     narrow = [s for s, r in enumerate(ranks) if r <= 16]
@@ -277,8 +295,8 @@ def test_empty_and_degenerate_batches():
         x, y0 = synthetic.make_activations(T, 1024, 1024, torch.bfloat16, seed=602, device="cuda")
         slots = torch.full((T,), 3, dtype=torch.int32, device="cuda")
         got = _apply("auto", proj, x, y0.clone(), slots)
-        exact, delta = _exact(proj, x, y0, slots)
-        _check(got, y0, exact, delta, slots, f"single-slot T={T}")
+        exact, mag = _exact(proj, x, y0, slots)
+        _check(got, y0, exact, mag, slots, f"single-slot T={T}")
     # a slot id beyond the resident slots is treated as "no adapter"
     slots = torch.tensor([0, 9, 1], dtype=torch.int32, device="cuda")
     x, y0 = synthetic.make_activations(3, 1024, 1024, torch.bfloat16, seed=603, device="cuda")
@@ -298,8 +316,8 @@ def test_strided_views_and_3d_inputs():
     y0 = yw.clone()
     slots = synthetic.decode_slots(40, 4, seed=702).cuda()
     _backend().add_lora([y], x, proj.a, proj.b, indices=slots, metadata=_metadata(slots), scaling=1.0)
-    exact, delta = _exact(proj, x.contiguous(), y0[:, 1024:2048].contiguous(), slots)
-    _check(yw[:, 1024:2048].contiguous(), y0[:, 1024:2048].contiguous(), exact, delta, slots, "strided")
+    exact, mag = _exact(proj, x.contiguous(), y0[:, 1024:2048].contiguous(), slots)
+    _check(yw[:, 1024:2048].contiguous(), y0[:, 1024:2048].contiguous(), exact, mag, slots, "strided")
     assert torch.equal(yw[:, :1024], y0[:, :1024]) and torch.equal(yw[:, 2048:], y0[:, 2048:])
 
     layer = LoRALinear(64, 48, bias=True, max_loras=2, max_lora_rank=8).cuda().to(torch.bfloat16)
