@@ -176,6 +176,9 @@ def main() -> None:
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--hot-layers", type=int, default=0,
+                    help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
+                         "(N=1 keeps the working set inside the last-level cache); 0 = every layer has its own")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; every box in this pool has one (use --gpus 1)")
@@ -187,6 +190,8 @@ def main() -> None:
     device = "cuda:0"
     torch.cuda.set_device(0)
     layers, slots = build_workload(device)
+    if args.hot_layers > 0:
+        layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
     step, launches = make_step(layers, slots, args.form, args.only)
 
     used = int(torch.unique(slots[slots >= 0]).numel())
@@ -240,6 +245,7 @@ def main() -> None:
                         "qkv/o/gate_up/down x 24 layers, per-layer weights and activations",
             "tokens": NUM_TOKENS, "adapters": NUM_SLOTS, "rank": RANK, "layers": NUM_LAYERS,
             "projections": names, "form": args.form, "launch": "eager" if args.eager else "graph replay",
+            "distinct_layer_buffers": args.hot_layers or NUM_LAYERS,
         },
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "us_per_decode_step": round(ms * 1e3, 2),

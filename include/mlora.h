@@ -35,9 +35,9 @@ extern "C" {
 /* which kernel family mlora_add_lora uses */
 #define MLORA_FORM_AUTO 0  /* library chooses from shapes and the plan */
 #define MLORA_FORM_TOKEN 1 /* one workgroup per token, any shape or dtype; needs no plan */
-#define MLORA_FORM_BGMV 2  /* segment tiles of <= 8 tokens, wave64 dot-product reductions */
-#define MLORA_FORM_SGMV 3  /* MFMA tiles for segments >= threshold, BGMV tiles for the rest */
-#define MLORA_FORM_MFMA 4  /* MFMA tiles for every segment */
+#define MLORA_FORM_BGMV 2  /* small tiles (<= 16 tokens of one slot), packed dot2 + wave64 reductions */
+#define MLORA_FORM_SGMV 3  /* 64-token MFMA tiles for segments >= threshold, small MFMA tiles for the rest */
+#define MLORA_FORM_MFMA 4  /* small tiles for every segment, both products on the matrix cores */
 
 /* error codes (negative) */
 #define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
@@ -148,10 +148,17 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
 #define MLORA_PLAN_HEADER_WORDS 16
 #define MLORA_PLAN_MAGIC_VALUE 0x4d4c5031 /* "MLP1" */
 
-/* Segment length from which a segment gets MFMA tiles, and the two tile heights. */
+/* Segment length from which a segment gets big (prefill) tiles, and the two tile heights. */
 #define MLORA_SEGMENT_THRESHOLD 16
-#define MLORA_TILE_SMALL 8
+#define MLORA_TILE_SMALL 16
 #define MLORA_TILE_BIG 64
+/* A small tile is a self-contained 128-byte record, so that a workgroup learns everything it
+ * needs from one load: words {slot, token count, first position in sorted_idx, 0}, then the 16
+ * token indices of the tile (entries past the count are 0, a valid row), then padding.
+ * A big tile is four words {slot, first position in sorted_idx, token count, 0}. */
+#define MLORA_SMALL_TILE_WORDS 32
+#define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
+#define MLORA_BIG_TILE_WORDS 4
 
 /* Arguments of the on-device metadata build: a stable counting sort of the tokens by
  * slot id.  The plan workspace (always written when non-NULL) feeds mlora_add_lora; the

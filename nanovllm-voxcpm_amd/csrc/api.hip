@@ -90,9 +90,11 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_MFMA && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
   }
   if (form == MLORA_FORM_AUTO) {
+    // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
+    // tiles for the long segments and 16-token tiles for the rest.
     if (!vec) form = MLORA_FORM_TOKEN;
     else if (!sgmv_supported(a)) form = MLORA_FORM_BGMV;
-    else form = a->num_tokens <= env_int("MLORA_BGMV_MAX_TOKENS", 1024) ? MLORA_FORM_BGMV : MLORA_FORM_SGMV;
+    else form = a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) ? MLORA_FORM_MFMA : MLORA_FORM_SGMV;
   }
   switch (form) {
     case MLORA_FORM_TOKEN:
@@ -103,10 +105,10 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     case MLORA_FORM_SGMV:
     case MLORA_FORM_MFMA: {
       if (!vec || !sgmv_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
-      if (form == MLORA_FORM_MFMA) return launch_sgmv(a, /*all_segments=*/true);
-      int rc = launch_bgmv(a, /*include_long=*/false);
+      if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
+      int rc = launch_decode(a, /*include_long=*/false);
       if (rc) return rc;
-      return launch_sgmv(a, /*all_segments=*/false);
+      return launch_sgmv(a);
     }
   }
   set_error("mlora_add_lora: unreachable form %d", form);
@@ -128,5 +130,5 @@ extern "C" int mlora_abi_version(void) { return MLORA_ABI_VERSION; }
 extern "C" const char* mlora_last_error(void) { return g_error; }
 
 extern "C" const char* mlora_build_info(void) {
-  return "mlora gfx950 (wave64; bgmv: dot2 + wave reductions; sgmv: bf16/f16 MFMA 16x16x32) built " __DATE__ " " __TIME__;
+  return "mlora gfx950 (wave64; small tiles: MFMA 16x16x32 or dot2 + wave reductions; big tiles: MFMA 16x16x32) built " __DATE__ " " __TIME__;
 }

@@ -1,5 +1,5 @@
-// BGMV form: one workgroup per (small tile, slice, column range).  A small tile is up to
-// eight tokens that share a slot, so A[slot] and B[slot] are streamed once for all of them.
+// BGMV form (vector ALU): one workgroup per (small tile, slice, column range).  A small tile is
+// up to sixteen tokens that share a slot; the workgroup takes them eight at a time.
 //   shrink  — every lane takes one 128-bit chunk of K, forms the partial dot products of its
 //             tile rows with eight A rows (packed dot2, fp32 accumulate) and the 64 partials per
 //             lane are folded across the wavefront with a halving butterfly (63 exchanges);
@@ -15,7 +15,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
-constexpr int kMT = MLORA_TILE_SMALL;
+constexpr int kMT = 8;  // tokens handled per pass over a small tile
 constexpr int kColTile = 512;  // output columns staged in LDS at a time
 constexpr int kMaxSplits = 64;
 
@@ -30,7 +30,7 @@ struct BgmvParams {
   void* y;
   int64_t xs, ys;
   const int32_t* plan;
-  int sorted_off, small_off;
+  int small_off;
   int T, K, num_slots, nsplit, include_long;
   float scaling;
   BgmvSplit split[kMaxSplits];
@@ -73,21 +73,23 @@ __global__ __launch_bounds__(kThreads) void bgmv_kernel(BgmvParams p) {
 
   // Workgroups b, b+8, b+16, ... share an XCD (and its L2): give them the column ranges of
   // one tile so that x rows and A[slot] are fetched into that L2 once.
-  const int b = blockIdx.x;
-  const int q = b >> 3;
-  const int split_id = q % p.nsplit;
-  const int tile = (q / p.nsplit) * 8 + (b & 7);
+  // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first, and
+  // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD
+  const int split_id = blockIdx.y;
+  const int tile = blockIdx.z * 8 + blockIdx.x;
   const int32_t* hdr = p.plan;
+  const int32_t* rec = p.plan + p.small_off + tile * MLORA_SMALL_TILE_WORDS;  // tile < capacity: in bounds
+  const int slot = rec[0], m_tile = rec[1];
   if (hdr[MLORA_PLAN_MAGIC] != MLORA_PLAN_MAGIC_VALUE || hdr[MLORA_PLAN_NUM_TOKENS] != p.T ||
       hdr[MLORA_PLAN_MAX_SLOTS] != p.num_slots)
     return;
   const int n_tiles = hdr[MLORA_PLAN_TILES_SHORT] + (p.include_long ? hdr[MLORA_PLAN_TILES_LONG_SMALL] : 0);
   if (tile >= n_tiles) return;
-  const i32x4 td = reinterpret_cast<const i32x4*>(p.plan + p.small_off)[tile];
-  const int slot = td[0], start = td[1], m = td[2];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int32_t* sorted = p.plan + p.sorted_off + start;
+  for (int part = 0; part * kMT < m_tile; ++part) {
+  const int m = m_tile - part * kMT < kMT ? m_tile - part * kMT : kMT;
+  const int32_t* sorted = rec + MLORA_SMALL_TILE_ROWS + part * kMT;
   int rows[kMT];
 #pragma unroll
   for (int t = 0; t < kMT; ++t) rows[t] = sorted[t < m ? t : 0];
@@ -184,6 +186,7 @@ __global__ __launch_bounds__(kThreads) void bgmv_kernel(BgmvParams p) {
     }
     __syncthreads();
   }
+  }  // next eight tokens of the tile
 }
 
 template <typename T>
@@ -203,7 +206,7 @@ int launch_bgmv(const MloraAddArgs* a, bool include_long) {
   p.x = a->x; p.y = a->y; p.xs = a->x_stride; p.ys = a->y_stride;
   p.plan = a->plan;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  p.sorted_off = lay.sorted_off; p.small_off = lay.small_off;
+  p.small_off = lay.small_off;
   p.T = a->num_tokens; p.K = a->k; p.num_slots = a->num_slots; p.include_long = include_long ? 1 : 0;
   p.scaling = a->scaling;
 
@@ -233,12 +236,11 @@ int launch_bgmv(const MloraAddArgs* a, bool include_long) {
   int cap = lay.cap_small;
   if (!include_long) {
     const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
-    const int per_seg = (MLORA_SEGMENT_THRESHOLD - 1 + kMT - 1) / kMT;
-    if (segs * per_seg < cap) cap = segs * per_seg;
+    if (segs < cap) cap = segs;  // a segment below the threshold is exactly one small tile
   }
   if (cap == 0) return 0;
   cap = (cap + 7) & ~7;
-  dim3 grid(static_cast<unsigned>(cap) * total);
+  dim3 grid(8, static_cast<unsigned>(total), static_cast<unsigned>(cap / 8));
   hipStream_t st = static_cast<hipStream_t>(a->stream);
   if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16>(p, a->r, grid, st);
   else launch_rank<_Float16>(p, a->r, grid, st);

@@ -84,7 +84,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // ---- plan workspace layout ------------------------------------------------------------
 // int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles
-// A tile is four words {slot, first position in sorted_idx, token count, 0}.
+// Small tiles are 32-word records (128-byte aligned), big tiles four words; see mlora.h.
 struct PlanLayout {
   int sorted_off, counts_off, offsets_off, small_off, big_off, cap_small, cap_big, total_words;
 };
@@ -97,11 +97,11 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   p.sorted_off = MLORA_PLAN_HEADER_WORDS;
   p.counts_off = p.sorted_off + round_up4(T);
   p.offsets_off = p.counts_off + round_up4(L + 1);
-  p.small_off = p.offsets_off + round_up4(L + 2);
+  p.small_off = (p.offsets_off + round_up4(L + 2) + 31) & ~31;
   p.cap_small = (T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs;
-  p.big_off = p.small_off + 4 * p.cap_small;
+  p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
   p.cap_big = T / MLORA_TILE_BIG + segs;
-  p.total_words = p.big_off + 4 * p.cap_big;
+  p.total_words = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
   return p;
 }
 

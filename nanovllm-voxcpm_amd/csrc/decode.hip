@@ -1,0 +1,348 @@
+// Small-tile form: one workgroup per (small tile, slice, column range).  A small tile is up
+// to sixteen tokens of one slot, described by a self-contained 128-byte record.
+//
+// A launch of this size (a few MB) is bound by memory latency, not bandwidth, so the kernel
+// is built around the number of dependent round trips to memory:
+//   0. the scalar launch arguments arrive preloaded in SGPRs (the kernel takes them as plain
+//      leading arguments for that purpose), so no fetch of the argument block comes first;
+//   1. the plan header, the tile record, this lane's token index and the column-range entry
+//      are fetched together — their addresses depend on nothing but the workgroup index — and
+//      one branch-free test decides whether the workgroup has work;
+//   2. every global load the workgroup needs — its K-range of the x rows and of A[slot], the
+//      B[slot] rows and the y rows of its output spans — is issued before any arithmetic.
+// Both products run on the matrix cores (v_mfma_f32_16x16x32, fp32 accumulate): the sixteen
+// token rows are the MFMA's N (shrink: M) dimension, so a half-empty tile costs nothing but
+// idle multiplier lanes.  The eight wavefronts split K for the shrink, sum their partial tiles
+// through LDS, keep the rank-r intermediate there as a hi + lo pair of operand-precision
+// values, and then each take 64-column spans of the expand; the B rows of a span are
+// interleaved across its four MFMAs so that a lane owns 16 consecutive columns of one token
+// and y is updated with 128-bit accesses.
+#include "common.h"
+#include "launch.h"
+
+namespace mlora {
+
+namespace {
+
+constexpr int kMaxSplits = 64;
+constexpr int kNW = 8;          // wavefronts per workgroup
+constexpr int kSpansAhead = 2;  // output spans per wavefront whose loads are issued up front
+
+template <typename T> struct Mma;
+template <> struct Mma<__bf16> {
+  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.bf, b.bf, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<_Float16> {
+  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.hf, b.hf, c, 0, 0, 0);
+  }
+};
+
+struct DecodeSplit {
+  const void* a;
+  const void* b;
+  int n, y_col, n0, n1;
+};
+
+struct DecodeSplits {
+  DecodeSplit split[kMaxSplits];
+};
+
+// KSPW: k-steps (32 elements of K) each wavefront covers when that is known at compile time
+// (K = 32 * kNW * KSPW), 0 when it has to be worked out from K at run time.
+template <typename T, int R, int KSPW>
+__global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                                            void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
+                                                            int include_long, int T_, int K, int num_slots, float scaling,
+                                                            DecodeSplits splits) {
+  constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
+  constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
+  constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
+  constexpr int NT = kNW * kWave;
+  constexpr int CH = KSPW > 0 ? KSPW : 4;  // k-steps whose loads are in flight together
+
+  __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
+  __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int lr = lane & 15, lg = lane >> 4;
+
+  // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first and
+  // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD: the column ranges of one
+  // tile share an XCD and its L2.
+  const int split_id = blockIdx.y;
+  const int tile = blockIdx.z * 8 + blockIdx.x;
+
+  // ---- round trip 1 ---------------------------------------------------------------------------
+  const int32_t* rec = plan + small_off + tile * MLORA_SMALL_TILE_WORDS;  // tile < capacity: in bounds
+  const int row = rec[MLORA_SMALL_TILE_ROWS + lr];
+  const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);       // slot, count, start, 0
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);      // magic, T, L, ...
+  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
+  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
+  const DecodeSplit sp = splits.split[split_id];
+  const int slot = rec0[0], m = rec0[1];
+  const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
+  // One exit test, evaluated without short-circuit, that consumes everything fetched above
+  // (the token index through its first lane), so that all of it is requested here, together,
+  // instead of piece by piece behind a chain of branches.
+  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) &
+                     int(slot < num_slots) & int(sp.n0 < sp.n1) & int(sp.a != nullptr) & int(sp.b != nullptr) &
+                     int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0);
+  if (!usable) return;
+
+  const bool live = lr < m;  // this lane's token exists
+  const T* xrow = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + lg * 8;
+  const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+  const T* arow[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int rr = rb * 16 + lr;
+    arow[rb] = A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + lg * 8;
+  }
+  const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
+  T* yrow = static_cast<T*>(yv_) + static_cast<int64_t>(row) * ys + sp.y_col + 16 * lg;
+
+  // ---- round trip 2: issue every load ---------------------------------------------------------
+  const int nks = K / 32;
+  const int ks0 = KSPW > 0 ? wave * KSPW : wave * nks / kNW;
+  const int ks1 = KSPW > 0 ? ks0 + KSPW : (wave + 1) * nks / kNW;
+  Pack8 xa[CH], aw[RB][CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int ks = ks0 + i;
+    if (KSPW > 0 || ks < ks1) {
+      xa[i].raw = load128(xrow + ks * 32);  // absent tokens read row 0; their results are never stored
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = load128(arow[rb] + ks * 32);
+    }
+  }
+  Pack8 bop[kSpansAhead][4][KSTEPS], yreg[kSpansAhead][2];
+#pragma unroll
+  for (int s = 0; s < kSpansAhead; ++s) {
+    const int c0 = sp.n0 + (wave + s * kNW) * 64;
+    if (c0 < sp.n1) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
+        n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          // lanes whose chunk lies beyond the rank fetch a valid chunk anyway: their H operand is
+          // zero, and an unconditional load keeps the whole batch of loads in flight together
+          const int kc = (lg + 4 * ks) & (R / 8 - 1);
+          bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        }
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        if (live && c0 + 16 * lg + 8 * half < sp.n1) yreg[s][half].raw = load128(yrow + c0 + 8 * half);
+    }
+  }
+
+  // ---- shrink: H[token, rank] partial over this wavefront's K range ----------------------------
+  f32x4 acc[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    if (KSPW > 0 || ks0 + i < ks1) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+    }
+  }
+  if (KSPW == 0) {
+    for (int ksb = ks0 + CH; ksb < ks1; ksb += CH) {  // K not known at compile time: further batches
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const int ks = ksb + i;
+        if (ks < ks1) {
+          xa[i].raw = load128(xrow + ks * 32);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = load128(arow[rb] + ks * 32);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        if (ksb + i < ks1) {
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+        }
+      }
+    }
+  }
+
+  // Sum the K-partials of the wavefronts.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
+  __syncthreads();
+  for (int e = tid; e < RB * 256; e += NT) {
+    const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+    const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+    if (r < R) {
+      const float v = sum * scaling;
+      const T hi = from_f32<T>(v);
+      s_hi[tok * HSTRIDE + r] = hi;
+      s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+    }
+  }
+  __syncthreads();
+
+  // ---- expand ---------------------------------------------------------------------------------
+  Pack8 hop[KSTEPS], hlo[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    const int kc = lg + 4 * ks;
+    if (kc * 8 < R) {
+      hop[ks].raw = load128(&s_hi[lr * HSTRIDE + kc * 8]);
+      hlo[ks].raw = load128(&s_lo[lr * HSTRIDE + kc * 8]);
+    } else {
+      hop[ks].raw = i32x4{0, 0, 0, 0};
+      hlo[ks].raw = i32x4{0, 0, 0, 0};
+    }
+  }
+
+  auto finish_span = [&](int c0, Pack8(&bo)[4][KSTEPS], Pack8(&yy)[2]) {
+    f32x4 out[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        out[j] = Mma<T>::run(bo[j][ks], hlo[ks], out[j]);
+        out[j] = Mma<T>::run(bo[j][ks], hop[ks], out[j]);
+      }
+    }
+    if (live) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (c0 + 16 * lg + 8 * half < sp.n1) {
+          float yf[8];
+          unpack8<T>(yy[half], yf);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            yf[i] += out[2 * half][i];
+            yf[4 + i] += out[2 * half + 1][i];
+          }
+          Pack8 r;
+          pack8<T>(yf, r);
+          store128(yrow + c0 + 8 * half, r.raw);
+        }
+      }
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < kSpansAhead; ++s) {
+    const int c0 = sp.n0 + (wave + s * kNW) * 64;
+    if (c0 < sp.n1) finish_span(c0, bop[s], yreg[s]);
+  }
+  for (int c0 = sp.n0 + (wave + kSpansAhead * kNW) * 64; c0 < sp.n1; c0 += kNW * 64) {  // wide ranges
+    Pack8 bo[4][KSTEPS], yy[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
+      n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = (lg + 4 * ks) & (R / 8 - 1);
+        bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+      }
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      if (live && c0 + 16 * lg + 8 * half < sp.n1) yy[half].raw = load128(yrow + c0 + 8 * half);
+    finish_span(c0, bo, yy);
+  }
+}
+
+struct Launch {
+  const MloraAddArgs* a;
+  int small_off, include_long;
+  dim3 grid;
+  const DecodeSplits* splits;
+};
+
+template <typename T, int R, int KSPW>
+void launch_one(const Launch& l) {
+  const MloraAddArgs* a = l.a;
+  hipLaunchKernelGGL((decode_kernel<T, R, KSPW>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+                     a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
+                     a->num_slots, a->scaling, *l.splits);
+}
+
+// The steps-per-wavefront specialisations kept: 4 (K = 1024) for every rank and 16 (K = 4096)
+// where the loads of sixteen steps still fit the register file.
+template <typename T, int R>
+void launch_kspw(const Launch& l, int kspw) {
+  if (kspw == 4) return launch_one<T, R, 4>(l);
+  if constexpr (R <= 16) {
+    if (kspw == 16) return launch_one<T, R, 16>(l);
+  }
+  launch_one<T, R, 0>(l);
+}
+
+template <typename T>
+void launch_rank(const Launch& l, int r, int kspw) {
+  switch (r) {
+    case 8: launch_kspw<T, 8>(l, kspw); break;
+    case 16: launch_kspw<T, 16>(l, kspw); break;
+    case 32: launch_kspw<T, 32>(l, kspw); break;
+    default: launch_kspw<T, 64>(l, kspw); break;
+  }
+}
+
+}  // namespace
+
+int launch_decode(const MloraAddArgs* a, bool include_long) {
+  DecodeSplits splits;
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+
+  // Column range per workgroup: every range repeats the shrink of its tile, so ranges are kept
+  // wide enough (default 1024 columns: two 64-column spans per wavefront) for the expand to
+  // outweigh that repeat.
+  int nt = env_int("MLORA_DECODE_NT", 1024);
+  if (nt < 64) nt = 64;
+  nt = (nt + 63) & ~63;
+  int total = 0;
+  for (;;) {
+    total = 0;
+    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
+    if (total <= kMaxSplits) break;
+    nt *= 2;
+  }
+  if (total == 0) return 0;
+  int s = 0;
+  for (int i = 0; i < a->num_slices; ++i) {
+    const MloraSlice& sl = a->slices[i];
+    for (int n0 = 0; n0 < sl.n; n0 += nt) {
+      DecodeSplit& d = splits.split[s++];
+      d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
+      d.n0 = n0; d.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
+    }
+  }
+  int cap = lay.cap_small;
+  if (!include_long) {  // a segment below the threshold is exactly one small tile
+    const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
+    if (segs < cap) cap = segs;
+  }
+  if (cap == 0) return 0;
+  cap = (cap + 7) & ~7;
+  Launch l;
+  l.a = a; l.small_off = lay.small_off; l.include_long = include_long ? 1 : 0; l.splits = &splits;
+  l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>(cap / 8));
+  const int nks = a->k / 32;
+  const int kspw = (nks % kNW == 0) ? nks / kNW : 0;
+  if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16>(l, a->r, kspw);
+  else launch_rank<_Float16>(l, a->r, kspw);
+  return check_launch("mlora_add_lora(small tiles, mfma)");
+}
+
+}  // namespace mlora

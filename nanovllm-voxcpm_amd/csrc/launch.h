@@ -10,13 +10,15 @@ int env_int(const char* name, int fallback);
 // token.hip: one workgroup per token; needs only token_to_slot.
 int launch_token_add(const MloraAddArgs* a);
 
-// bgmv.hip: small tiles (<= 8 tokens of one slot) from the plan.  include_long selects
+// bgmv.hip: small tiles (<= 16 tokens of one slot) on the vector ALU.  include_long selects
 // whether the small tiles of segments at or above the threshold are walked too.
 int launch_bgmv(const MloraAddArgs* a, bool include_long);
 
-// sgmv.hip: MFMA tiles.  all_segments additionally sends the short segments through the
-// 16-row MFMA variant instead of leaving them to launch_bgmv.
+// decode.hip: the same small tiles with both products on the matrix cores.
+int launch_decode(const MloraAddArgs* a, bool include_long);
+
+// sgmv.hip: 64-token MFMA tiles of the segments at or above the threshold.
 bool sgmv_supported(const MloraAddArgs* a);
-int launch_sgmv(const MloraAddArgs* a, bool all_segments);
+int launch_sgmv(const MloraAddArgs* a);
 
 }  // namespace mlora

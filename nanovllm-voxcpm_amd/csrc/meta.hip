@@ -196,21 +196,22 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
     if (p.compact_offsets) p.compact_offsets[i + 1] = 0;
   }
 
-  // Tile lists of the plan.
+  // Tile lists of the plan.  A small-tile record starts with its header and sixteen zeroed row
+  // entries; the scatter below overwrites the entries that exist.
+  i32x4* small = p.plan ? reinterpret_cast<i32x4*>(p.plan + lay.small_off) : nullptr;
   if (p.plan) {
-    i32x4* small = reinterpret_cast<i32x4*>(p.plan + lay.small_off);
     i32x4* big = reinterpret_cast<i32x4*>(p.plan + lay.big_off);
-    for (int q = tid; q < n_short; q += kMetaThreads) {
-      int b = find_bucket(ts_short, NB, q);
-      int j = q - ts_short[b], c = total[b];
-      int left = c - j * MLORA_TILE_SMALL;
-      small[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_SMALL, left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL, 0};
-    }
-    for (int q = tid; q < n_long; q += kMetaThreads) {
-      int b = find_bucket(ts_long, NB, q);
-      int j = q - ts_long[b], c = total[b];
-      int left = c - j * MLORA_TILE_SMALL;
-      small[n_short + q] = i32x4{b - 1, off[b] + j * MLORA_TILE_SMALL, left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL, 0};
+    for (int q = tid; q < n_short + n_long; q += kMetaThreads) {
+      const bool is_short = q < n_short;
+      const int* ts = is_short ? ts_short : ts_long;
+      const int qq = is_short ? q : q - n_short;
+      const int b = find_bucket(ts, NB, qq);
+      const int j = qq - ts[b], c = total[b];
+      const int left = c - j * MLORA_TILE_SMALL;
+      i32x4* rec = small + q * (MLORA_SMALL_TILE_WORDS / 4);
+      rec[0] = i32x4{b - 1, left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL, off[b] + j * MLORA_TILE_SMALL, 0};
+#pragma unroll
+      for (int w = 1; w < MLORA_SMALL_TILE_WORDS / 4; ++w) rec[w] = i32x4{0, 0, 0, 0};
     }
     for (int q = tid; q < n_big; q += kMetaThreads) {
       int b = find_bucket(ts_big, NB, q);
@@ -219,6 +220,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       big[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
     }
   }
+  __syncthreads();
 
   // Stable scatter: every wave walks its span again in token order.  The rank of a token
   // among the equal keys of its 64-token step comes from a ballot; the running cursor of
@@ -244,7 +246,12 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       if (take && key == k) {
         const int r = cursor + __popcll(group & lt_mask);
         if (k >= 1) {
-          if (plan_sorted) plan_sorted[off[k] + r] = t;
+          if (plan_sorted) {
+            plan_sorted[off[k] + r] = t;
+            const int c = total[k];
+            const int q = (c < MLORA_SEGMENT_THRESHOLD ? ts_short[k] : n_short + ts_long[k]) + r / MLORA_TILE_SMALL;
+            p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (r % MLORA_TILE_SMALL)] = t;
+          }
           if (p.sorted_idx) p.sorted_idx[n_neg + off[k] + r] = t;
         } else if (p.sorted_idx) {
           p.sorted_idx[r] = t;

@@ -62,16 +62,17 @@ __global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
   __shared__ __attribute__((aligned(16))) T s_hb[MTB * HSTRIDE];  // leading part of H
   __shared__ __attribute__((aligned(16))) T s_hl[MTB * HSTRIDE];  // remainder H - hi
 
-  const int b = blockIdx.x;
-  const int q = b >> 3;
-  const int split_id = q % p.nsplit;
-  const int tile = (q / p.nsplit) * 8 + (b & 7);
+  // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first, and
+  // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD
+  const int split_id = blockIdx.y;
+  const int tile = blockIdx.z * 8 + blockIdx.x;
+  // header and tile record are fetched together (the record address is in bounds for every
+  // workgroup of the grid, whether or not the tile exists)
   const int32_t* hdr = p.plan;
-  if (hdr[MLORA_PLAN_MAGIC] != MLORA_PLAN_MAGIC_VALUE || hdr[MLORA_PLAN_NUM_TOKENS] != p.T ||
-      hdr[MLORA_PLAN_MAX_SLOTS] != p.num_slots)
-    return;
-  if (tile >= hdr[p.count_word]) return;
   const i32x4 td = reinterpret_cast<const i32x4*>(p.plan + p.tiles_off)[tile];
+  const int magic = hdr[MLORA_PLAN_MAGIC], plan_t = hdr[MLORA_PLAN_NUM_TOKENS], plan_l = hdr[MLORA_PLAN_MAX_SLOTS];
+  const int n_tiles = hdr[p.count_word];
+  if (magic != MLORA_PLAN_MAGIC_VALUE || plan_t != p.T || plan_l != p.num_slots || tile >= n_tiles) return;
   const int slot = td[0], start = td[1], m = td[2];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -251,29 +252,26 @@ int fill_splits(const MloraAddArgs* a, int nt, SgmvSplit* out) {
   return total;
 }
 
-int launch_tiles(const MloraAddArgs* a, bool short_tiles) {
+}  // namespace
+
+bool sgmv_supported(const MloraAddArgs* a) { return a->k % 32 == 0 && a->k >= 32; }
+
+// 64-token tiles of the segments at or above the threshold.
+int launch_sgmv(const MloraAddArgs* a) {
   SgmvParams p;
   p.x = a->x; p.y = a->y; p.xs = a->x_stride; p.ys = a->y_stride; p.plan = a->plan;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
   p.sorted_off = lay.sorted_off;
   p.T = a->num_tokens; p.K = a->k; p.num_slots = a->num_slots; p.scaling = a->scaling;
-  const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
-  int cap;
-  if (short_tiles) {
-    p.tiles_off = lay.small_off; p.count_word = MLORA_PLAN_TILES_SHORT;
-    const int per_seg = (MLORA_SEGMENT_THRESHOLD - 1 + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
-    cap = segs * per_seg < lay.cap_small ? segs * per_seg : lay.cap_small;
-  } else {
-    p.tiles_off = lay.big_off; p.count_word = MLORA_PLAN_TILES_LONG_BIG;
-    cap = lay.cap_big;
-  }
+  p.tiles_off = lay.big_off; p.count_word = MLORA_PLAN_TILES_LONG_BIG;
+  int cap = lay.cap_big;
   if (cap == 0) return 0;
   int cols = 0;
   for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
   if (cols == 0) return 0;
   // Aim for a few workgroups per CU: tiles x column ranges of about 1024 workgroups.
   const int target = env_int("MLORA_SGMV_WGS", 1024);
-  const int est_tiles = short_tiles ? cap : a->num_tokens / MLORA_TILE_BIG + 1;
+  const int est_tiles = a->num_tokens / MLORA_TILE_BIG + 1;
   int nt = env_int("MLORA_SGMV_NT", 0);
   if (nt <= 0) {
     const long long want = static_cast<long long>(cols) * est_tiles / (target > 0 ? target : 1);
@@ -281,28 +279,11 @@ int launch_tiles(const MloraAddArgs* a, bool short_tiles) {
   }
   p.nsplit = fill_splits(a, nt, p.split);
   cap = (cap + 7) & ~7;
-  dim3 grid(static_cast<unsigned>(cap) * p.nsplit);
+  dim3 grid(8, static_cast<unsigned>(p.nsplit), static_cast<unsigned>(cap / 8));
   hipStream_t st = static_cast<hipStream_t>(a->stream);
-  if (short_tiles) {
-    if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16, 16>(p, a->r, grid, st);
-    else launch_rank<_Float16, 16>(p, a->r, grid, st);
-  } else {
-    if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16, MLORA_TILE_BIG>(p, a->r, grid, st);
-    else launch_rank<_Float16, MLORA_TILE_BIG>(p, a->r, grid, st);
-  }
-  return check_launch(short_tiles ? "mlora_add_lora(mfma, short tiles)" : "mlora_add_lora(mfma, big tiles)");
-}
-
-}  // namespace
-
-bool sgmv_supported(const MloraAddArgs* a) { return a->k % 32 == 0 && a->k >= 32; }
-
-int launch_sgmv(const MloraAddArgs* a, bool all_segments) {
-  if (all_segments) {
-    int rc = launch_tiles(a, /*short_tiles=*/true);
-    if (rc) return rc;
-  }
-  return launch_tiles(a, /*short_tiles=*/false);
+  if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16, MLORA_TILE_BIG>(p, a->r, grid, st);
+  else launch_rank<_Float16, MLORA_TILE_BIG>(p, a->r, grid, st);
+  return check_launch("mlora_add_lora(mfma, big tiles)");
 }
 
 }  // namespace mlora

@@ -39,7 +39,8 @@ PLAN_HEADER_WORDS = 16
     PLAN_MAX_SEGMENT,
 ) = range(11)
 PLAN_MAGIC_VALUE = 0x4D4C5031
-SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 8, 64
+SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 16, 64
+SMALL_TILE_WORDS, SMALL_TILE_ROWS, BIG_TILE_WORDS = 32, 4, 4
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 

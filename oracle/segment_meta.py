@@ -103,7 +103,7 @@ def graph_layout(token_to_slot: list[int] | None, no_lora_flag: bool, max_rows: 
                 num_tokens_per_slot=counts, slot_start_offsets=offsets)
 
 
-def plan_tiles(token_to_slot: list[int], max_slots: int, threshold: int = 16, small: int = 8, big: int = 64):
+def plan_tiles(token_to_slot: list[int], max_slots: int, threshold: int = 16, small: int = 16, big: int = 64):
     """Work lists the apply kernels walk, derived from the engine layout: for every slot in
     ascending order its segment is cut into tiles (slot, first position in sorted_idx, count).
     Returns (short_small, long_small, long_big): small tiles of segments shorter than

@@ -60,10 +60,10 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
         assert int(got[name]) == C.sizeof(st), name
         for field, _ in st._fields_:
             assert int(got[f"{name}.{field}"]) == getattr(st, field).offset, f"{name}.{field}"
-    assert _hip.MAX_SLICES == 8 and _hip.TILE_SMALL == 8 and _hip.TILE_BIG == 64 and _hip.SEGMENT_THRESHOLD == 16
+    assert _hip.MAX_SLICES == 8 and _hip.TILE_SMALL == 16 and _hip.TILE_BIG == 64 and _hip.SEGMENT_THRESHOLD == 16
     text = HEADER.read_text()
     for macro, value in (("MLORA_MAX_SLICES", 8), ("MLORA_MAX_SLOTS", _hip.MAX_SLOTS), ("MLORA_MAX_RANK", _hip.MAX_RANK),
-                         ("MLORA_TILE_SMALL", 8), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
+                         ("MLORA_TILE_SMALL", 16), ("MLORA_SMALL_TILE_WORDS", _hip.SMALL_TILE_WORDS), ("MLORA_BIG_TILE_WORDS", _hip.BIG_TILE_WORDS), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
                          ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS)):
         assert re.search(rf"#define {macro} {value}\b", text), macro
 
