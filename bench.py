@@ -12,7 +12,7 @@ not from the 256 MB last-level cache.
 Prints ONE JSON line.  `value` = algorithmic bytes of a step / time of a step, inputs
 resident in HBM, the step replayed as a captured graph (decode runs under graph replay in
 the serving engine).  `roofline` is quoted for the kernel every launch of the step uses
-(bgmv_kernel<bf16, rank 16>): algorithmic bytes of an average launch / average launch time.
+(decode_kernel<bf16, rank 16>, the small-tile MFMA kernel): algorithmic bytes of an average launch / average launch time.
 `cpu_baseline` times the reference's torch formulation (per-token F.linear loop) of one layer
 of the same workload on the host cores.
 """
@@ -179,6 +179,9 @@ def main() -> None:
     ap.add_argument("--hot-layers", type=int, default=0,
                     help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
                          "(N=1 keeps the working set inside the last-level cache); 0 = every layer has its own")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
+                         "that rocprof byte counters of the same run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; every box in this pool has one (use --gpus 1)")
@@ -199,6 +202,13 @@ def main() -> None:
     names = [args.only] if args.only else list(ORDER)
     per_proj = {n: algorithmic_bytes(layers[0][n][0].k, layers[0][n][0].widths, t_lora, used, RANK, NUM_TOKENS) for n in names}
     step_bytes = NUM_LAYERS * sum(per_proj.values())
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # 256 MiB read + 256 MiB written by one elementwise copy kernel
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(3):
         step()
@@ -255,13 +265,16 @@ def main() -> None:
         "us_per_launch_by_projection": per_proj_us,
         "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
         "roofline": {
-            "kernel": "bgmv_kernel<bf16, rank 16>" if args.form in ("auto", "bgmv") else args.form,
+            "kernel": {"auto": "decode_kernel<bf16,16>", "mfma": "decode_kernel<bf16,16>", "bgmv": "bgmv_kernel<bf16,16>"}.get(args.form, args.form),
             "bound": "hbm",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # HBM bytes per average launch from the two rocprofv3 --pmc runs of this workload
+            # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 256 MiB copy in the same runs);
+            # only quoted for the configuration those runs covered
+            "traffic": 9670000 if (args.form == "auto" and not args.only and not args.hot_layers) else None,
             "bytes_per_launch": round(launch_bytes),
             "us_per_launch": round(launch_us, 3),
         },
