@@ -1,20 +1,24 @@
 """Benchmark of the fused multi-LoRA apply on one MI355X.
 
-Workload (BASELINE.json configs[1], "decode BGMV bf16"): one decode step of a 24-layer
+Default workload (BASELINE.json configs[1], "decode BGMV bf16"): one decode step of a 24-layer
 decoder — 256 tokens (one per sequence), 32 resident adapters of rank 16, adapter ids uniform,
 LoRA applied to the stacked q|k|v [1024|256|256], o [1024->1024], gate|up [1024->2x4096] and
-down [4096->1024] projections of every layer.  A "step" is the LoRA work of that decode step:
-one on-device metadata build plus 24 x 4 fused shrink+expand launches, issued through the
-same backend entry (`LoRABackend.add_lora`) the LoRA linears call.  Every layer owns its
-weights and its activation buffers (about 0.75 GB in total), so a step streams from HBM and
-not from the 256 MB last-level cache.
+down [4096->1024] projections of every layer.  A "step" is the LoRA work of that step: one
+on-device metadata build plus 24 x 4 fused shrink+expand calls, issued through the same backend
+entry (`LoRABackend.add_lora`) the LoRA linears call.  Every layer owns its weights and its
+activation buffers (about 0.75 GB in total), so a step streams from HBM and not from the 256 MB
+last-level cache.
 
-Prints ONE JSON line.  `value` = algorithmic bytes of a step / time of a step, inputs
-resident in HBM, the step replayed as a captured graph (decode runs under graph replay in
-the serving engine).  `roofline` is quoted for the kernel every launch of the step uses
-(decode_kernel<bf16, rank 16>, the small-tile MFMA kernel): algorithmic bytes of an average launch / average launch time.
-`cpu_baseline` times the reference's torch formulation (per-token F.linear loop) of one layer
-of the same workload on the host cores.
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / time of a step, inputs resident
+in HBM, the step replayed as a captured graph (decode runs under graph replay in the serving
+engine).  `roofline` is quoted for the kernel that does the work of the step: algorithmic bytes
+of an average launch / average launch time.  `cpu_baseline` times the reference's torch
+formulation (per-token F.linear loop) of one layer of the same workload on the host cores.
+
+`--workload prefill` (configs[2]: 16 sequences of 64..1024 tokens, 8 adapters of rank 64, a
+quarter of the sequences without adapter) and `--workload mixed` (configs[3]: 2 x 2048-token
+chunks + 4096 decodes, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity) time the
+same 24 x 4 calls on those batches; they are measurement aids, the driver runs the default.
 """
 
 from __future__ import annotations
@@ -31,9 +35,22 @@ for p in (ROOT, ROOT / "nanovllm-voxcpm_amd"):
     if str(p) not in sys.path:
         sys.path.insert(0, str(p))
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-NUM_LAYERS, NUM_TOKENS, NUM_SLOTS, RANK = 24, 256, 32, 16
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16, published
+NUM_LAYERS = 24
 ORDER = ("qkv", "o", "gate_up", "down")
+
+WORKLOADS = {
+    "decode": dict(slots=32, rank=16, distinct_layers=24,
+                   text="decode BGMV bf16 (BASELINE configs[1]): 256 tokens, 32 adapters, rank 16, "
+                        "qkv/o/gate_up/down x 24 layers, per-layer weights and activations"),
+    "prefill": dict(slots=8, rank=64, distinct_layers=4,
+                    text="prefill SGMV bf16 (BASELINE configs[2]): 16 sequences of 64..1024 tokens, 8 adapters, "
+                         "rank 64, 25% of sequences without adapter, qkv/o/gate_up/down x 24 layers"),
+    "mixed": dict(slots=128, rank=64, distinct_layers=4,
+                  text="mixed bf16 (BASELINE configs[3]): 2 x 2048-token chunks + 4096 decodes, 128 adapters of "
+                       "ranks {8,16,32,64} padded to 64, Zipf(1.1), qkv/o/gate_up/down x 24 layers"),
+}
 
 
 def algorithmic_bytes(k: int, widths: list[int], t_lora: int, used_slots: int, rank: int, num_tokens: int) -> int:
@@ -43,25 +60,45 @@ def algorithmic_bytes(k: int, widths: list[int], t_lora: int, used_slots: int, r
     return 2 * (t_lora * k + used_slots * s * rank * k + used_slots * rank * n + 2 * t_lora * n) + 4 * num_tokens
 
 
-def build_workload(device: str):
+def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int) -> int:
+    return 2 * t_lora * rank * (len(widths) * k + sum(widths))
+
+
+def build_workload(name: str, device: str):
+    """Per-layer (projection weights, x, y) for the distinct layers of the workload and the
+    batch's slot vector.  Layers beyond the distinct ones reuse buffers round-robin (the distinct
+    set alone exceeds the 256 MB last-level cache)."""
     import torch
 
     from nanovllm_voxcpm_amd import synthetic
 
-    layers = []
-    for layer in range(NUM_LAYERS):
+    spec = WORKLOADS[name]
+    if name == "decode":
+        slots = synthetic.decode_slots(256, spec["slots"], seed=7)
+        ranks = None
+    elif name == "prefill":
+        slots, _ = synthetic.prefill_slots(16, spec["slots"], seed=301)
+        ranks = None
+    else:
+        slots = synthetic.mixed_slots(seed=402)
+        ranks = synthetic.heterogeneous_ranks(spec["slots"], seed=400)
+    num_tokens = slots.numel()
+    distinct = []
+    for layer in range(spec["distinct_layers"]):
         entry = {}
-        for j, name in enumerate(ORDER):
-            proj = synthetic.make_projection(name, NUM_SLOTS, RANK, torch.bfloat16, seed=1000 + 16 * layer + j, device=device)
-            x, y = synthetic.make_activations(NUM_TOKENS, proj.k, sum(proj.widths), torch.bfloat16, seed=5000 + 16 * layer + j, device=device)
-            entry[name] = (proj, x, y)
-        layers.append(entry)
-    slots = synthetic.decode_slots(NUM_TOKENS, NUM_SLOTS, seed=7).to(device)
-    return layers, slots
+        for j, proj_name in enumerate(ORDER):
+            proj = synthetic.make_projection(proj_name, spec["slots"], spec["rank"], torch.bfloat16,
+                                             seed=1000 + 16 * layer + j, device=device, true_ranks=ranks)
+            x, y = synthetic.make_activations(num_tokens, proj.k, sum(proj.widths), torch.bfloat16,
+                                              seed=5000 + 16 * layer + j, device=device)
+            entry[proj_name] = (proj, x, y)
+        distinct.append(entry)
+    layers = [distinct[i % len(distinct)] for i in range(NUM_LAYERS)]
+    return layers, slots.to(device)
 
 
 def make_step(layers, slots, form: str, only: str | None = None):
-    """Returns step(): metadata build + every fused apply of one decode step, via the backend."""
+    """Returns step(): metadata build + every fused apply of one step, via the backend."""
     from nanovllm_voxcpm_amd.lora import HipLoRABackend, LoRAMetadata
 
     backend = HipLoRABackend(form)
@@ -112,7 +149,7 @@ def capture(step):
     return graph
 
 
-def cpu_baseline(layers, slots, budget_s: float = 20.0) -> dict:
+def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
     """The reference's torch LoRA computation on the host: per-token F.linear(F.linear(x_t, A[s]),
     B[s]) accumulate (oracle.per_token_add_lora), fp32, one layer of the same workload, all host
     threads.  Reported in the metric's unit: algorithmic bytes of what was run / time."""
@@ -123,13 +160,14 @@ def cpu_baseline(layers, slots, budget_s: float = 20.0) -> dict:
     threads = torch.get_num_threads()
     entry = layers[0]
     slots_cpu = slots.cpu()
+    num_tokens = slots_cpu.numel()
     work = []
     for name in ORDER:
         proj, x, y = entry[name]
         work.append((proj, x.cpu().float(), y.cpu().float(), [a.cpu().float() for a in proj.a], [b.cpu().float() for b in proj.b]))
     used = int(torch.unique(slots_cpu[slots_cpu >= 0]).numel())
     t_lora = int((slots_cpu >= 0).sum())
-    layer_bytes = sum(algorithmic_bytes(p.k, p.widths, t_lora, used, RANK, NUM_TOKENS) for p, *_ in work)
+    layer_bytes = sum(algorithmic_bytes(p.k, p.widths, t_lora, used, rank, num_tokens) for p, *_ in work)
 
     def one_layer():
         for proj, x, y, a, b in work:
@@ -158,7 +196,7 @@ def cpu_baseline(layers, slots, budget_s: float = 20.0) -> dict:
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"1 of {NUM_LAYERS} layers of the same decode step (4 projections, 256 tokens, 32 adapters, rank 16), fp32, "
+        "sample": f"1 of {NUM_LAYERS} layers of the same step (4 projections, {num_tokens} tokens, rank {rank}), fp32, "
                   f"per-token torch loop, median of {len(times)} runs",
         "us_per_layer": round(med * 1e6, 1),
         "us_per_step_extrapolated": round(med * 1e6 * NUM_LAYERS, 1),
@@ -172,13 +210,14 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="decode", choices=sorted(WORKLOADS))
     ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | sgmv | token")
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--hot-layers", type=int, default=0,
                     help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
-                         "(N=1 keeps the working set inside the last-level cache); 0 = every layer has its own")
+                         "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
                          "that rocprof byte counters of the same run are scaled by")
@@ -192,36 +231,45 @@ def main() -> None:
         sys.exit("bench.py: no ROCm GPU visible")
     device = "cuda:0"
     torch.cuda.set_device(0)
-    layers, slots = build_workload(device)
+    spec = WORKLOADS[args.workload]
+    rank = spec["rank"]
+    layers, slots = build_workload(args.workload, device)
     if args.hot_layers > 0:
         layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
     step, launches = make_step(layers, slots, args.form, args.only)
 
+    num_tokens = slots.numel()
     used = int(torch.unique(slots[slots >= 0]).numel())
     t_lora = int((slots >= 0).sum())
     names = [args.only] if args.only else list(ORDER)
-    per_proj = {n: algorithmic_bytes(layers[0][n][0].k, layers[0][n][0].widths, t_lora, used, RANK, NUM_TOKENS) for n in names}
+    shapes = {n: layers[0][n][0] for n in names}
+    per_proj = {n: algorithmic_bytes(p.k, p.widths, t_lora, used, rank, num_tokens) for n, p in shapes.items()}
+    per_proj_flops = {n: algorithmic_flops(p.k, p.widths, t_lora, rank) for n, p in shapes.items()}
     step_bytes = NUM_LAYERS * sum(per_proj.values())
+    step_flops = NUM_LAYERS * sum(per_proj_flops.values())
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
-        dst.copy_(src)  # 256 MiB read + 256 MiB written by one elementwise copy kernel
+        dst.copy_(src)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(3):
+    heavy = args.workload != "decode"
+    steps = args.steps if not heavy else max(3, min(args.steps, 30))
+    warmup = args.warmup if not heavy else max(1, min(args.warmup, 3))
+    for _ in range(2):
         step()
     torch.cuda.synchronize()
-    eager_ms = time_region(step, max(5, min(args.steps, 50)))
+    eager_ms = time_region(step, max(3, min(steps, 50)))
     if args.eager:
         runner = step
     else:
         graph = capture(step)
         runner = graph.replay
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         runner()
-    ms = time_region(runner, args.steps)
+    ms = time_region(runner, steps)
 
     # per-projection time: the same step restricted to one projection (24 launches)
     per_proj_us = {}
@@ -229,21 +277,26 @@ def main() -> None:
         for n in ORDER:
             sub, cnt = make_step(layers, slots, args.form, n)
             g = capture(sub)
-            for _ in range(5):
+            for _ in range(2):
                 g.replay()
-            per_proj_us[n] = round(time_region(g.replay, max(20, args.steps // 4)) * 1e3 / cnt, 3)
+            per_proj_us[n] = round(time_region(g.replay, max(3, steps // 4)) * 1e3 / cnt, 3)
 
     value = step_bytes / (ms * 1e-3) / 1e9
     launch_bytes = step_bytes / launches
     launch_us = ms * 1e3 / launches
     achieved = launch_bytes / (launch_us * 1e-6) / 1e9
+    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers
+    kernel = {"decode": "decode_kernel<bf16,16>", "prefill": "sgmv_kernel<bf16,64,64>",
+              "mixed": "sgmv_kernel<bf16,64,64> + decode_kernel<bf16,64>"}[args.workload]
+    if args.form == "bgmv":
+        kernel = "bgmv_kernel<bf16>"
     out = {
         "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -251,36 +304,39 @@ def main() -> None:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": "decode BGMV bf16 (BASELINE configs[1]): 256 tokens, 32 adapters, rank 16, "
-                        "qkv/o/gate_up/down x 24 layers, per-layer weights and activations",
-            "tokens": NUM_TOKENS, "adapters": NUM_SLOTS, "rank": RANK, "layers": NUM_LAYERS,
-            "projections": names, "form": args.form, "launch": "eager" if args.eager else "graph replay",
-            "distinct_layer_buffers": args.hot_layers or NUM_LAYERS,
+            "workload": spec["text"],
+            "tokens": num_tokens, "tokens_with_adapter": t_lora, "adapters": spec["slots"], "adapters_in_batch": used,
+            "rank": rank, "layers": NUM_LAYERS, "projections": names, "form": args.form,
+            "launch": "eager" if args.eager else "graph replay",
+            "distinct_layer_buffers": args.hot_layers or spec["distinct_layers"],
         },
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-        "us_per_decode_step": round(ms * 1e3, 2),
-        "us_per_decode_step_eager": round(eager_ms * 1e3, 2),
+        "us_per_step": round(ms * 1e3, 2),
+        "us_per_step_eager": round(eager_ms * 1e3, 2),
         "algorithmic_bytes_per_step": step_bytes,
+        "algorithmic_flops_per_step": step_flops,
+        "tflops": round(step_flops / (ms * 1e-3) / 1e12, 2),
+        "pct_of_mfma_bf16_peak": round(100 * step_flops / (ms * 1e-3) / 1e12 / MFMA_BF16_TFLOPS, 3),
         "launches_per_step": launches + 1,
         "us_per_launch_by_projection": per_proj_us,
         "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
         "roofline": {
-            "kernel": {"auto": "decode_kernel<bf16,16>", "mfma": "decode_kernel<bf16,16>", "bgmv": "bgmv_kernel<bf16,16>"}.get(args.form, args.form),
+            "kernel": kernel,
             "bound": "hbm",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per average launch from the two rocprofv3 --pmc runs of this workload
+            # HBM bytes per average launch from the two rocprofv3 --pmc runs of the default workload
             # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 256 MiB copy in the same runs);
             # only quoted for the configuration those runs covered
-            "traffic": 9670000 if (args.form == "auto" and not args.only and not args.hot_layers) else None,
+            "traffic": 9670000 if default_run else None,
             "bytes_per_launch": round(launch_bytes),
             "us_per_launch": round(launch_us, 3),
         },
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(layers, slots)
+    if not args.no_cpu_baseline and args.workload == "decode":
+        out["cpu_baseline"] = cpu_baseline(layers, slots, rank)
     print(json.dumps(out))
 
 

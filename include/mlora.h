@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MLORA_ABI_VERSION 1
+#define MLORA_ABI_VERSION 2
 
 /* element types of x / y / A / B */
 #define MLORA_DTYPE_F32 0
@@ -36,7 +36,8 @@ extern "C" {
 #define MLORA_FORM_AUTO 0  /* library chooses from shapes and the plan */
 #define MLORA_FORM_TOKEN 1 /* one workgroup per token, any shape or dtype; needs no plan */
 #define MLORA_FORM_BGMV 2  /* small tiles (<= 16 tokens of one slot), packed dot2 + wave64 reductions */
-#define MLORA_FORM_SGMV 3  /* 64-token MFMA tiles for segments >= threshold, small MFMA tiles for the rest */
+#define MLORA_FORM_SGMV 3  /* 64-token MFMA tiles for segments >= threshold (shrink launch + expand launch through
+                              the workspace), small MFMA tiles for the rest */
 #define MLORA_FORM_MFMA 4  /* small tiles for every segment, both products on the matrix cores */
 
 /* error codes (negative) */
@@ -72,7 +73,7 @@ typedef struct MloraAddArgs {
   int64_t x_stride;
   int64_t y_stride;
   const int32_t* token_to_slot; /* [T] on device */
-  const int32_t* plan;    /* workspace filled by mlora_plan_build for this token_to_slot, or NULL
+  const int32_t* plan;    /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
                              (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it) */
   int32_t num_tokens;     /* T */
   int32_t k;              /* K, input features */
@@ -83,9 +84,18 @@ typedef struct MloraAddArgs {
   int32_t form;           /* MLORA_FORM_* */
   float scaling;
   MloraSlice slices[MLORA_MAX_SLICES];
+  void* workspace;        /* device scratch for the rank-r intermediate of MLORA_FORM_SGMV, 16-byte
+                             aligned, or NULL (AUTO then keeps to the small-tile form).  Counterpart of
+                             the [S, T, r] buffer the reference allocates between its two kernels
+                             (reference: nanovllm_voxcpm/lora.py:299-381).  Contents need not be kept
+                             between calls; calls that share it must be ordered on one stream. */
+  int64_t workspace_bytes; /* >= mlora_add_workspace_bytes(T, num_slices, r, dtype) to be used */
 } MloraAddArgs;
 
 int mlora_add_lora(const MloraAddArgs* args);
+
+/* Bytes of MloraAddArgs.workspace that let mlora_add_lora use MLORA_FORM_SGMV. */
+size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);
 
 /* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0
  * for rows with s_t < 0 (the reference zero-fills the buffer first).

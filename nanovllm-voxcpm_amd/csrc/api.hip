@@ -94,8 +94,10 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     // tiles for the long segments and 16-token tiles for the rest.
     if (!vec) form = MLORA_FORM_TOKEN;
     else if (!sgmv_supported(a)) form = MLORA_FORM_BGMV;
-    else form = a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) ? MLORA_FORM_MFMA : MLORA_FORM_SGMV;
+    else if (a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
+    else form = MLORA_FORM_SGMV;
   }
+  if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && vec && sgmv_supported(a) && !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
   switch (form) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
@@ -106,6 +108,11 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     case MLORA_FORM_MFMA: {
       if (!vec || !sgmv_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
+      if (!sgmv_workspace_ok(a)) {
+        set_error("mlora_add_lora: SGMV form needs a 16-byte aligned workspace of %zu bytes and no empty slice",
+                  sgmv_workspace_bytes(a->num_tokens, a->num_slices, a->r, a->dtype));
+        return MLORA_E_INVALID;
+      }
       int rc = launch_decode(a, /*include_long=*/false);
       if (rc) return rc;
       return launch_sgmv(a);
@@ -113,6 +120,10 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   }
   set_error("mlora_add_lora: unreachable form %d", form);
   return MLORA_E_INVALID;
+}
+
+extern "C" size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype) {
+  return sgmv_workspace_bytes(num_tokens, num_slices, r, dtype);
 }
 
 extern "C" uint64_t mlora_stream_capture_id(void* stream) {
@@ -130,5 +141,5 @@ extern "C" int mlora_abi_version(void) { return MLORA_ABI_VERSION; }
 extern "C" const char* mlora_last_error(void) { return g_error; }
 
 extern "C" const char* mlora_build_info(void) {
-  return "mlora gfx950 (wave64; small tiles: MFMA 16x16x32 or dot2 + wave reductions; big tiles: MFMA 16x16x32) built " __DATE__ " " __TIME__;
+  return "mlora gfx950 (wave64; small tiles: MFMA 16x16x32 or dot2 + wave reductions; big tiles: MFMA 16x16x32 shrink + expand) built " __DATE__ " " __TIME__;
 }

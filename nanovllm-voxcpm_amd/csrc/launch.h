@@ -17,8 +17,11 @@ int launch_bgmv(const MloraAddArgs* a, bool include_long);
 // decode.hip: the same small tiles with both products on the matrix cores.
 int launch_decode(const MloraAddArgs* a, bool include_long);
 
-// sgmv.hip: 64-token MFMA tiles of the segments at or above the threshold.
+// sgmv.hip: 64-token MFMA tiles of the segments at or above the threshold, as a shrink launch
+// and an expand launch that meet in the caller's workspace.
 bool sgmv_supported(const MloraAddArgs* a);
+bool sgmv_workspace_ok(const MloraAddArgs* a);
+size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype);
 int launch_sgmv(const MloraAddArgs* a);
 
 }  // namespace mlora

@@ -1,16 +1,28 @@
-// SGMV form: one workgroup per (segment tile, slice, column range), both products on the
-// matrix cores (v_mfma_f32_16x16x32 bf16 / f16, fp32 accumulate).
-//   shrink  — H[tokens x r] = X_tile . A[slot]^T.  The four wavefronts split K; every lane
-//             feeds the MFMA straight from 128-bit global loads of x rows and A rows, so
-//             neither operand is read twice by a workgroup.  The four partial tiles are
-//             summed through LDS and the rank-r intermediate is kept there as a hi + lo pair of
-//             operand-precision values (about 16 significant bits), so the expand loses nothing
-//             that would show after the final rounding of y.
-//   expand  — OUT^T[cols x tokens] = B[slot] . H^T.  The B rows fed to the four MFMAs of a
-//             64-column span are interleaved (row rho of MFMA j is column 16*(rho/4) + 4j + rho%4)
-//             so that a lane ends up with 16 consecutive output columns of one token: y is
-//             read, accumulated and written with 128-bit accesses, a full 128-byte line per
-//             token per quarter-wave, with no transposition pass.
+// SGMV form for the 64-token tiles of long segments: two launches that meet in a small
+// workspace, both on the matrix cores (v_mfma_f32_16x16x32 bf16 / f16, fp32 accumulate).
+//
+//   shrink — H^T[rank x tokens] = A[slot] . X_tile^T for a (tile, slice, K part).  What bounds
+//            this product is the number of bytes a compute unit pulls through its vector L1
+//            (hits cost as much as misses there), so each operand element passes through it once
+//            per workgroup: the A[slot] slab of the workgroup's K part is copied to LDS with
+//            row-contiguous 128-bit loads and shared by the four wavefronts, each of which owns
+//            sixteen tokens of the tile and streams their x rows straight from global memory
+//            into the MFMA operand layout, a whole batch of k-steps in flight at a time.  No
+//            wavefront shares a sum with another, so the accumulators go straight to the
+//            workspace as fp32; when K is split across workgroups each part writes its own
+//            partial.  x is read from HBM once per slice.
+//   expand — OUT^T[cols x tokens] = B[slot] . H^T for a (tile, column range).  The H tile is
+//            staged in LDS once (K partials summed, scaled, and split into a hi + lo pair of
+//            operand-precision values, about 16 significant bits: the expand loses nothing that
+//            would show after the final rounding of y); a wavefront owns 64-column spans: it
+//            fetches the span's B rows and the y rows of all four 16-token blocks up front, then
+//            runs the MFMAs block by block and writes y back.  The B rows fed to the four MFMAs
+//            of a span are interleaved (row rho of MFMA j is column 16*(rho/4) + 4j + rho%4) so
+//            that a lane ends up with 16 consecutive output columns of one token: y moves in
+//            128-bit accesses, a full 128-byte line per token per wavefront, with no
+//            transposition pass.
+// Splitting the two products means no column range repeats the shrink of its tile, and each
+// kernel keeps only its own operands in registers (more wavefronts per SIMD to hide latency).
 #include "common.h"
 #include "launch.h"
 
@@ -18,9 +30,8 @@ namespace mlora {
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / kWave;
 constexpr int kMaxSplits = 64;
+constexpr int kExpandWaves = 4;
 
 template <typename T> struct Mma;
 template <> struct Mma<__bf16> {
@@ -34,184 +45,275 @@ template <> struct Mma<_Float16> {
   }
 };
 
-struct SgmvSplit {
-  const void* a;
+struct ShrinkSlices {
+  const void* a[MLORA_MAX_SLICES];
+};
+
+struct ExpandSplit {
   const void* b;
-  int n, y_col, n0, n1;
+  int n, y_col, n0, n1, slice, pad;
 };
 
-struct SgmvParams {
-  const void* x;
-  void* y;
-  int64_t xs, ys;
-  const int32_t* plan;
-  int sorted_off, tiles_off, count_word;
-  int T, K, num_slots, nsplit;
-  float scaling;
-  SgmvSplit split[kMaxSplits];
+struct ExpandSplits {
+  ExpandSplit split[kMaxSplits];
 };
 
-template <typename T, int R, int MTB>
-__global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
-  constexpr int TB = MTB / 16;                  // 16-token blocks per tile
-  constexpr int RB = (R + 15) / 16;             // 16-rank blocks
-  constexpr int KSTEPS = (R + 31) / 32;         // MFMA k-steps of the expand
-  constexpr int HSTRIDE = R + 8;                // padded LDS row of the intermediate
+// ---- shrink -------------------------------------------------------------------------------------
+// grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  KR: columns of
+// K per LDS slab (the workgroup's K part is a whole number of slabs).
+constexpr int kShrinkWaves = 4;
 
-  __shared__ __attribute__((aligned(16))) float s_red[kWaves * RB * 64 * 4];
-  __shared__ __attribute__((aligned(16))) T s_hb[MTB * HSTRIDE];  // leading part of H
-  __shared__ __attribute__((aligned(16))) T s_hl[MTB * HSTRIDE];  // remainder H - hi
+template <typename T, int R, int KR>
+__global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                                                          float* __restrict__ hws, int64_t xs, int tiles_off,
+                                                                          int sorted_off, int T_, int K, int num_slots, int num_slices,
+                                                                          int ksplit, int krange, ShrinkSlices sl) {
+  constexpr int RB = (R + 15) / 16;      // 16-rank blocks
+  constexpr int NT = kShrinkWaves * kWave;
+  constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
+  constexpr int CPR = KR / 8;            // 16-byte chunks per slab row
+  constexpr int TOTAL = R * CPR;         // chunks per slab
+  constexpr int CHUNKS = (TOTAL + NT - 1) / NT;  // chunks each thread copies per slab
+  constexpr int SB = CHUNKS < 8 ? CHUNKS : 8;    // chunks in flight together
+  constexpr int KS = KR / 32;            // k-steps per slab
+  constexpr int XB = KS < 16 ? KS : 16;  // x loads in flight together
+  static_assert(CHUNKS % SB == 0 && KS % XB == 0, "slab shape");
 
-  // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first, and
-  // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD
-  const int split_id = blockIdx.y;
-  const int tile = blockIdx.z * 8 + blockIdx.x;
-  // header and tile record are fetched together (the record address is in bounds for every
-  // workgroup of the grid, whether or not the tile exists)
-  const int32_t* hdr = p.plan;
-  const i32x4 td = reinterpret_cast<const i32x4*>(p.plan + p.tiles_off)[tile];
-  const int magic = hdr[MLORA_PLAN_MAGIC], plan_t = hdr[MLORA_PLAN_NUM_TOKENS], plan_l = hdr[MLORA_PLAN_MAX_SLOTS];
-  const int n_tiles = hdr[p.count_word];
-  if (magic != MLORA_PLAN_MAGIC_VALUE || plan_t != p.T || plan_l != p.num_slots || tile >= n_tiles) return;
-  const int slot = td[0], start = td[1], m = td[2];
+  __shared__ __attribute__((aligned(16))) T s_a[R * ASTRIDE];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
-  const int32_t* sorted = p.plan + p.sorted_off + start;
-  const SgmvSplit sp = p.split[split_id];
-  const int K = p.K;
+  const int slice = blockIdx.y / ksplit, kpart = blockIdx.y % ksplit;
+  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
 
-  // Token row of this lane in each 16-token block (rows past the tile repeat its first row:
-  // they feed the MFMA harmlessly and are never written back).
+  const i32x4 td = reinterpret_cast<const i32x4*>(plan + tiles_off)[tile];  // in bounds for the whole grid
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
+  const int n_tiles = plan[MLORA_PLAN_TILES_LONG_BIG];
+  const int slot = td[0], start = td[1], m = td[2];
+  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
+                     int(slot < num_slots);
+  if (!usable) return;
+
+  const int k0 = kpart * krange;
+  const int nslab = krange / KR;
+  const bool active = wave * 16 < m;  // this wavefront's token block exists
+  // token row of this lane (lanes past the end of the tile repeat its last token: they feed the
+  // MFMA harmlessly and are never written back)
+  const int ti = wave * 16 + lr;
+  const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
+  const T* xptr = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + k0 + lg * 8;
+  const T* A = static_cast<const T*>(sl.a[slice]) + static_cast<int64_t>(slot) * R * K + k0;
+
+  f32x4 acc[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int slab = 0; slab < nslab; ++slab) {
+    const T* Aslab = A + slab * KR;
+    const T* xslab = xptr + slab * KR;
+    // the first batch of x loads goes out together with the slab copy
+    Pack8 xa[XB];
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < XB; ++i) xa[i].raw = load128(xslab + i * 32);
+    }
+    if (slab > 0) __syncthreads();  // everyone is done reading the previous slab
+#pragma unroll
+    for (int c0 = 0; c0 < CHUNKS; c0 += SB) {
+      i32x4 v[SB];
+#pragma unroll
+      for (int i = 0; i < SB; ++i) {
+        const int c = (c0 + i) * NT + tid;
+        if (TOTAL % NT == 0 || c < TOTAL) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < SB; ++i) {
+        const int c = (c0 + i) * NT + tid;
+        if (TOTAL % NT == 0 || c < TOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
+      }
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int kb = 0; kb < KS; kb += XB) {
+        if (kb > 0) {
+#pragma unroll
+          for (int i = 0; i < XB; ++i) xa[i].raw = load128(xslab + (kb + i) * 32);
+        }
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            const int rr = rb * 16 + lr;
+            Pack8 aw;
+            aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + (kb + i) * 32 + lg * 8]);
+            acc[rb] = Mma<T>::run(aw, xa[i], acc[rb]);
+          }
+        }
+      }
+    }
+  }
+
+  // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
+  if (active && ti < m) {
+    float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice) * R;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int r0 = rb * 16 + 4 * lg;
+      if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
+    }
+  }
+}
+
+// ---- expand -------------------------------------------------------------------------------------
+// grid (8, column ranges, tiles / 8), four wavefronts.
+template <typename T, int R>
+__global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
+                                                                          void* __restrict__ yv_, int64_t ys, int tiles_off,
+                                                                          int sorted_off, int T_, int num_slots, int num_slices,
+                                                                          int ksplit, float scaling, ExpandSplits splits) {
+  constexpr int TB = MLORA_TILE_BIG / 16;
+  constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps
+  constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
+  constexpr int NT = kExpandWaves * kWave;
+  constexpr int CPR = R / 8;             // groups of eight ranks per token
+
+  __shared__ __attribute__((aligned(16))) T s_h[MLORA_TILE_BIG * HSTRIDE];
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+
+  const i32x4 td = reinterpret_cast<const i32x4*>(plan + tiles_off)[tile];
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
+  const int n_tiles = plan[MLORA_PLAN_TILES_LONG_BIG];
+  const ExpandSplit sp = splits.split[blockIdx.y];
+  const int slot = td[0], start = td[1], m = td[2];
+  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
+                     int(slot < num_slots) & int(sp.n0 < sp.n1);
+  if (!usable) return;
+
+  // token rows first: the y loads below wait on them
+  const int32_t* sorted = plan + sorted_off + start;
   int row[TB];
 #pragma unroll
   for (int tb = 0; tb < TB; ++tb) {
     const int ti = tb * 16 + lr;
-    row[tb] = sorted[ti < m ? ti : 0];
+    row[tb] = sorted[ti < m ? ti : m - 1];
   }
 
-  // ---- shrink ---------------------------------------------------------------------------
+  // H tile -> LDS: sum the K partials, scale, split into leading part and remainder (absent
+  // tokens get zeros)
   {
-    const T* x = static_cast<const T*>(p.x);
-    const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
-    const T* xptr[TB];
-    const T* aptr[RB];
-#pragma unroll
-    for (int tb = 0; tb < TB; ++tb) xptr[tb] = x + static_cast<int64_t>(row[tb]) * p.xs + lg * 8;
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const int rr = rb * 16 + lr;
-      aptr[rb] = A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + lg * 8;
-    }
-    f32x4 acc[TB][RB];
-#pragma unroll
-    for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[tb][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    const int nks = K / 32;
-    const int ks0 = wave * nks / kWaves, ks1 = (wave + 1) * nks / kWaves;
-    for (int ks = ks0; ks < ks1; ++ks) {
-      Pack8 xa[TB], aw[RB];
-#pragma unroll
-      for (int tb = 0; tb < TB; ++tb)
-        if (tb * 16 < m) xa[tb].raw = load128(xptr[tb] + ks * 32);
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) aw[rb].raw = load128(aptr[rb] + ks * 32);
-#pragma unroll
-      for (int tb = 0; tb < TB; ++tb)
-        if (tb * 16 < m) {
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb) acc[tb][rb] = Mma<T>::run(xa[tb], aw[rb], acc[tb][rb]);
+    const int64_t hrow = static_cast<int64_t>(num_slices) * R;
+    const int64_t part = static_cast<int64_t>(T_) * hrow;
+    const float* src = hws + static_cast<int64_t>(start) * hrow + sp.slice * R;
+    for (int c = tid; c < MLORA_TILE_BIG * CPR; c += NT) {
+      const int tok = c / CPR, ch = c % CPR;
+      Pack8 hi, lo;
+      hi.raw = i32x4{0, 0, 0, 0};
+      lo.raw = i32x4{0, 0, 0, 0};
+      if (tok < m) {
+        const float* q = src + tok * hrow + ch * 8;
+        f32x4 s0 = *reinterpret_cast<const f32x4*>(q), s1 = *reinterpret_cast<const f32x4*>(q + 4);
+        for (int kp = 1; kp < ksplit; ++kp) {
+          const f32x4 t0 = *reinterpret_cast<const f32x4*>(q + kp * part), t1 = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+          s0[0] += t0[0]; s0[1] += t0[1]; s0[2] += t0[2]; s0[3] += t0[3];
+          s1[0] += t1[0]; s1[1] += t1[1]; s1[2] += t1[2]; s1[3] += t1[3];
         }
-    }
-
-    // Sum the four K-partials one 16-token block at a time and keep the result in LDS at the
-    // operand precision.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
+        float v[8], rem[8];
 #pragma unroll
-    for (int tb = 0; tb < TB; ++tb) {
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
-        *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[tb][rb];
-      __syncthreads();
-      const int ln = tid >> 2, i = tid & 3;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-        const int tok = tb * 16 + 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-        if (r < R) {
-          const float v = sum * p.scaling;
-          const T hi = from_f32<T>(v);
-          s_hb[tok * HSTRIDE + r] = hi;
-          s_hl[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+        for (int i = 0; i < 4; ++i) {
+          v[i] = s0[i] * scaling;
+          v[4 + i] = s1[i] * scaling;
         }
+        pack8<T>(v, hi);
+        float back[8];
+        unpack8<T>(hi, back);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
+        pack8<T>(rem, lo);
       }
-      __syncthreads();
+      *reinterpret_cast<i32x4*>(&s_h[tok * HSTRIDE + ch * 8]) = hi.raw;
+      *reinterpret_cast<i32x4*>(&s_h[tok * HSTRIDE + R + ch * 8]) = lo.raw;
     }
   }
-
-  // ---- expand ---------------------------------------------------------------------------
-  Pack8 hop[TB][KSTEPS], hlo[TB][KSTEPS];
-#pragma unroll
-  for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int kc = lg + 4 * ks;
-      if (kc * 8 < R) {
-        hop[tb][ks].raw = load128(&s_hb[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-        hlo[tb][ks].raw = load128(&s_hl[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-      } else {
-        hop[tb][ks].raw = i32x4{0, 0, 0, 0};
-        hlo[tb][ks].raw = i32x4{0, 0, 0, 0};
-      }
-    }
 
   const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
-  T* y = static_cast<T*>(p.y) + sp.y_col;
-  for (int c0 = sp.n0 + wave * 64; c0 < sp.n1; c0 += kWaves * 64) {
-    Pack8 bop[4][KSTEPS];
+  T* ybase = static_cast<T*>(yv_) + sp.y_col;
+  const T* ysrc[TB];
+#pragma unroll
+  for (int tb = 0; tb < TB; ++tb) ysrc[tb] = ybase + static_cast<int64_t>(row[tb]) * ys;
+  __syncthreads();
+
+  for (int c0 = sp.n0 + wave * 64; c0 < sp.n1; c0 += kExpandWaves * 64) {
+    // every load of the span is issued here: B rows (lanes whose chunk lies beyond the rank fetch
+    // a valid chunk anyway, their H operand is zero) and the y rows of all token blocks (absent
+    // tokens and columns past the range read a valid address and are never stored)
+    Pack8 bop[4][KSTEPS], yreg[TB][2];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
       n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = lg + 4 * ks;
-        if (kc * 8 < R) bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-        else bop[j][ks].raw = i32x4{0, 0, 0, 0};
+        const int kc = (lg + 4 * ks) & (R / 8 - 1);
+        bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
       }
     }
+    int col[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int c = c0 + 16 * lg + 8 * half;
+      col[half] = c < sp.n1 ? c : sp.n1 - 8;
+    }
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) yreg[tb][half].raw = load128(ysrc[tb] + col[half]);
+
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) {
       if (tb * 16 >= m) continue;
-      f32x4 acc[4];
+      Pack8 hop[KSTEPS], hlo[KSTEPS];
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = lg + 4 * ks;
+        if (kc * 8 < R) {
+          hop[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+          hlo[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
+        } else {
+          hop[ks].raw = i32x4{0, 0, 0, 0};
+          hlo[ks].raw = i32x4{0, 0, 0, 0};
+        }
+      }
+      f32x4 out[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          acc[j] = Mma<T>::run(bop[j][ks], hlo[tb][ks], acc[j]);
-          acc[j] = Mma<T>::run(bop[j][ks], hop[tb][ks], acc[j]);
+          out[j] = Mma<T>::run(bop[j][ks], hlo[ks], out[j]);
+          out[j] = Mma<T>::run(bop[j][ks], hop[ks], out[j]);
         }
       }
       if (tb * 16 + lr < m) {
-        T* yp = y + static_cast<int64_t>(row[tb]) * p.ys + c0 + 16 * lg;
+        T* yp = const_cast<T*>(ysrc[tb]);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           if (c0 + 16 * lg + 8 * half < sp.n1) {
-            Pack8 yv;
-            yv.raw = load128(yp + 8 * half);
             float yf[8];
-            unpack8<T>(yv, yf);
+            unpack8<T>(yreg[tb][half], yf);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              yf[i] += acc[2 * half][i];
-              yf[4 + i] += acc[2 * half + 1][i];
+              yf[i] += out[2 * half][i];
+              yf[4 + i] += out[2 * half + 1][i];
             }
-            pack8<T>(yf, yv);
-            store128(yp + 8 * half, yv.raw);
+            Pack8 r;
+            pack8<T>(yf, r);
+            store128(yp + col[half], r.raw);
           }
         }
       }
@@ -219,18 +321,61 @@ __global__ __launch_bounds__(kThreads) void sgmv_kernel(SgmvParams p) {
   }
 }
 
-template <typename T, int MTB>
-void launch_rank(const SgmvParams& p, int r, dim3 grid, hipStream_t st) {
-  switch (r) {
-    case 8: hipLaunchKernelGGL((sgmv_kernel<T, 8, MTB>), grid, dim3(kThreads), 0, st, p); break;
-    case 16: hipLaunchKernelGGL((sgmv_kernel<T, 16, MTB>), grid, dim3(kThreads), 0, st, p); break;
-    case 32: hipLaunchKernelGGL((sgmv_kernel<T, 32, MTB>), grid, dim3(kThreads), 0, st, p); break;
-    default: hipLaunchKernelGGL((sgmv_kernel<T, 64, MTB>), grid, dim3(kThreads), 0, st, p); break;
+struct ShrinkLaunch {
+  const MloraAddArgs* a;
+  PlanLayout lay;
+  ShrinkSlices sl;
+  int tiles8;  // tile capacity / 8
+  int ksplit, krange;
+};
+
+template <typename T, int R, int KR>
+void launch_shrink_one(const ShrinkLaunch& l) {
+  const MloraAddArgs* a = l.a;
+  dim3 grid(8, static_cast<unsigned>(a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
+  hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
+                     a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.sorted_off,
+                     a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.sl);
+}
+
+template <typename T, int R>
+void launch_shrink_slab(const ShrinkLaunch& l, int kr) {
+  switch (kr) {
+    case 128: launch_shrink_one<T, R, 128>(l); break;
+    case 256: launch_shrink_one<T, R, 256>(l); break;
+    case 512: launch_shrink_one<T, R, 512>(l); break;
+    default: launch_shrink_one<T, R, 1024>(l); break;
   }
 }
 
+template <typename T>
+void launch_shrink_rank(const ShrinkLaunch& l, int kr) {
+  switch (l.a->r) {
+    case 8: launch_shrink_slab<T, 8>(l, kr); break;
+    case 16: launch_shrink_slab<T, 16>(l, kr); break;
+    case 32: launch_shrink_slab<T, 32>(l, kr); break;
+    default: launch_shrink_slab<T, 64>(l, kr); break;
+  }
+}
+
+template <typename T>
+void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, dim3 grid, int ksplit, const ExpandSplits& sp) {
+  hipStream_t st = static_cast<hipStream_t>(a->stream);
+  const float* h = static_cast<const float*>(a->workspace);
+#define MLORA_EXPAND(RR)                                                                                                     \
+  hipLaunchKernelGGL((sgmv_expand_kernel<T, RR>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, a->y_stride,     \
+                     lay.big_off, lay.sorted_off, a->num_tokens, a->num_slots, a->num_slices, ksplit, a->scaling, sp)
+  switch (a->r) {
+    case 8: MLORA_EXPAND(8); break;
+    case 16: MLORA_EXPAND(16); break;
+    case 32: MLORA_EXPAND(32); break;
+    default: MLORA_EXPAND(64); break;
+  }
+#undef MLORA_EXPAND
+}
+
 // Column ranges of about `nt` columns (a multiple of 256: four wavefronts of 64 columns).
-int fill_splits(const MloraAddArgs* a, int nt, SgmvSplit* out) {
+int fill_splits(const MloraAddArgs* a, int nt, ExpandSplit* out) {
   nt = (nt + 255) & ~255;
   if (nt < 256) nt = 256;
   int total;
@@ -244,8 +389,8 @@ int fill_splits(const MloraAddArgs* a, int nt, SgmvSplit* out) {
   for (int i = 0; i < a->num_slices; ++i) {
     const MloraSlice& sl = a->slices[i];
     for (int n0 = 0; n0 < sl.n; n0 += nt) {
-      SgmvSplit& sp = out[s++];
-      sp.a = sl.a; sp.b = sl.b; sp.n = sl.n; sp.y_col = sl.y_col;
+      ExpandSplit& sp = out[s++];
+      sp.b = sl.b; sp.n = sl.n; sp.y_col = sl.y_col; sp.slice = i; sp.pad = 0;
       sp.n0 = n0; sp.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
     }
   }
@@ -254,36 +399,82 @@ int fill_splits(const MloraAddArgs* a, int nt, SgmvSplit* out) {
 
 }  // namespace
 
-bool sgmv_supported(const MloraAddArgs* a) { return a->k % 32 == 0 && a->k >= 32; }
+// One fp32 partial of the intermediate: [T, slices, r].
+static size_t partial_bytes(int num_tokens, int num_slices, int r) {
+  return static_cast<size_t>(num_tokens) * static_cast<size_t>(num_slices) * static_cast<size_t>(r) * sizeof(float);
+}
+
+// Room for the most K parts the shrink ever uses.
+constexpr int kMaxKSplit = 4;
+
+size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype) {
+  (void)dtype;
+  if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
+  return kMaxKSplit * partial_bytes(num_tokens, num_slices, r);
+}
+
+bool sgmv_supported(const MloraAddArgs* a) { return a->k % 128 == 0 && a->k >= 128; }
+
+// A workspace that holds at least one partial can be used (fewer K parts are taken then).
+bool sgmv_workspace_ok(const MloraAddArgs* a) {
+  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 15)) return false;
+  for (int i = 0; i < a->num_slices; ++i)
+    if (a->slices[i].n <= 0) return false;  // every slice owns a workspace column block
+  return a->workspace_bytes > 0 && static_cast<size_t>(a->workspace_bytes) >= partial_bytes(a->num_tokens, a->num_slices, a->r);
+}
 
 // 64-token tiles of the segments at or above the threshold.
 int launch_sgmv(const MloraAddArgs* a) {
-  SgmvParams p;
-  p.x = a->x; p.y = a->y; p.xs = a->x_stride; p.ys = a->y_stride; p.plan = a->plan;
-  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  p.sorted_off = lay.sorted_off;
-  p.T = a->num_tokens; p.K = a->k; p.num_slots = a->num_slots; p.scaling = a->scaling;
-  p.tiles_off = lay.big_off; p.count_word = MLORA_PLAN_TILES_LONG_BIG;
-  int cap = lay.cap_big;
+  ShrinkLaunch l;
+  l.a = a;
+  l.lay = plan_layout(a->num_tokens, a->num_slots);
+  int cap = l.lay.cap_big;
   if (cap == 0) return 0;
+  cap = (cap + 7) & ~7;
+  l.tiles8 = cap / 8;
   int cols = 0;
-  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+  for (int i = 0; i < a->num_slices; ++i) {
+    cols += a->slices[i].n;
+    l.sl.a[i] = a->slices[i].a;
+  }
+  for (int i = a->num_slices; i < MLORA_MAX_SLICES; ++i) l.sl.a[i] = nullptr;
   if (cols == 0) return 0;
-  // Aim for a few workgroups per CU: tiles x column ranges of about 1024 workgroups.
-  const int target = env_int("MLORA_SGMV_WGS", 1024);
   const int est_tiles = a->num_tokens / MLORA_TILE_BIG + 1;
+
+  // shrink: LDS slab width (the A slab of r rows has to fit next to nothing else), then K parts
+  // so that the grid has a few workgroups per compute unit
+  int kr = env_int("MLORA_SGMV_KR", 0);
+  if (kr != 128 && kr != 256 && kr != 512 && kr != 1024) kr = 512;
+  while (kr > 128 && (a->k % kr != 0)) kr /= 2;
+  const int max_parts = static_cast<int>(static_cast<size_t>(a->workspace_bytes) / partial_bytes(a->num_tokens, a->num_slices, a->r));
+  int ksplit = env_int("MLORA_SGMV_KSPLIT", 0);
+  if (ksplit <= 0) {
+    ksplit = 1;
+    while (ksplit < kMaxKSplit && static_cast<long long>(est_tiles) * a->num_slices * ksplit < 512 && a->k % (kr * ksplit * 2) == 0) ksplit *= 2;
+  }
+  if (ksplit > max_parts) ksplit = max_parts;
+  if (ksplit > kMaxKSplit) ksplit = kMaxKSplit;
+  while (ksplit > 1 && a->k % (kr * ksplit) != 0) --ksplit;
+  l.ksplit = ksplit;
+  l.krange = a->k / ksplit;
+  if (a->dtype == MLORA_DTYPE_BF16) launch_shrink_rank<__bf16>(l, kr);
+  else launch_shrink_rank<_Float16>(l, kr);
+  int rc = check_launch("mlora_add_lora(sgmv shrink)");
+  if (rc) return rc;
+
+  // expand: tiles x column ranges of about 2048 workgroups
+  ExpandSplits splits;
+  const int target = env_int("MLORA_SGMV_WGS", 2048);
   int nt = env_int("MLORA_SGMV_NT", 0);
   if (nt <= 0) {
     const long long want = static_cast<long long>(cols) * est_tiles / (target > 0 ? target : 1);
     nt = want > 8192 ? 8192 : static_cast<int>(want);
   }
-  p.nsplit = fill_splits(a, nt, p.split);
-  cap = (cap + 7) & ~7;
-  dim3 grid(8, static_cast<unsigned>(p.nsplit), static_cast<unsigned>(cap / 8));
-  hipStream_t st = static_cast<hipStream_t>(a->stream);
-  if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16, MLORA_TILE_BIG>(p, a->r, grid, st);
-  else launch_rank<_Float16, MLORA_TILE_BIG>(p, a->r, grid, st);
-  return check_launch("mlora_add_lora(mfma, big tiles)");
+  const int nsplit = fill_splits(a, nt, splits.split);
+  dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(l.tiles8));
+  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, grid, ksplit, splits);
+  else launch_expand_rank<_Float16>(a, l.lay, grid, ksplit, splits);
+  return check_launch("mlora_add_lora(sgmv expand)");
 }
 
 }  // namespace mlora

@@ -46,6 +46,7 @@ _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: D
 
 EXPORTS = (
     "mlora_add_lora",
+    "mlora_add_workspace_bytes",
     "mlora_shrink",
     "mlora_expand",
     "mlora_plan_workspace_bytes",
@@ -80,6 +81,8 @@ class MloraAddArgs(C.Structure):
         ("form", C.c_int32),
         ("scaling", C.c_float),
         ("slices", MloraSlice * MAX_SLICES),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_int64),
     ]
 
 
@@ -203,6 +206,8 @@ def load() -> C.CDLL:
         fn.restype = C.c_int
     lib.mlora_plan_workspace_bytes.argtypes = [C.c_int32, C.c_int32]
     lib.mlora_plan_workspace_bytes.restype = C.c_size_t
+    lib.mlora_add_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.mlora_add_workspace_bytes.restype = C.c_size_t
     lib.mlora_stream_capture_id.argtypes = [C.c_void_p]
     lib.mlora_stream_capture_id.restype = C.c_uint64
     lib.mlora_abi_version.argtypes = []
@@ -250,6 +255,11 @@ def plan_workspace_words(num_tokens: int, max_slots: int) -> int:
     return (load().mlora_plan_workspace_bytes(num_tokens, max_slots) + 3) // 4
 
 
+def add_workspace_bytes(num_tokens: int, num_slices: int, r: int, dtype: torch.dtype) -> int:
+    """Bytes of scratch that let the fused apply use the two-launch form for long segments."""
+    return int(load().mlora_add_workspace_bytes(num_tokens, num_slices, r, dtype_code(dtype)))
+
+
 def add_lora(
     y: torch.Tensor,
     x: torch.Tensor,
@@ -260,6 +270,7 @@ def add_lora(
     plan: torch.Tensor | None,
     scaling: float,
     form: int = FORM_AUTO,
+    workspace: torch.Tensor | None = None,
 ) -> None:
     """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice."""
     lib = load()
@@ -288,6 +299,9 @@ def add_lora(
         s.b = b.data_ptr()
         s.n = b.size(1)
         s.y_col = col
+    if workspace is not None:
+        args.workspace = workspace.data_ptr()
+        args.workspace_bytes = workspace.numel() * workspace.element_size()
     _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
 
 

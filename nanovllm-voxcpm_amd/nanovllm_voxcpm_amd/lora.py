@@ -96,6 +96,14 @@ _VECTOR_RANKS = (8, 16, 32, 64)
 _PLAN_ATTR = "_mlora_segment_plans"
 
 
+def _small_batch_tokens() -> int:
+    """Batch size up to which the library keeps to its one-launch small-tile form."""
+    try:
+        return int(os.environ.get("MLORA_SMALL_BATCH_TOKENS", "1024"))
+    except ValueError:
+        return 1024
+
+
 class HipLoRABackend:
     """``LoRABackend`` whose arithmetic runs in the hand-written gfx950 kernels."""
 
@@ -251,11 +259,16 @@ class HipLoRABackend:
                 a_list = [lora_a_slices[i] for i in chunk]
                 b_list = [lora_b_slices[i] for i in chunk]
                 c_list = [cols[i] for i in chunk]
-                plan = None
+                plan = scratch = None
                 form = _hip.FORMS[self.form]
                 if form != _hip.FORM_TOKEN and self._vectorisable(x2, target, a_list, b_list, c_list):
                     plan = self._plan_for(metadata, tts, a_list[0].size(0)).workspace
-                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form)
+                    if form == _hip.FORM_SGMV or (form == _hip.FORM_AUTO and x2.size(0) > _small_batch_tokens()):
+                        # scratch for the rank-r intermediate between the two launches of the
+                        # long-segment form (the caching allocator makes this a pointer bump)
+                        nbytes = _hip.add_workspace_bytes(x2.size(0), len(chunk), a_list[0].size(-2), x2.dtype)
+                        scratch = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch)
         if staged is not None:
             staged.copy_(target)
         return outputs
