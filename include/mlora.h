@@ -73,8 +73,9 @@ typedef struct MloraAddArgs {
   int64_t x_stride;
   int64_t y_stride;
   const int32_t* token_to_slot; /* [T] on device */
-  const int32_t* plan;    /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
-                             (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it) */
+  int32_t* plan;          /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
+                             (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it).  Read-only
+                             for the caller; launches keep transient arrival counters in it */
   int32_t num_tokens;     /* T */
   int32_t k;              /* K, input features */
   int32_t r;              /* rank dimension of the A/B buffers (max_lora_rank) */
@@ -84,8 +85,10 @@ typedef struct MloraAddArgs {
   int32_t form;           /* MLORA_FORM_* */
   float scaling;
   MloraSlice slices[MLORA_MAX_SLICES];
-  void* workspace;        /* device scratch for the rank-r intermediate of MLORA_FORM_SGMV, 16-byte
-                             aligned, or NULL (AUTO then keeps to the small-tile form).  Counterpart of
+  void* workspace;        /* device scratch for the rank-r intermediate: between the two launches of
+                             MLORA_FORM_SGMV, and between workgroups that share one shrink in the
+                             small-tile form; 16-byte aligned, or NULL (AUTO then keeps to the
+                             small-tile form, one workgroup per shrink).  Counterpart of
                              the [S, T, r] buffer the reference allocates between its two kernels
                              (reference: nanovllm_voxcpm/lora.py:299-381).  Contents need not be kept
                              between calls; calls that share it must be ordered on one stream. */
@@ -94,7 +97,8 @@ typedef struct MloraAddArgs {
 
 int mlora_add_lora(const MloraAddArgs* args);
 
-/* Bytes of MloraAddArgs.workspace that let mlora_add_lora use MLORA_FORM_SGMV. */
+/* Bytes of MloraAddArgs.workspace that let mlora_add_lora use every form it has for this shape
+ * (a smaller workspace is legal: the library then splits K less, or not at all). */
 size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);
 
 /* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0
@@ -169,6 +173,10 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
 #define MLORA_BIG_TILE_WORDS 4
+/* Behind the tile lists the plan holds MLORA_COOP_SPLITS int32 counters per small tile: when
+ * several workgroups share the shrink of one tile they count their arrivals there.  They are
+ * zero whenever no launch is in flight, so calls that share a plan must be ordered on one stream. */
+#define MLORA_COOP_SPLITS 8
 
 /* Arguments of the on-device metadata build: a stable counting sort of the tokens by
  * slot id.  The plan workspace (always written when non-NULL) feeds mlora_add_lora; the

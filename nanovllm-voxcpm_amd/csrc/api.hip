@@ -113,8 +113,6 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
                   sgmv_workspace_bytes(a->num_tokens, a->num_slices, a->r, a->dtype));
         return MLORA_E_INVALID;
       }
-      int rc = launch_decode(a, /*include_long=*/false);
-      if (rc) return rc;
       return launch_sgmv(a);
     }
   }
@@ -123,7 +121,9 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
 }
 
 extern "C" size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype) {
-  return sgmv_workspace_bytes(num_tokens, num_slices, r, dtype);
+  if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
+  const size_t big = sgmv_workspace_bytes(num_tokens, num_slices, r, dtype), small = decode_workspace_bytes(r);
+  return big > small ? big : small;
 }
 
 extern "C" uint64_t mlora_stream_capture_id(void* stream) {

@@ -86,7 +86,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles
 // Small tiles are 32-word records (128-byte aligned), big tiles four words; see mlora.h.
 struct PlanLayout {
-  int sorted_off, counts_off, offsets_off, small_off, big_off, cap_small, cap_big, total_words;
+  int sorted_off, counts_off, offsets_off, small_off, big_off, coop_off, cap_small, cap_big, total_words;
 };
 
 __host__ __device__ inline int round_up4(int v) { return (v + 3) & ~3; }
@@ -98,10 +98,14 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   p.counts_off = p.sorted_off + round_up4(T);
   p.offsets_off = p.counts_off + round_up4(L + 1);
   p.small_off = (p.offsets_off + round_up4(L + 2) + 31) & ~31;
-  p.cap_small = (T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs;
+  // capacities are multiples of eight: launches walk the tile lists in groups of eight (one
+  // tile per XCD), and every record such a grid may touch has to exist
+  p.cap_small = ((T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs + 7) & ~7;
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
-  p.cap_big = T / MLORA_TILE_BIG + segs;
-  p.total_words = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
+  p.cap_big = (T / MLORA_TILE_BIG + segs + 7) & ~7;
+  // arrival counters of the workgroups that share one small tile's shrink (zero between launches)
+  p.coop_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
+  p.total_words = p.coop_off + MLORA_COOP_SPLITS * p.cap_small;
   return p;
 }
 

@@ -51,11 +51,19 @@ struct DecodeSplits {
 };
 
 // KSPW: k-steps (32 elements of K) each wavefront covers when that is known at compile time
-// (K = 32 * kNW * KSPW), 0 when it has to be worked out from K at run time.
+// (K = 32 * kNW * KSPW << kshift), 0 when it has to be worked out from K at run time.
+//
+// A compute unit fills its caches from cold memory far more slowly than the chip as a whole
+// can deliver, so when K is large and the grid small, 1 << kshift workgroups share the shrink
+// of a (tile, column range): each covers one part of K, leaves its partial sums in `partials`
+// and counts its arrival in `counters`; the last to arrive adds the parts up in a fixed order
+// (the result does not depend on who is last) and does the expand.  Nobody waits: the others
+// simply exit.  The counter is back at zero when the launch ends.
 template <typename T, int R, int KSPW>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
+                                                            int kshift, int32_t* __restrict__ counters, float* __restrict__ partials,
                                                             DecodeSplits splits) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
@@ -66,6 +74,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
   __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
   __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
+  __shared__ int s_arrived;
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
@@ -73,7 +82,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first and
   // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD: the column ranges of one
   // tile share an XCD and its L2.
-  const int split_id = blockIdx.y;
+  const int split_id = blockIdx.y >> kshift, kpart = blockIdx.y & ((1 << kshift) - 1);
   const int tile = blockIdx.z * 8 + blockIdx.x;
 
   // ---- round trip 1 ---------------------------------------------------------------------------
@@ -108,9 +117,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   T* yrow = static_cast<T*>(yv_) + static_cast<int64_t>(row) * ys + sp.y_col + 16 * lg;
 
   // ---- round trip 2: issue every load ---------------------------------------------------------
-  const int nks = K / 32;
-  const int ks0 = KSPW > 0 ? wave * KSPW : wave * nks / kNW;
-  const int ks1 = KSPW > 0 ? ks0 + KSPW : (wave + 1) * nks / kNW;
+  const int nks = (K / 32) >> kshift;  // k-steps of this workgroup's part of K
+  const int ks0 = kpart * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
+  const int ks1 = KSPW > 0 ? ks0 + KSPW : kpart * nks + (wave + 1) * nks / kNW;
   Pack8 xa[CH], aw[RB][CH];
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
@@ -180,13 +189,51 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
   __syncthreads();
-  for (int e = tid; e < RB * 256; e += NT) {
-    const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-    float sum = 0.f;
+  if (kshift == 0) {
+    for (int e = tid; e < RB * 256; e += NT) {
+      const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+      float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-    const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-    if (r < R) {
+      for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+      const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+      if (r < R) {
+        const float v = sum * scaling;
+        const T hi = from_f32<T>(v);
+        s_hi[tok * HSTRIDE + r] = hi;
+        s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+      }
+    }
+  } else {
+    // This part's sums -> memory, then count the arrival.  Everything the workgroups exchange is
+    // written and read with device-scope atomic accesses, which are performed at the level of
+    // the memory system all compute units share, so no cache has to be flushed: a workgroup
+    // only waits for its own stores to be acknowledged before it is counted.
+    const int group = tile * gridDim.y + (split_id << kshift);  // first of the workgroups sharing this shrink
+    float* mine = partials + static_cast<int64_t>(group + kpart) * (16 * R);
+    for (int e = tid; e < RB * 256; e += NT) {
+      const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+      const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+      if (r < R) __hip_atomic_store(mine + tok * R + r, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      int32_t* ctr = counters + tile * MLORA_COOP_SPLITS + split_id;
+      const int before = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == (1 << kshift) - 1) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_arrived = before;
+    }
+    __syncthreads();
+    if (s_arrived != (1 << kshift) - 1) return;  // someone else finishes this tile
+    const float* parts = partials + static_cast<int64_t>(group) * (16 * R);
+    for (int e = tid; e < 16 * R; e += NT) {
+      float sum = 0.f;
+      for (int kp = 0; kp < (1 << kshift); ++kp)
+        sum += __hip_atomic_load(parts + kp * (16 * R) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int tok = e / R, r = e % R;
       const float v = sum * scaling;
       const T hi = from_f32<T>(v);
       s_hi[tok * HSTRIDE + r] = hi;
@@ -265,7 +312,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 
 struct Launch {
   const MloraAddArgs* a;
-  int small_off, include_long;
+  int small_off, include_long, kshift;
+  int32_t* counters;
   dim3 grid;
   const DecodeSplits* splits;
 };
@@ -275,7 +323,7 @@ void launch_one(const Launch& l) {
   const MloraAddArgs* a = l.a;
   hipLaunchKernelGGL((decode_kernel<T, R, KSPW>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
-                     a->num_slots, a->scaling, *l.splits);
+                     a->num_slots, a->scaling, l.kshift, l.counters, static_cast<float*>(a->workspace), *l.splits);
 }
 
 // The steps-per-wavefront specialisations kept: 4 (K = 1024) for every rank and 16 (K = 4096)
@@ -300,6 +348,10 @@ void launch_rank(const Launch& l, int r, int kspw) {
 }
 
 }  // namespace
+
+// Workspace that lets the small-tile form share a shrink between workgroups: it is only done
+// for grids of at most 128 (tile, column range) pairs, four parts each, 16 x r sums per part.
+size_t decode_workspace_bytes(int r) { return static_cast<size_t>(128) * 4 * 16 * r * sizeof(float); }
 
 int launch_decode(const MloraAddArgs* a, bool include_long) {
   DecodeSplits splits;
@@ -335,10 +387,29 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
   }
   if (cap == 0) return 0;
   cap = (cap + 7) & ~7;
+  // Workgroups sharing one shrink: only worth its extra round trip through memory when a
+  // workgroup would otherwise pull a long K through a single compute unit while most of the
+  // chip idles; needs room for the partial sums in the caller's workspace.
+  const int nks_all = a->k / 32;
+  int kshift = 0;
+  const int want = env_int("MLORA_DECODE_KPARTS", 0);
+  if (total <= MLORA_COOP_SPLITS && a->workspace && !(reinterpret_cast<uintptr_t>(a->workspace) & 15)) {
+    int parts = 1;
+    if (want > 0) parts = want;
+    else if (a->k >= 2048 && static_cast<long long>(cap) * total <= 128) parts = 4;
+    while (parts > 1) {
+      const size_t need = static_cast<size_t>(cap) * total * parts * 16 * a->r * sizeof(float);
+      if ((parts & (parts - 1)) == 0 && nks_all % (parts * kNW) == 0 && static_cast<size_t>(a->workspace_bytes) >= need) break;
+      parts /= 2;
+    }
+    while ((1 << kshift) < parts) ++kshift;
+  }
   Launch l;
   l.a = a; l.small_off = lay.small_off; l.include_long = include_long ? 1 : 0; l.splits = &splits;
-  l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>(cap / 8));
-  const int nks = a->k / 32;
+  l.kshift = kshift;
+  l.counters = a->plan + lay.coop_off;
+  l.grid = dim3(8, static_cast<unsigned>(total << kshift), static_cast<unsigned>(cap / 8));
+  const int nks = nks_all >> kshift;
   const int kspw = (nks % kNW == 0) ? nks / kNW : 0;
   if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16>(l, a->r, kspw);
   else launch_rank<_Float16>(l, a->r, kspw);

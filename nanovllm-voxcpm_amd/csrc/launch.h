@@ -16,6 +16,7 @@ int launch_bgmv(const MloraAddArgs* a, bool include_long);
 
 // decode.hip: the same small tiles with both products on the matrix cores.
 int launch_decode(const MloraAddArgs* a, bool include_long);
+size_t decode_workspace_bytes(int r);
 
 // sgmv.hip: 64-token MFMA tiles of the segments at or above the threshold, as a shrink launch
 // and an expand launch that meet in the caller's workspace.

@@ -219,6 +219,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       int left = c - j * MLORA_TILE_BIG;
       big[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
     }
+    for (int i = tid; i < MLORA_COOP_SPLITS * lay.cap_small; i += kMetaThreads) p.plan[lay.coop_off + i] = 0;
   }
   __syncthreads();
 

@@ -58,6 +58,36 @@ struct ExpandSplits {
   ExpandSplit split[kMaxSplits];
 };
 
+// A unit of work of either kernel: up to 64 tokens of one slot.  Workgroups below `big_cap` take
+// the 64-token tiles of the long segments; the ones above take the short segments (fewer than
+// sixteen tokens, one small-tile record each), so that one pair of launches covers the batch.
+struct TileRef {
+  int slot, start, m, ok;
+};
+
+__device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, int big_off, int small_off, int big_cap, int tile,
+                                              int T_, int num_slots) {
+  // both candidate records and the header are requested together (every address is in bounds
+  // for the whole grid); the choice between them costs no second round trip
+  const int sidx = tile >= big_cap ? tile - big_cap : 0;
+  const i32x4 big = reinterpret_cast<const i32x4*>(plan + big_off)[tile < big_cap ? tile : 0];
+  const i32x4 small = *reinterpret_cast<const i32x4*>(plan + small_off + sidx * MLORA_SMALL_TILE_WORDS);
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
+  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);
+  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);
+  const bool is_big = tile < big_cap;
+  TileRef t;
+  t.slot = is_big ? big[0] : small[0];
+  t.start = is_big ? big[1] : small[2];
+  t.m = is_big ? big[2] : small[1];
+  const int limit = is_big ? hdr2[MLORA_PLAN_TILES_LONG_BIG - 8] : hdr1[MLORA_PLAN_TILES_SHORT - 4];
+  const int index = is_big ? tile : sidx;
+  t.ok = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+         int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(index < limit) & int(t.m > 0) & int(t.slot >= 0) &
+         int(t.slot < num_slots);
+  return t;
+}
+
 // ---- shrink -------------------------------------------------------------------------------------
 // grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  KR: columns of
 // K per LDS slab (the workgroup's K part is a whole number of slabs).
@@ -65,9 +95,10 @@ constexpr int kShrinkWaves = 4;
 
 template <typename T, int R, int KR>
 __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
-                                                                          float* __restrict__ hws, int64_t xs, int tiles_off,
-                                                                          int sorted_off, int T_, int K, int num_slots, int num_slices,
-                                                                          int ksplit, int krange, ShrinkSlices sl) {
+                                                                          float* __restrict__ hws, int64_t xs, int big_off,
+                                                                          int small_off, int big_cap, int sorted_off, int T_, int K,
+                                                                          int num_slots, int num_slices, int ksplit, int krange,
+                                                                          ShrinkSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -86,14 +117,9 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
   const int slice = blockIdx.y / ksplit, kpart = blockIdx.y % ksplit;
   const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
 
-  const i32x4 td = reinterpret_cast<const i32x4*>(plan + tiles_off)[tile];  // in bounds for the whole grid
-  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
-  const int n_tiles = plan[MLORA_PLAN_TILES_LONG_BIG];
-  const int slot = td[0], start = td[1], m = td[2];
-  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
-                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
-                     int(slot < num_slots);
-  if (!usable) return;
+  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
+  if (!tr.ok) return;
+  const int slot = tr.slot, start = tr.start, m = tr.m;
 
   const int k0 = kpart * krange;
   const int nslab = krange / KR;
@@ -167,12 +193,19 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
 }
 
 // ---- expand -------------------------------------------------------------------------------------
-// grid (8, column ranges, tiles / 8), four wavefronts.
+// grid (8, column ranges, tiles / 8), four wavefronts.  OUT[tokens x cols] = H . B[slot]^T with
+// the tokens as MFMA rows: in the accumulator layout a lane then holds four tokens of one column,
+// and with the B rows of the eight MFMAs of a 128-column span interleaved (MFMA j takes column
+// 8 * (lane % 16) + j) it holds eight consecutive columns of each of those tokens.  Sixteen
+// consecutive lanes therefore cover 256 contiguous bytes of one y row: y is read and written in
+// fully coalesced 128-bit accesses.
+constexpr int kSpan = 128;
+
 template <typename T, int R>
 __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
-                                                                          void* __restrict__ yv_, int64_t ys, int tiles_off,
-                                                                          int sorted_off, int T_, int num_slots, int num_slices,
-                                                                          int ksplit, float scaling, ExpandSplits splits) {
+                                                                          void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
+                                                                          int big_cap, int sorted_off, int T_, int num_slots,
+                                                                          int num_slices, int ksplit, float scaling, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps
   constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
@@ -180,29 +213,20 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
   constexpr int CPR = R / 8;             // groups of eight ranks per token
 
   __shared__ __attribute__((aligned(16))) T s_h[MLORA_TILE_BIG * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) int s_row[MLORA_TILE_BIG];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
   const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
 
-  const i32x4 td = reinterpret_cast<const i32x4*>(plan + tiles_off)[tile];
-  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
-  const int n_tiles = plan[MLORA_PLAN_TILES_LONG_BIG];
+  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
   const ExpandSplit sp = splits.split[blockIdx.y];
-  const int slot = td[0], start = td[1], m = td[2];
-  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
-                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
-                     int(slot < num_slots) & int(sp.n0 < sp.n1);
-  if (!usable) return;
+  if (!(tr.ok & int(sp.n0 < sp.n1))) return;
+  const int slot = tr.slot, start = tr.start, m = tr.m;
 
-  // token rows first: the y loads below wait on them
-  const int32_t* sorted = plan + sorted_off + start;
-  int row[TB];
-#pragma unroll
-  for (int tb = 0; tb < TB; ++tb) {
-    const int ti = tb * 16 + lr;
-    row[tb] = sorted[ti < m ? ti : m - 1];
-  }
+  // token rows of the tile (entries past its end repeat the last token: a valid row to read,
+  // never written)
+  if (tid < MLORA_TILE_BIG) s_row[tid] = plan[sorted_off + start + (tid < m ? tid : m - 1)];
 
   // H tile -> LDS: sum the K partials, scale, split into leading part and remainder (absent
   // tokens get zeros)
@@ -240,22 +264,26 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
       *reinterpret_cast<i32x4*>(&s_h[tok * HSTRIDE + R + ch * 8]) = lo.raw;
     }
   }
+  __syncthreads();
 
   const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
   T* ybase = static_cast<T*>(yv_) + sp.y_col;
-  const T* ysrc[TB];
+  // rows of this lane's four tokens in every token block
+  const T* yrow[TB][4];
 #pragma unroll
-  for (int tb = 0; tb < TB; ++tb) ysrc[tb] = ybase + static_cast<int64_t>(row[tb]) * ys;
-  __syncthreads();
+  for (int tb = 0; tb < TB; ++tb) {
+    const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[tb * 16 + 4 * lg]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) yrow[tb][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
+  }
 
-  for (int c0 = sp.n0 + wave * 64; c0 < sp.n1; c0 += kExpandWaves * 64) {
-    // every load of the span is issued here: B rows (lanes whose chunk lies beyond the rank fetch
-    // a valid chunk anyway, their H operand is zero) and the y rows of all token blocks (absent
-    // tokens and columns past the range read a valid address and are never stored)
-    Pack8 bop[4][KSTEPS], yreg[TB][2];
+  for (int c0 = sp.n0 + wave * kSpan; c0 < sp.n1; c0 += kExpandWaves * kSpan) {
+    // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
+    // their H operand is zero; columns past the range repeat the last one and are never stored)
+    Pack8 bop[8][KSTEPS];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
+    for (int j = 0; j < 8; ++j) {
+      int n = c0 + 8 * lr + j;
       n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -263,57 +291,55 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
         bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
       }
     }
-    int col[2];
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int c = c0 + 16 * lg + 8 * half;
-      col[half] = c < sp.n1 ? c : sp.n1 - 8;
-    }
-#pragma unroll
-    for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-      for (int half = 0; half < 2; ++half) yreg[tb][half].raw = load128(ysrc[tb] + col[half]);
+    const int c = c0 + 8 * lr;
+    const bool col_ok = c < sp.n1;
+    const int cl = col_ok ? c : sp.n1 - 8;
 
 #pragma unroll
-    for (int tb = 0; tb < TB; ++tb) {
-      if (tb * 16 >= m) continue;
-      Pack8 hop[KSTEPS], hlo[KSTEPS];
+    for (int tp = 0; tp < TB; tp += 2) {  // two token blocks at a time: their y rows are in flight together
+      if (tp * 16 >= m) continue;
+      Pack8 yreg[2][4];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = lg + 4 * ks;
-        if (kc * 8 < R) {
-          hop[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-          hlo[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
-        } else {
-          hop[ks].raw = i32x4{0, 0, 0, 0};
-          hlo[ks].raw = i32x4{0, 0, 0, 0};
-        }
-      }
-      f32x4 out[4];
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < 4; ++i) yreg[u][i].raw = load128(yrow[tp + u][i] + cl);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int tb = tp + u;
+        if (tb * 16 >= m) continue;
+        Pack8 hop[KSTEPS], hlo[KSTEPS];
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          out[j] = Mma<T>::run(bop[j][ks], hlo[ks], out[j]);
-          out[j] = Mma<T>::run(bop[j][ks], hop[ks], out[j]);
+          const int kc = lg + 4 * ks;
+          if (kc * 8 < R) {
+            hop[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+            hlo[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
+          } else {
+            hop[ks].raw = i32x4{0, 0, 0, 0};
+            hlo[ks].raw = i32x4{0, 0, 0, 0};
+          }
         }
-      }
-      if (tb * 16 + lr < m) {
-        T* yp = const_cast<T*>(ysrc[tb]);
+        f32x4 out[8];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          if (c0 + 16 * lg + 8 * half < sp.n1) {
+        for (int j = 0; j < 8; ++j) {
+          out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
+            out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
+          }
+        }
+        // lane holds out[token 16*tb + 4*lg + i][column c0 + 8*lr + j]
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (col_ok && tb * 16 + 4 * lg + i < m) {
             float yf[8];
-            unpack8<T>(yreg[tb][half], yf);
+            unpack8<T>(yreg[u][i], yf);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              yf[i] += out[2 * half][i];
-              yf[4 + i] += out[2 * half + 1][i];
-            }
+            for (int j = 0; j < 8; ++j) yf[j] += out[j][i];
             Pack8 r;
             pack8<T>(yf, r);
-            store128(yp + col[half], r.raw);
+            store128(const_cast<T*>(yrow[tb][i]) + c, r.raw);
           }
         }
       }
@@ -325,7 +351,8 @@ struct ShrinkLaunch {
   const MloraAddArgs* a;
   PlanLayout lay;
   ShrinkSlices sl;
-  int tiles8;  // tile capacity / 8
+  int tiles8;   // grid extent over tiles / 8
+  int big_cap;  // workgroups below this index take 64-token tiles, the rest short segments
   int ksplit, krange;
 };
 
@@ -334,8 +361,8 @@ void launch_shrink_one(const ShrinkLaunch& l) {
   const MloraAddArgs* a = l.a;
   dim3 grid(8, static_cast<unsigned>(a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
   hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
-                     a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.sorted_off,
-                     a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.sl);
+                     a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
+                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.sl);
 }
 
 template <typename T, int R>
@@ -359,12 +386,13 @@ void launch_shrink_rank(const ShrinkLaunch& l, int kr) {
 }
 
 template <typename T>
-void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, dim3 grid, int ksplit, const ExpandSplits& sp) {
+void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, int big_cap, dim3 grid, int ksplit, const ExpandSplits& sp) {
   hipStream_t st = static_cast<hipStream_t>(a->stream);
   const float* h = static_cast<const float*>(a->workspace);
 #define MLORA_EXPAND(RR)                                                                                                     \
   hipLaunchKernelGGL((sgmv_expand_kernel<T, RR>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, a->y_stride,     \
-                     lay.big_off, lay.sorted_off, a->num_tokens, a->num_slots, a->num_slices, ksplit, a->scaling, sp)
+                     lay.big_off, lay.small_off, big_cap, lay.sorted_off, a->num_tokens, a->num_slots, a->num_slices, ksplit,    \
+                     a->scaling, sp)
   switch (a->r) {
     case 8: MLORA_EXPAND(8); break;
     case 16: MLORA_EXPAND(16); break;
@@ -374,10 +402,10 @@ void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, dim3 grid,
 #undef MLORA_EXPAND
 }
 
-// Column ranges of about `nt` columns (a multiple of 256: four wavefronts of 64 columns).
+// Column ranges of about `nt` columns (a multiple of 512: four wavefronts of 128 columns).
 int fill_splits(const MloraAddArgs* a, int nt, ExpandSplit* out) {
-  nt = (nt + 255) & ~255;
-  if (nt < 256) nt = 256;
+  nt = (nt + 511) & ~511;
+  if (nt < 512) nt = 512;
   int total;
   for (;;) {
     total = 0;
@@ -423,14 +451,16 @@ bool sgmv_workspace_ok(const MloraAddArgs* a) {
   return a->workspace_bytes > 0 && static_cast<size_t>(a->workspace_bytes) >= partial_bytes(a->num_tokens, a->num_slices, a->r);
 }
 
-// 64-token tiles of the segments at or above the threshold.
+// Every segment of the batch: 64-token tiles of the long ones, one short tile each for the rest.
 int launch_sgmv(const MloraAddArgs* a) {
   ShrinkLaunch l;
   l.a = a;
   l.lay = plan_layout(a->num_tokens, a->num_slots);
-  int cap = l.lay.cap_big;
+  l.big_cap = (l.lay.cap_big + 7) & ~7;
+  int short_cap = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;  // a short segment is one small tile
+  if (short_cap > l.lay.cap_small) short_cap = l.lay.cap_small;
+  const int cap = l.big_cap + ((short_cap + 7) & ~7);
   if (cap == 0) return 0;
-  cap = (cap + 7) & ~7;
   l.tiles8 = cap / 8;
   int cols = 0;
   for (int i = 0; i < a->num_slices; ++i) {
@@ -472,8 +502,8 @@ int launch_sgmv(const MloraAddArgs* a) {
   }
   const int nsplit = fill_splits(a, nt, splits.split);
   dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(l.tiles8));
-  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, grid, ksplit, splits);
-  else launch_expand_rank<_Float16>(a, l.lay, grid, ksplit, splits);
+  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, l.big_cap, grid, ksplit, splits);
+  else launch_expand_rank<_Float16>(a, l.lay, l.big_cap, grid, ksplit, splits);
   return check_launch("mlora_add_lora(sgmv expand)");
 }
 

@@ -96,14 +96,6 @@ _VECTOR_RANKS = (8, 16, 32, 64)
 _PLAN_ATTR = "_mlora_segment_plans"
 
 
-def _small_batch_tokens() -> int:
-    """Batch size up to which the library keeps to its one-launch small-tile form."""
-    try:
-        return int(os.environ.get("MLORA_SMALL_BATCH_TOKENS", "1024"))
-    except ValueError:
-        return 1024
-
-
 class HipLoRABackend:
     """``LoRABackend`` whose arithmetic runs in the hand-written gfx950 kernels."""
 
@@ -112,6 +104,7 @@ class HipLoRABackend:
         if name not in _hip.FORMS:
             raise ValueError(f"unknown LoRA kernel form {name!r}; expected one of {sorted(_hip.FORMS)}")
         self.form = name
+        self._scratch: dict = {}
 
     # -- capability ---------------------------------------------------------------------
     def availability(self) -> LoRAAvailability:
@@ -166,6 +159,23 @@ class HipLoRABackend:
                 cache.clear()
             plan = cache[key] = build_segment_plan(tts, max_slots)
         return plan
+
+    def _scratch_for(self, x: torch.Tensor, num_slices: int, rank: int) -> torch.Tensor:
+        """Device scratch for the rank-r intermediate (between the two launches of the
+        long-segment form, or between workgroups sharing one shrink).  One buffer per
+        (device, stream), grown on demand: calls on one stream are ordered, so they can share
+        it; a buffer first created while a graph is being captured belongs to that graph's
+        memory pool and is not kept for later eager calls."""
+        nbytes = _hip.add_workspace_bytes(x.size(0), num_slices, rank, x.dtype)
+        stream = torch.cuda.current_stream(x.device)
+        capture = _hip.stream_capture_id(x.device)
+        key = (x.device, stream.cuda_stream, capture)
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < nbytes:
+            if len(self._scratch) >= 8:
+                self._scratch.clear()
+            buf = self._scratch[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=x.device)
+        return buf
 
     @staticmethod
     def _vectorisable(x: torch.Tensor, y: torch.Tensor, a_list, b_list, cols) -> bool:
@@ -263,11 +273,7 @@ class HipLoRABackend:
                 form = _hip.FORMS[self.form]
                 if form != _hip.FORM_TOKEN and self._vectorisable(x2, target, a_list, b_list, c_list):
                     plan = self._plan_for(metadata, tts, a_list[0].size(0)).workspace
-                    if form == _hip.FORM_SGMV or (form == _hip.FORM_AUTO and x2.size(0) > _small_batch_tokens()):
-                        # scratch for the rank-r intermediate between the two launches of the
-                        # long-segment form (the caching allocator makes this a pointer bump)
-                        nbytes = _hip.add_workspace_bytes(x2.size(0), len(chunk), a_list[0].size(-2), x2.dtype)
-                        scratch = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+                    scratch = self._scratch_for(x2, len(chunk), a_list[0].size(-2))
                 _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch)
         if staged is not None:
             staged.copy_(target)

@@ -124,6 +124,43 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
+@pytest.mark.parametrize("parts", [1, 2, 4, 8])
+@pytest.mark.parametrize("name,rank", [("down", 16), ("down", 64), ("qkv", 16), ("gate_up", 8)])
+def test_shrink_shared_between_workgroups(name, rank, parts, monkeypatch):
+    """Small-tile form with the shrink of a tile split over several workgroups (the last one to
+    arrive adds the parts up and does the expand): parity for every part count, bit-identical
+    results from one launch to the next (the order of the sum is fixed, whoever arrives last),
+    slot -1 rows untouched, and the arrival counters back at zero after every launch."""
+    from nanovllm_voxcpm_amd import synthetic
+    from nanovllm_voxcpm_amd.lora import _PLAN_ATTR
+
+    print(f"shared shrink {name} r={rank} parts={parts}", flush=True)
+    monkeypatch.setenv("MLORA_DECODE_KPARTS", str(parts))
+    proj = _make(name, 12, rank, torch.bfloat16, seed=130 + rank)
+    T = 90
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=131, device="cuda")
+    g = torch.Generator().manual_seed(132)
+    slots = torch.randint(-1, 12, (T,), generator=g, dtype=torch.int32)
+    slots[:20] = 3  # one segment above the threshold: two small tiles of the same slot
+    slots = slots.cuda()
+    backend = _backend("mfma")
+    meta = _metadata(slots)
+    runs = []
+    for _ in range(3):
+        y = y0.clone()
+        blocks = list(y.split(proj.widths, dim=-1))
+        backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0,
+                         y_packed=y if len(blocks) > 1 else None)
+        runs.append(y)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(runs[0], y0, exact, mag, slots, f"shared/{name}/r{rank}/p{parts}")
+    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    (plan,) = getattr(meta, _PLAN_ATTR).values()
+    words = plan.workspace.tolist()
+    cap_small = ((T + 15) // 16 + 12 + 7) & ~7
+    assert words[-8 * cap_small:] == [0] * (8 * cap_small)
+
+
 def test_config2_matches_reference_torch_loop():
     """The same batch against the reference's torch formulation (per-token F.linear loop) on the
     host.  With fp32 accumulation (the loop run on fp32 copies of the bf16 values) every element
@@ -515,9 +552,11 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     counts_off = sorted_off + r4(T)
     offsets_off = counts_off + r4(L + 1)
     small_off = (offsets_off + r4(L + 2) + 31) & ~31
-    cap_small = (T + 15) // 16 + min(L, T)
+    cap_small = ((T + 15) // 16 + min(L, T) + 7) & ~7
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
-    assert len(ws) == big_off + 4 * (T // 64 + min(L, T))
+    coop_off = big_off + 4 * ((T // 64 + min(L, T) + 7) & ~7)
+    assert len(ws) == coop_off + 8 * cap_small
+    assert ws[coop_off:] == [0] * (8 * cap_small)  # arrival counters rest at zero
     assert ws[sorted_off : sorted_off + len(s)] == s
     dense = [0] * (L + 1)
     for slot, n in zip(a, c):
