@@ -54,17 +54,26 @@ struct DecodeSplits {
 // (K = 32 * kNW * KSPW << kshift), 0 when it has to be worked out from K at run time.
 //
 // A compute unit fills its caches from cold memory far more slowly than the chip as a whole
-// can deliver, so when K is large and the grid small, 1 << kshift workgroups share the shrink
-// of a (tile, column range): each covers one part of K, leaves its partial sums in `partials`
-// and counts its arrival in `counters`; the last to arrive adds the parts up in a fixed order
-// (the result does not depend on who is last) and does the expand.  Nobody waits: the others
-// simply exit.  The counter is back at zero when the launch ends.
+// can deliver, so 1 << kshift workgroups can share the shrink of a tile: each covers one part
+// of K, leaves its partial sums in `partials` and counts its arrival in `counters`.  Two ways
+// to go on from there:
+//   mode 1 — the last to arrive adds the parts up and does the expand of the column range; the
+//            others simply exit.  Nobody waits.
+//   mode 2 — every workgroup also owns one part of the slice's columns: it waits (bounded, by
+//            `spin_ticks` of the 100 MHz clock) until all parts have arrived, adds them up and
+//            does the expand of its own columns, so both A[slot] and B[slot] are spread over
+//            the compute units.  A workgroup whose wait runs out computes the missing parts
+//            itself: the wait is a shortcut, never a dependency.
+// The parts are always added in the same order, so the result does not depend on timing.  All
+// exchanged words are written and read with device-scope atomic accesses, which are performed
+// at the level of the memory system that all compute units share, so no cache has to be
+// flushed.  The counter is back at zero when the launch ends.
 template <typename T, int R, int KSPW>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
-                                                            int kshift, int32_t* __restrict__ counters, float* __restrict__ partials,
-                                                            DecodeSplits splits) {
+                                                            int kshift, int mode, int spin_ticks, int32_t* __restrict__ counters,
+                                                            float* __restrict__ partials, DecodeSplits splits) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
@@ -82,7 +91,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first and
   // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD: the column ranges of one
   // tile share an XCD and its L2.
-  const int split_id = blockIdx.y >> kshift, kpart = blockIdx.y & ((1 << kshift) - 1);
+  const int group = blockIdx.y >> kshift, kpart = blockIdx.y & ((1 << kshift) - 1);
+  const int split_id = mode == 2 ? blockIdx.y : group;  // mode 2: every part has its own column range
   const int tile = blockIdx.z * 8 + blockIdx.x;
 
   // ---- round trip 1 ---------------------------------------------------------------------------
@@ -100,7 +110,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // instead of piece by piece behind a chain of branches.
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) &
-                     int(slot < num_slots) & int(sp.n0 < sp.n1) & int(sp.a != nullptr) & int(sp.b != nullptr) &
+                     int(slot < num_slots) & (int(sp.n0 < sp.n1) | int(mode == 2)) & int(sp.a != nullptr) & int(sp.b != nullptr) &
                      int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0);
   if (!usable) return;
 
@@ -204,12 +214,12 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       }
     }
   } else {
-    // This part's sums -> memory, then count the arrival.  Everything the workgroups exchange is
-    // written and read with device-scope atomic accesses, which are performed at the level of
-    // the memory system all compute units share, so no cache has to be flushed: a workgroup
-    // only waits for its own stores to be acknowledged before it is counted.
-    const int group = tile * gridDim.y + (split_id << kshift);  // first of the workgroups sharing this shrink
-    float* mine = partials + static_cast<int64_t>(group + kpart) * (16 * R);
+    // This part's sums -> memory, then count the arrival (a workgroup only waits for its own
+    // stores to be acknowledged before it is counted).
+    constexpr int kArrive = 1, kDepart = 1 << 16;
+    const int P = 1 << kshift;
+    const int first = tile * gridDim.y + (group << kshift);  // first of the workgroups sharing this shrink
+    float* mine = partials + static_cast<int64_t>(first + kpart) * (16 * R);
     for (int e = tid; e < RB * 256; e += NT) {
       const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
       float sum = 0.f;
@@ -220,24 +230,95 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    int32_t* ctr = counters + tile * MLORA_COOP_SPLITS + group;
     if (tid == 0) {
-      int32_t* ctr = counters + tile * MLORA_COOP_SPLITS + split_id;
-      const int before = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (before == (1 << kshift) - 1) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_arrived = before;
+      int v = __hip_atomic_fetch_add(ctr, kArrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kArrive;
+      if (mode == 1) {
+        if (v == P) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        const long long t0 = wall_clock64();
+        while ((v & 0xffff) < P && wall_clock64() - t0 < spin_ticks) {
+          __builtin_amdgcn_s_sleep(2);
+          v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (spin_ticks < 0) v = 0;  // diagnostic: never take the shortcut
+      }
+      s_arrived = (v & 0xffff) >= P;
     }
     __syncthreads();
-    if (s_arrived != (1 << kshift) - 1) return;  // someone else finishes this tile
-    const float* parts = partials + static_cast<int64_t>(group) * (16 * R);
-    for (int e = tid; e < 16 * R; e += NT) {
-      float sum = 0.f;
-      for (int kp = 0; kp < (1 << kshift); ++kp)
-        sum += __hip_atomic_load(parts + kp * (16 * R) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int tok = e / R, r = e % R;
-      const float v = sum * scaling;
-      const T hi = from_f32<T>(v);
-      s_hi[tok * HSTRIDE + r] = hi;
-      s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+    if (s_arrived) {
+      const float* parts = partials + static_cast<int64_t>(first) * (16 * R);
+      for (int e = tid; e < 16 * R; e += NT) {
+        float sum = 0.f;
+        for (int kp = 0; kp < P; ++kp)
+          sum += __hip_atomic_load(parts + kp * (16 * R) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int tok = e / R, r = e % R;
+        const float v = sum * scaling;
+        const T hi = from_f32<T>(v);
+        s_hi[tok * HSTRIDE + r] = hi;
+        s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+      }
+    } else if (mode == 1) {
+      return;  // someone else finishes this tile
+    } else {
+      // The other parts did not show up in time: compute every part here, with the same split
+      // of K over the wavefronts and the same order of additions as the workgroups that own them.
+      constexpr int EPT = (RB * 256 + NT - 1) / NT;
+      float total[EPT];
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) total[n] = 0.f;
+      for (int kp = 0; kp < P; ++kp) {
+        const int b0 = kp * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
+        const int b1 = KSPW > 0 ? b0 + KSPW : kp * nks + (wave + 1) * nks / kNW;
+        f32x4 part[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) part[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ks = b0; ks < b1; ++ks) {
+          Pack8 xv8, av8[RB];
+          xv8.raw = load128(xrow + ks * 32);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) av8[rb].raw = load128(arow[rb] + ks * 32);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) part[rb] = Mma<T>::run(xv8, av8[rb], part[rb]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = part[rb];
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < EPT; ++n) {
+          const int e = tid + n * NT;
+          if (e < RB * 256) {
+            const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+            total[n] += sum;
+          }
+        }
+      }
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) {
+        const int e = tid + n * NT;
+        if (e < RB * 256) {
+          const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+          const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+          if (r < R) {
+            const float v = total[n] * scaling;
+            const T hi = from_f32<T>(v);
+            s_hi[tok * HSTRIDE + r] = hi;
+            s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+          }
+        }
+      }
+    }
+    if (mode == 2) {
+      __syncthreads();  // every thread is done with the exchanged parts
+      if (tid == 0) {
+        const int v = __hip_atomic_fetch_add(ctr, kDepart, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kDepart;
+        if (v == (P | (P << 16))) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if (sp.n0 >= sp.n1) return;  // a part without columns of its own
     }
   }
   __syncthreads();
@@ -312,7 +393,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 
 struct Launch {
   const MloraAddArgs* a;
-  int small_off, include_long, kshift;
+  int small_off, include_long, kshift, mode, spin_ticks;
   int32_t* counters;
   dim3 grid;
   const DecodeSplits* splits;
@@ -323,14 +404,17 @@ void launch_one(const Launch& l) {
   const MloraAddArgs* a = l.a;
   hipLaunchKernelGGL((decode_kernel<T, R, KSPW>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
-                     a->num_slots, a->scaling, l.kshift, l.counters, static_cast<float*>(a->workspace), *l.splits);
+                     a->num_slots, a->scaling, l.kshift, l.mode, l.spin_ticks, l.counters, static_cast<float*>(a->workspace),
+                     *l.splits);
 }
 
-// The steps-per-wavefront specialisations kept: 4 (K = 1024) for every rank and 16 (K = 4096)
-// where the loads of sixteen steps still fit the register file.
+// The steps-per-wavefront specialisations kept: 1, 2 and 4 (K or a part of K = 256, 512, 1024)
+// for every rank and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
   if (kspw == 4) return launch_one<T, R, 4>(l);
+  if (kspw == 2) return launch_one<T, R, 2>(l);
+  if (kspw == 1) return launch_one<T, R, 1>(l);
   if constexpr (R <= 16) {
     if (kspw == 16) return launch_one<T, R, 16>(l);
   }
@@ -347,39 +431,30 @@ void launch_rank(const Launch& l, int r, int kspw) {
   }
 }
 
+// Largest power of two <= want that divides the k-steps into whole steps per wavefront and
+// whose partial sums (units x parts x 16 x r floats) fit the caller's workspace.
+int usable_parts(const MloraAddArgs* a, int want, long long units) {
+  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 15)) return 1;
+  const int nks = a->k / 32;
+  int parts = 1;
+  while (parts * 2 <= want) parts *= 2;
+  while (parts > 1) {
+    const size_t need = static_cast<size_t>(units) * parts * 16 * a->r * sizeof(float);
+    if (nks % (parts * kNW) == 0 && static_cast<size_t>(a->workspace_bytes) >= need) break;
+    parts /= 2;
+  }
+  return parts;
+}
+
 }  // namespace
 
-// Workspace that lets the small-tile form share a shrink between workgroups: it is only done
-// for grids of at most 128 (tile, column range) pairs, four parts each, 16 x r sums per part.
-size_t decode_workspace_bytes(int r) { return static_cast<size_t>(128) * 4 * 16 * r * sizeof(float); }
+// Workspace that lets the small-tile form share a shrink between workgroups: room for 1024
+// partial tiles of 16 x r sums (sharing is only chosen for grids that fit).
+size_t decode_workspace_bytes(int r) { return static_cast<size_t>(1024) * 16 * r * sizeof(float); }
 
 int launch_decode(const MloraAddArgs* a, bool include_long) {
   DecodeSplits splits;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-
-  // Column range per workgroup: every range repeats the shrink of its tile, so ranges are kept
-  // wide enough (default 1024 columns: two 64-column spans per wavefront) for the expand to
-  // outweigh that repeat.
-  int nt = env_int("MLORA_DECODE_NT", 1024);
-  if (nt < 64) nt = 64;
-  nt = (nt + 63) & ~63;
-  int total = 0;
-  for (;;) {
-    total = 0;
-    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
-    if (total <= kMaxSplits) break;
-    nt *= 2;
-  }
-  if (total == 0) return 0;
-  int s = 0;
-  for (int i = 0; i < a->num_slices; ++i) {
-    const MloraSlice& sl = a->slices[i];
-    for (int n0 = 0; n0 < sl.n; n0 += nt) {
-      DecodeSplit& d = splits.split[s++];
-      d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
-      d.n0 = n0; d.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
-    }
-  }
   int cap = lay.cap_small;
   if (!include_long) {  // a segment below the threshold is exactly one small tile
     const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
@@ -387,29 +462,85 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
   }
   if (cap == 0) return 0;
   cap = (cap + 7) & ~7;
-  // Workgroups sharing one shrink: only worth its extra round trip through memory when a
-  // workgroup would otherwise pull a long K through a single compute unit while most of the
-  // chip idles; needs room for the partial sums in the caller's workspace.
-  const int nks_all = a->k / 32;
-  int kshift = 0;
-  const int want = env_int("MLORA_DECODE_KPARTS", 0);
-  if (total <= MLORA_COOP_SPLITS && a->workspace && !(reinterpret_cast<uintptr_t>(a->workspace) & 15)) {
-    int parts = 1;
-    if (want > 0) parts = want;
-    else if (a->k >= 2048 && static_cast<long long>(cap) * total <= 128) parts = 4;
-    while (parts > 1) {
-      const size_t need = static_cast<size_t>(cap) * total * parts * 16 * a->r * sizeof(float);
-      if ((parts & (parts - 1)) == 0 && nks_all % (parts * kNW) == 0 && static_cast<size_t>(a->workspace_bytes) >= need) break;
-      parts /= 2;
-    }
-    while ((1 << kshift) < parts) ++kshift;
-  }
+
+  int live = 0;
+  for (int i = 0; i < a->num_slices; ++i) live += a->slices[i].n > 0;
+  if (live == 0) return 0;
+
   Launch l;
   l.a = a; l.small_off = lay.small_off; l.include_long = include_long ? 1 : 0; l.splits = &splits;
-  l.kshift = kshift;
   l.counters = a->plan + lay.coop_off;
-  l.grid = dim3(8, static_cast<unsigned>(total << kshift), static_cast<unsigned>(cap / 8));
-  const int nks = nks_all >> kshift;
+  l.spin_ticks = env_int("MLORA_DECODE_SPIN_TICKS", 20000);  // 200 us of the 100 MHz clock
+  l.kshift = 0;
+  l.mode = 0;
+  int total = 0;
+
+  // Mode 2: the workgroups of a (tile, slice) each take one part of K and one part of the columns.
+  // The exchange costs a few trips through memory (about 2 us measured), which pays when K is
+  // long (4096: 8.9 -> 7.9 us per launch at 32 tiles) and does not at K = 1024.
+  int mode = env_int("MLORA_DECODE_MODE", -1);
+  const int want = env_int("MLORA_DECODE_KPARTS", 0);
+  if (mode == 2 || (mode < 0 && a->k >= 2048)) {
+    int parts = 1;
+    if (live == a->num_slices && live <= MLORA_COOP_SPLITS) parts = usable_parts(a, want > 0 ? want : 4, static_cast<long long>(cap) * live);
+    if (parts > 1 && (mode == 2 || static_cast<long long>(cap) * live * parts <= 1024)) {
+      int s = 0;
+      for (int i = 0; i < a->num_slices; ++i) {
+        const MloraSlice& sl = a->slices[i];
+        const int w = ((sl.n + parts - 1) / parts + 63) & ~63;  // columns per part, whole 64-column spans
+        for (int j = 0; j < parts; ++j) {
+          DecodeSplit& d = splits.split[s++];
+          d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
+          d.n0 = j * w < sl.n ? j * w : sl.n;
+          d.n1 = (j + 1) * w < sl.n ? (j + 1) * w : sl.n;
+        }
+      }
+      total = s;
+      l.mode = 2;
+      while ((1 << l.kshift) < parts) ++l.kshift;
+    } else if (mode == 2) {
+      mode = 0;
+    }
+  }
+  if (l.mode == 0) {
+    // Column range per workgroup: every range repeats the shrink of its tile, so ranges are kept
+    // wide enough (default 1024 columns: two 64-column spans per wavefront) for the expand to
+    // outweigh that repeat.
+    int nt = env_int("MLORA_DECODE_NT", 1024);
+    if (nt < 64) nt = 64;
+    nt = (nt + 63) & ~63;
+    for (;;) {
+      total = 0;
+      for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
+      if (total <= kMaxSplits) break;
+      nt *= 2;
+    }
+    if (total == 0) return 0;
+    int s = 0;
+    for (int i = 0; i < a->num_slices; ++i) {
+      const MloraSlice& sl = a->slices[i];
+      for (int n0 = 0; n0 < sl.n; n0 += nt) {
+        DecodeSplit& d = splits.split[s++];
+        d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
+        d.n0 = n0; d.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
+      }
+    }
+    // Mode 1: workgroups sharing the shrink of a (tile, column range), the last one finishing it.
+    // Only worth its extra round trip through memory when a workgroup would otherwise pull a long
+    // K through a single compute unit while most of the chip idles.
+    if ((mode == 1 || mode < 0) && total <= MLORA_COOP_SPLITS) {
+      int parts = 1;
+      if (want > 0) parts = want;
+      else if (a->k >= 2048 && static_cast<long long>(cap) * total <= 128) parts = 4;
+      parts = usable_parts(a, parts, static_cast<long long>(cap) * total);
+      if (parts > 1) {
+        l.mode = 1;
+        while ((1 << l.kshift) < parts) ++l.kshift;
+      }
+    }
+  }
+  l.grid = dim3(8, static_cast<unsigned>(l.mode == 2 ? total : total << l.kshift), static_cast<unsigned>(cap / 8));
+  const int nks = (a->k / 32) >> l.kshift;
   const int kspw = (nks % kNW == 0) ? nks / kNW : 0;
   if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16>(l, a->r, kspw);
   else launch_rank<_Float16>(l, a->r, kspw);

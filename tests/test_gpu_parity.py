@@ -124,18 +124,23 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
+@pytest.mark.parametrize("mode", [1, 2])
 @pytest.mark.parametrize("parts", [1, 2, 4, 8])
 @pytest.mark.parametrize("name,rank", [("down", 16), ("down", 64), ("qkv", 16), ("gate_up", 8)])
-def test_shrink_shared_between_workgroups(name, rank, parts, monkeypatch):
-    """Small-tile form with the shrink of a tile split over several workgroups (the last one to
-    arrive adds the parts up and does the expand): parity for every part count, bit-identical
-    results from one launch to the next (the order of the sum is fixed, whoever arrives last),
-    slot -1 rows untouched, and the arrival counters back at zero after every launch."""
+def test_shrink_shared_between_workgroups(name, rank, parts, mode, monkeypatch):
+    """Small-tile form with the shrink of a tile split over several workgroups.  Mode 1: the last
+    one to arrive adds the parts up and does the expand.  Mode 2: every workgroup waits (bounded)
+    for the parts and expands its own columns; with the wait disabled from the host every
+    workgroup takes the path that computes all parts itself.  Checked: parity for every part
+    count, bit-identical results from one launch to the next and between the waiting and the
+    non-waiting path (the order of the sum is fixed, whatever the timing), slot -1 rows untouched,
+    and the arrival counters back at zero after every launch."""
     from nanovllm_voxcpm_amd import synthetic
     from nanovllm_voxcpm_amd.lora import _PLAN_ATTR
 
-    print(f"shared shrink {name} r={rank} parts={parts}", flush=True)
+    print(f"shared shrink {name} r={rank} parts={parts} mode={mode}", flush=True)
     monkeypatch.setenv("MLORA_DECODE_KPARTS", str(parts))
+    monkeypatch.setenv("MLORA_DECODE_MODE", str(mode))
     proj = _make(name, 12, rank, torch.bfloat16, seed=130 + rank)
     T = 90
     x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=131, device="cuda")
@@ -146,15 +151,17 @@ def test_shrink_shared_between_workgroups(name, rank, parts, monkeypatch):
     backend = _backend("mfma")
     meta = _metadata(slots)
     runs = []
-    for _ in range(3):
+    for spin in ("20000", "20000", "-1", "0"):
+        monkeypatch.setenv("MLORA_DECODE_SPIN_TICKS", spin)
         y = y0.clone()
         blocks = list(y.split(proj.widths, dim=-1))
         backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0,
                          y_packed=y if len(blocks) > 1 else None)
         runs.append(y)
     exact, mag = _exact(proj, x, y0, slots)
-    _check(runs[0], y0, exact, mag, slots, f"shared/{name}/r{rank}/p{parts}")
-    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    _check(runs[0], y0, exact, mag, slots, f"shared/{name}/r{rank}/p{parts}/m{mode}")
+    for other in runs[1:]:
+        assert torch.equal(runs[0], other)
     (plan,) = getattr(meta, _PLAN_ATTR).values()
     words = plan.workspace.tolist()
     cap_small = ((T + 15) // 16 + 12 + 7) & ~7
