@@ -195,22 +195,53 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
 // ---- expand -------------------------------------------------------------------------------------
 // grid (8, column ranges, tiles / 8), four wavefronts.  OUT[tokens x cols] = H . B[slot]^T with
 // the tokens as MFMA rows: in the accumulator layout a lane then holds four tokens of one column,
-// and with the B rows of the eight MFMAs of a 128-column span interleaved (MFMA j takes column
-// 8 * (lane % 16) + j) it holds eight consecutive columns of each of those tokens.  Sixteen
-// consecutive lanes therefore cover 256 contiguous bytes of one y row: y is read and written in
-// fully coalesced 128-bit accesses.
-constexpr int kSpan = 128;
+// and with the B rows of the CPL MFMAs of a span of 16 * CPL columns interleaved (MFMA j takes
+// column CPL * (lane % 16) + j) it holds CPL consecutive columns of each of those tokens.
+// Sixteen consecutive lanes therefore cover 32 * CPL contiguous bytes of one y row: y is read
+// and written in fully coalesced accesses (128-bit for CPL = 8, 64-bit for CPL = 4; the narrower
+// span needs half the registers, so more wavefronts and more of their loads are in flight).
+// TPF: token blocks whose y rows are requested together.
+template <typename T, int N> union alignas(N * sizeof(T)) YVec {
+  T e[N];
+  uint32_t u[N / 2];
+};
 
-template <typename T, int R>
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int N> struct YRaw;
+template <> struct YRaw<4> { typedef u32x2 type; };
+template <> struct YRaw<8> { typedef u32x4 type; };
+
+// y is touched once per launch: with `nt` it is moved with the non-temporal hint so that it does
+// not push the B rows, which every tile of a slot re-reads, out of the L2.
+template <typename T, int N>
+__device__ __forceinline__ YVec<T, N> load_y(const T* p, int nt) {
+  typedef typename YRaw<N>::type Raw;
+  YVec<T, N> v;
+  Raw r = nt ? __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p)) : *reinterpret_cast<const Raw*>(p);
+  __builtin_memcpy(&v, &r, sizeof(r));
+  return v;
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
+  typedef typename YRaw<N>::type Raw;
+  Raw r;
+  __builtin_memcpy(&r, &v, sizeof(r));
+  if (nt) __builtin_nontemporal_store(r, reinterpret_cast<Raw*>(p));
+  else *reinterpret_cast<Raw*>(p) = r;
+}
+
+template <typename T, int R, int CPL, int TPF>
 __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                                                           void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
                                                                           int big_cap, int sorted_off, int T_, int num_slots,
-                                                                          int num_slices, int ksplit, float scaling, ExpandSplits splits) {
+                                                                          int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps
   constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
   constexpr int NT = kExpandWaves * kWave;
   constexpr int CPR = R / 8;             // groups of eight ranks per token
+  constexpr int SPAN = 16 * CPL;         // columns of one span
 
   __shared__ __attribute__((aligned(16))) T s_h[MLORA_TILE_BIG * HSTRIDE];
   __shared__ __attribute__((aligned(16))) int s_row[MLORA_TILE_BIG];
@@ -268,22 +299,14 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
 
   const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
   T* ybase = static_cast<T*>(yv_) + sp.y_col;
-  // rows of this lane's four tokens in every token block
-  const T* yrow[TB][4];
-#pragma unroll
-  for (int tb = 0; tb < TB; ++tb) {
-    const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[tb * 16 + 4 * lg]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) yrow[tb][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
-  }
 
-  for (int c0 = sp.n0 + wave * kSpan; c0 < sp.n1; c0 += kExpandWaves * kSpan) {
+  for (int c0 = sp.n0 + wave * SPAN; c0 < sp.n1; c0 += kExpandWaves * SPAN) {
     // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
     // their H operand is zero; columns past the range repeat the last one and are never stored)
-    Pack8 bop[8][KSTEPS];
+    Pack8 bop[CPL][KSTEPS];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      int n = c0 + 8 * lr + j;
+    for (int j = 0; j < CPL; ++j) {
+      int n = c0 + CPL * lr + j;
       n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -291,20 +314,26 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
         bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
       }
     }
-    const int c = c0 + 8 * lr;
+    const int c = c0 + CPL * lr;
     const bool col_ok = c < sp.n1;
     const int cl = col_ok ? c : sp.n1 - 8;
 
 #pragma unroll
-    for (int tp = 0; tp < TB; tp += 2) {  // two token blocks at a time: their y rows are in flight together
+    for (int tp = 0; tp < TB; tp += TPF) {  // TPF token blocks at a time: their y rows are in flight together
       if (tp * 16 >= m) continue;
-      Pack8 yreg[2][4];
+      YVec<T, CPL> yreg[TPF][4];
+      T* yrow[TPF][4];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < TPF; ++u) {
+        const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[(tp + u) * 16 + 4 * lg]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) yreg[u][i].raw = load128(yrow[tp + u][i] + cl);
+        for (int i = 0; i < 4; ++i) {
+          yrow[u][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
+          yreg[u][i] = load_y<T, CPL>(yrow[u][i] + cl, nt);
+        }
+      }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < TPF; ++u) {
         const int tb = tp + u;
         if (tb * 16 >= m) continue;
         Pack8 hop[KSTEPS], hlo[KSTEPS];
@@ -319,9 +348,9 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
             hlo[ks].raw = i32x4{0, 0, 0, 0};
           }
         }
-        f32x4 out[8];
+        f32x4 out[CPL];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < CPL; ++j) {
           out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -329,17 +358,14 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
             out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
           }
         }
-        // lane holds out[token 16*tb + 4*lg + i][column c0 + 8*lr + j]
+        // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (col_ok && tb * 16 + 4 * lg + i < m) {
-            float yf[8];
-            unpack8<T>(yreg[u][i], yf);
+            YVec<T, CPL> r;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) yf[j] += out[j][i];
-            Pack8 r;
-            pack8<T>(yf, r);
-            store128(const_cast<T*>(yrow[tb][i]) + c, r.raw);
+            for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(yreg[u][i].e[j]) + out[j][i]);
+            store_y<T, CPL>(yrow[u][i] + c, r, nt);
           }
         }
       }
@@ -386,13 +412,19 @@ void launch_shrink_rank(const ShrinkLaunch& l, int kr) {
 }
 
 template <typename T>
-void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, int big_cap, dim3 grid, int ksplit, const ExpandSplits& sp) {
+void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, int big_cap, dim3 grid, int ksplit, int cpl, const ExpandSplits& sp) {
   hipStream_t st = static_cast<hipStream_t>(a->stream);
   const float* h = static_cast<const float*>(a->workspace);
+  const int nt = env_int("MLORA_SGMV_NT_HINT", 0);
 #define MLORA_EXPAND(RR)                                                                                                     \
-  hipLaunchKernelGGL((sgmv_expand_kernel<T, RR>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, a->y_stride,     \
+  if (cpl == 4)                                                                                                              \
+    hipLaunchKernelGGL((sgmv_expand_kernel<T, RR, 4, 4>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y,          \
+                       a->y_stride, lay.big_off, lay.small_off, big_cap, lay.sorted_off, a->num_tokens, a->num_slots,        \
+                       a->num_slices, ksplit, a->scaling, nt, sp);                                                           \
+  else                                                                                                                       \
+    hipLaunchKernelGGL((sgmv_expand_kernel<T, RR, 8, 2>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, a->y_stride, \
                      lay.big_off, lay.small_off, big_cap, lay.sorted_off, a->num_tokens, a->num_slots, a->num_slices, ksplit,    \
-                     a->scaling, sp)
+                     a->scaling, nt, sp)
   switch (a->r) {
     case 8: MLORA_EXPAND(8); break;
     case 16: MLORA_EXPAND(16); break;
@@ -501,9 +533,10 @@ int launch_sgmv(const MloraAddArgs* a) {
     nt = want > 8192 ? 8192 : static_cast<int>(want);
   }
   const int nsplit = fill_splits(a, nt, splits.split);
+  const int cpl = env_int("MLORA_SGMV_CPL", 8) == 4 ? 4 : 8;
   dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(l.tiles8));
-  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, l.big_cap, grid, ksplit, splits);
-  else launch_expand_rank<_Float16>(a, l.lay, l.big_cap, grid, ksplit, splits);
+  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, l.big_cap, grid, ksplit, cpl, splits);
+  else launch_expand_rank<_Float16>(a, l.lay, l.big_cap, grid, ksplit, cpl, splits);
   return check_launch("mlora_add_lora(sgmv expand)");
 }
 
