@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
                                                                           float* __restrict__ hws, int64_t xs, int big_off,
                                                                           int small_off, int big_cap, int sorted_off, int T_, int K,
                                                                           int num_slots, int num_slices, int ksplit, int krange,
-                                                                          ShrinkSlices sl) {
+                                                                          int all_slices, ShrinkSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -114,7 +114,10 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
-  const int slice = blockIdx.y / ksplit, kpart = blockIdx.y % ksplit;
+  // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
+  // registers (its K part is a single batch then), instead of one workgroup per slice
+  const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
+  const int nsl = all_slices ? num_slices : 1;
   const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
 
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
@@ -129,6 +132,9 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
   const int ti = wave * 16 + lr;
   const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
   const T* xptr = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + k0 + lg * 8;
+  Pack8 xa[XB];
+ for (int si = 0; si < nsl; ++si) {
+  const int slice = slice0 + si;
   const T* A = static_cast<const T*>(sl.a[slice]) + static_cast<int64_t>(slot) * R * K + k0;
 
   f32x4 acc[RB];
@@ -138,13 +144,13 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
   for (int slab = 0; slab < nslab; ++slab) {
     const T* Aslab = A + slab * KR;
     const T* xslab = xptr + slab * KR;
-    // the first batch of x loads goes out together with the slab copy
-    Pack8 xa[XB];
-    if (active) {
+    // the first batch of x loads goes out together with the slab copy (later slices of an
+    // all-slices walk already hold it)
+    if (active && si == 0) {
 #pragma unroll
       for (int i = 0; i < XB; ++i) xa[i].raw = load128(xslab + i * 32);
     }
-    if (slab > 0) __syncthreads();  // everyone is done reading the previous slab
+    if (slab > 0 || si > 0) __syncthreads();  // everyone is done reading the previous slab
 #pragma unroll
     for (int c0 = 0; c0 < CHUNKS; c0 += SB) {
       i32x4 v[SB];
@@ -190,6 +196,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
       if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
     }
   }
+ }
 }
 
 // ---- expand -------------------------------------------------------------------------------------
@@ -379,16 +386,16 @@ struct ShrinkLaunch {
   ShrinkSlices sl;
   int tiles8;   // grid extent over tiles / 8
   int big_cap;  // workgroups below this index take 64-token tiles, the rest short segments
-  int ksplit, krange;
+  int ksplit, krange, all_slices;
 };
 
 template <typename T, int R, int KR>
 void launch_shrink_one(const ShrinkLaunch& l) {
   const MloraAddArgs* a = l.a;
-  dim3 grid(8, static_cast<unsigned>(a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
+  dim3 grid(8, static_cast<unsigned>(l.all_slices ? l.ksplit : a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
   hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
-                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.sl);
+                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, l.sl);
 }
 
 template <typename T, int R>
@@ -517,6 +524,17 @@ int launch_sgmv(const MloraAddArgs* a) {
   if (ksplit > max_parts) ksplit = max_parts;
   if (ksplit > kMaxKSplit) ksplit = kMaxKSplit;
   while (ksplit > 1 && a->k % (kr * ksplit) != 0) --ksplit;
+  // three or more slices: one workgroup walks them all with the x rows it already holds, when
+  // its K part is a single batch of loads (measured on the prefill batch: qkv 31.9 -> 29.6 us per
+  // call; with two slices the shorter chain of separate workgroups wins, gate_up 76.6 vs 77.8)
+  l.all_slices = 0;
+  if (a->num_slices >= env_int("MLORA_SGMV_ALL_SLICES", 3) && kr <= 512) {
+    const int parts = a->k / kr;
+    if (parts <= kMaxKSplit && parts <= max_parts) {
+      ksplit = parts;
+      l.all_slices = 1;
+    }
+  }
   l.ksplit = ksplit;
   l.krange = a->k / ksplit;
   if (a->dtype == MLORA_DTYPE_BF16) launch_shrink_rank<__bf16>(l, kr);
