@@ -47,6 +47,9 @@ WORKLOADS = {
     "prefill": dict(slots=8, rank=64, distinct_layers=4,
                     text="prefill SGMV bf16 (BASELINE configs[2]): 16 sequences of 64..1024 tokens, 8 adapters, "
                          "rank 64, 25% of sequences without adapter, qkv/o/gate_up/down x 24 layers"),
+    "backbone": dict(slots=32, rank=32, distinct_layers=24,
+                     text="synthetic backbone bf16 (BASELINE configs[4]): 24 layers, hidden 1024, 16 q / 2 kv heads, "
+                          "SwiGLU 4096, 64 decode streams, context U[128,2048], 32 rank-32 adapters on all linears"),
     "mixed": dict(slots=128, rank=64, distinct_layers=4,
                   text="mixed bf16 (BASELINE configs[3]): 2 x 2048-token chunks + 4096 decodes, 128 adapters of "
                        "ranks {8,16,32,64} padded to 64, Zipf(1.1), qkv/o/gate_up/down x 24 layers"),
@@ -205,6 +208,60 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
     }
 
 
+def run_backbone(args) -> None:
+    """BASELINE configs[4]: decode-step latency of a synthetic 24-layer decoder (hidden 1024, 16 query /
+    2 KV heads of 64, SwiGLU 4096, RMSNorm; 64 streams with context lengths U[128, 2048]; 32 rank-32
+    adapters on all linears) with the LoRA kernels against the same step with LoRA disabled."""
+    import torch
+
+    from nanovllm_voxcpm_amd.backbone import MiniDecoder
+    from nanovllm_voxcpm_amd.utils.context import LoRAContext, reset_lora_context, set_lora_context
+
+    device = "cuda:0"
+    streams, adapters, rank = 64, 32, 32
+    model = MiniDecoder(max_loras=adapters, rank=rank).to(device=device, dtype=torch.bfloat16)
+    model.init_random(seed=500, adapters=adapters, rank=rank)
+    g = torch.Generator().manual_seed(501)
+    positions = torch.randint(128, 2049, (streams,), generator=g).to(device)
+    slots = torch.randint(0, adapters, (streams,), generator=g, dtype=torch.int32).to(device)
+    x = torch.randn(streams, model.hidden, generator=g).to(torch.bfloat16).to(device)
+    caches = model.make_cache(streams, 2049, torch.bfloat16, device, seed=502)
+
+    def timed(lora_on: bool):
+        reset_lora_context()
+        if lora_on:
+            set_lora_context(LoRAContext(token_to_slot=slots, no_lora_flag=False))
+        with torch.inference_mode():
+            for _ in range(2):
+                out = model(x, caches, positions)
+            torch.cuda.synchronize()
+            eager = time_region(lambda: model(x, caches, positions), 5)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = model(x, caches, positions)
+            for _ in range(args.warmup):
+                graph.replay()
+            ms = time_region(graph.replay, args.steps)
+        reset_lora_context()
+        return ms, eager, out.float().clone()
+
+    off_ms, off_eager, y_off = timed(False)
+    on_ms, on_eager, y_on = timed(True)
+    print(json.dumps({
+        "metric": "decode-step latency of the synthetic backbone, LoRA kernels on vs LoRA disabled (us), 1 GPU",
+        "value": round(on_ms * 1e3, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(on_ms, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": WORKLOADS["backbone"]["text"], "streams": streams, "adapters": adapters, "rank": rank,
+                   "launch": "graph replay"},
+        "us_per_step_lora_off": round(off_ms * 1e3, 2),
+        "us_lora_cost": round((on_ms - off_ms) * 1e3, 2),
+        "lora_overhead_pct": round(100 * (on_ms - off_ms) / off_ms, 2),
+        "us_per_step_eager": {"lora_on": round(on_eager * 1e3, 1), "lora_off": round(off_eager * 1e3, 1)},
+        "lora_changes_output": bool((y_on - y_off).abs().max().item() > 0),
+    }))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -233,6 +290,9 @@ def main() -> None:
     torch.cuda.set_device(0)
     spec = WORKLOADS[args.workload]
     rank = spec["rank"]
+    if args.workload == "backbone":
+        run_backbone(args)
+        return
     layers, slots = build_workload(args.workload, device)
     if args.hot_layers > 0:
         layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
