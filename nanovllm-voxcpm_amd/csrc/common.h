@@ -102,7 +102,7 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   // tile per XCD), and every record such a grid may touch has to exist
   p.cap_small = ((T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs + 7) & ~7;
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
-  p.cap_big = (T / MLORA_TILE_BIG + segs + 7) & ~7;
+  p.cap_big = (T / MLORA_TILE_BIG + segs + 31) & ~31;  // groups of up to four tiles, eight groups abreast
   // arrival counters of the workgroups that share one small tile's shrink (zero between launches)
   p.coop_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
   p.total_words = p.coop_off + MLORA_COOP_SPLITS * p.cap_small;

@@ -238,10 +238,10 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
   else *reinterpret_cast<Raw*>(p) = r;
 }
 
-template <typename T, int R, int CPL, int TPF>
+template <typename T, int R, int CPL, int TPF, int G>
 __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                                                           void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
-                                                                          int big_cap, int sorted_off, int T_, int num_slots,
+                                                                          int big_units, int sorted_off, int T_, int num_slots,
                                                                           int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps
@@ -250,129 +250,169 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
   constexpr int CPR = R / 8;             // groups of eight ranks per token
   constexpr int SPAN = 16 * CPL;         // columns of one span
 
-  __shared__ __attribute__((aligned(16))) T s_h[MLORA_TILE_BIG * HSTRIDE];
-  __shared__ __attribute__((aligned(16))) int s_row[MLORA_TILE_BIG];
+  __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) int s_row[G * MLORA_TILE_BIG];
+  __shared__ int s_slot[G], s_m[G];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
-  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  // A workgroup takes G consecutive 64-token tiles (consecutive tiles mostly belong to one slot,
+  // whose B rows then stay in registers across them), or, past `big_units`, one short segment.
+  const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const bool is_big = unit < big_units;
+  const int sidx = is_big ? 0 : unit - big_units;
 
-  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
+  // header and every candidate record are requested together (all addresses are in bounds for
+  // the whole grid)
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
+  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);
+  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);
+  const i32x4 small = *reinterpret_cast<const i32x4*>(plan + small_off + sidx * MLORA_SMALL_TILE_WORDS);
+  i32x4 big[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) big[g] = reinterpret_cast<const i32x4*>(plan + big_off)[is_big ? unit * G + g : 0];
   const ExpandSplit sp = splits.split[blockIdx.y];
-  if (!(tr.ok & int(sp.n0 < sp.n1))) return;
-  const int slot = tr.slot, start = tr.start, m = tr.m;
+  const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
+  int slot[G], start[G], m[G], any = 0;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const bool have = is_big ? unit * G + g < n_big : (g == 0 && sidx < n_short);
+    slot[g] = is_big ? big[g][0] : small[0];
+    start[g] = is_big ? big[g][1] : small[2];
+    m[g] = is_big ? big[g][2] : small[1];
+    if (!have || m[g] <= 0 || slot[g] < 0 || slot[g] >= num_slots) m[g] = 0;
+    any |= m[g];
+  }
+  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
+  if (!usable) return;
 
-  // token rows of the tile (entries past its end repeat the last token: a valid row to read,
-  // never written)
-  if (tid < MLORA_TILE_BIG) s_row[tid] = plan[sorted_off + start + (tid < m ? tid : m - 1)];
-
-  // H tile -> LDS: sum the K partials, scale, split into leading part and remainder (absent
-  // tokens get zeros)
+  // token rows (entries past the end of a tile repeat its last token: a valid row to read, never
+  // written) and the H tiles -> LDS: K partials summed, scaled, split into leading part and
+  // remainder (absent tokens get zeros)
   {
     const int64_t hrow = static_cast<int64_t>(num_slices) * R;
     const int64_t part = static_cast<int64_t>(T_) * hrow;
-    const float* src = hws + static_cast<int64_t>(start) * hrow + sp.slice * R;
-    for (int c = tid; c < MLORA_TILE_BIG * CPR; c += NT) {
-      const int tok = c / CPR, ch = c % CPR;
-      Pack8 hi, lo;
-      hi.raw = i32x4{0, 0, 0, 0};
-      lo.raw = i32x4{0, 0, 0, 0};
-      if (tok < m) {
-        const float* q = src + tok * hrow + ch * 8;
-        f32x4 s0 = *reinterpret_cast<const f32x4*>(q), s1 = *reinterpret_cast<const f32x4*>(q + 4);
-        for (int kp = 1; kp < ksplit; ++kp) {
-          const f32x4 t0 = *reinterpret_cast<const f32x4*>(q + kp * part), t1 = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
-          s0[0] += t0[0]; s0[1] += t0[1]; s0[2] += t0[2]; s0[3] += t0[3];
-          s1[0] += t1[0]; s1[1] += t1[1]; s1[2] += t1[2]; s1[3] += t1[3];
-        }
-        float v[8], rem[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          v[i] = s0[i] * scaling;
-          v[4 + i] = s1[i] * scaling;
-        }
-        pack8<T>(v, hi);
-        float back[8];
-        unpack8<T>(hi, back);
+    for (int g = 0; g < G; ++g) {
+      if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; }
+      if (m[g] == 0) continue;
+      if (tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
+      const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
+      for (int c = tid; c < MLORA_TILE_BIG * CPR; c += NT) {
+        const int tok = c / CPR, ch = c % CPR;
+        Pack8 hi, lo;
+        hi.raw = i32x4{0, 0, 0, 0};
+        lo.raw = i32x4{0, 0, 0, 0};
+        if (tok < m[g]) {
+          const float* q = src + tok * hrow + ch * 8;
+          f32x4 s0 = *reinterpret_cast<const f32x4*>(q), s1 = *reinterpret_cast<const f32x4*>(q + 4);
+          for (int kp = 1; kp < ksplit; ++kp) {
+            const f32x4 t0 = *reinterpret_cast<const f32x4*>(q + kp * part), t1 = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+            s0[0] += t0[0]; s0[1] += t0[1]; s0[2] += t0[2]; s0[3] += t0[3];
+            s1[0] += t1[0]; s1[1] += t1[1]; s1[2] += t1[2]; s1[3] += t1[3];
+          }
+          float v[8], rem[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
-        pack8<T>(rem, lo);
+          for (int i = 0; i < 4; ++i) {
+            v[i] = s0[i] * scaling;
+            v[4 + i] = s1[i] * scaling;
+          }
+          pack8<T>(v, hi);
+          float back[8];
+          unpack8<T>(hi, back);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
+          pack8<T>(rem, lo);
+        }
+        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
+        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
       }
-      *reinterpret_cast<i32x4*>(&s_h[tok * HSTRIDE + ch * 8]) = hi.raw;
-      *reinterpret_cast<i32x4*>(&s_h[tok * HSTRIDE + R + ch * 8]) = lo.raw;
     }
   }
   __syncthreads();
 
-  const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
   T* ybase = static_cast<T*>(yv_) + sp.y_col;
 
   for (int c0 = sp.n0 + wave * SPAN; c0 < sp.n1; c0 += kExpandWaves * SPAN) {
-    // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
-    // their H operand is zero; columns past the range repeat the last one and are never stored)
     Pack8 bop[CPL][KSTEPS];
-#pragma unroll
-    for (int j = 0; j < CPL; ++j) {
-      int n = c0 + CPL * lr + j;
-      n = n < sp.n1 ? n : sp.n1 - 1;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = (lg + 4 * ks) & (R / 8 - 1);
-        bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-      }
-    }
+    int loaded = -1;  // slot whose B rows are in bop
     const int c = c0 + CPL * lr;
     const bool col_ok = c < sp.n1;
     const int cl = col_ok ? c : sp.n1 - 8;
 
-#pragma unroll
-    for (int tp = 0; tp < TB; tp += TPF) {  // TPF token blocks at a time: their y rows are in flight together
-      if (tp * 16 >= m) continue;
-      YVec<T, CPL> yreg[TPF][4];
-      T* yrow[TPF][4];
-#pragma unroll
-      for (int u = 0; u < TPF; ++u) {
-        const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[(tp + u) * 16 + 4 * lg]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          yrow[u][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
-          yreg[u][i] = load_y<T, CPL>(yrow[u][i] + cl, nt);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < TPF; ++u) {
-        const int tb = tp + u;
-        if (tb * 16 >= m) continue;
-        Pack8 hop[KSTEPS], hlo[KSTEPS];
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int kc = lg + 4 * ks;
-          if (kc * 8 < R) {
-            hop[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-            hlo[ks].raw = *reinterpret_cast<const i32x4*>(&s_h[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
-          } else {
-            hop[ks].raw = i32x4{0, 0, 0, 0};
-            hlo[ks].raw = i32x4{0, 0, 0, 0};
-          }
-        }
-        f32x4 out[CPL];
+    for (int g = 0; g < G; ++g) {
+      const int mg = s_m[g];
+      if (mg == 0) continue;
+      const int sg = s_slot[g];
+      if (sg != loaded) {
+        // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
+        // their H operand is zero; columns past the range repeat the last one and are never stored)
+        const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
-          out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+          int n = c0 + CPL * lr + j;
+          n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) {
-            out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
-            out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
+            const int kc = (lg + 4 * ks) & (R / 8 - 1);
+            bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
           }
         }
-        // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
+        loaded = sg;
+      }
+      const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
+      const int* rowg = s_row + g * MLORA_TILE_BIG;
+
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (col_ok && tb * 16 + 4 * lg + i < m) {
-            YVec<T, CPL> r;
+      for (int tp = 0; tp < TB; tp += TPF) {  // TPF token blocks at a time: their y rows are in flight together
+        if (tp * 16 >= mg) continue;
+        YVec<T, CPL> yreg[TPF][4];
+        T* yrow[TPF][4];
 #pragma unroll
-            for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(yreg[u][i].e[j]) + out[j][i]);
-            store_y<T, CPL>(yrow[u][i] + c, r, nt);
+        for (int u = 0; u < TPF; ++u) {
+          const i32x4 rows = *reinterpret_cast<const i32x4*>(&rowg[(tp + u) * 16 + 4 * lg]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            yrow[u][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
+            yreg[u][i] = load_y<T, CPL>(yrow[u][i] + cl, nt);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < TPF; ++u) {
+          const int tb = tp + u;
+          if (tb * 16 >= mg) continue;
+          Pack8 hop[KSTEPS], hlo[KSTEPS];
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int kc = lg + 4 * ks;
+            if (kc * 8 < R) {
+              hop[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+              hlo[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
+            } else {
+              hop[ks].raw = i32x4{0, 0, 0, 0};
+              hlo[ks].raw = i32x4{0, 0, 0, 0};
+            }
+          }
+          f32x4 out[CPL];
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) {
+            out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+              out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
+              out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
+            }
+          }
+          // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (col_ok && tb * 16 + 4 * lg + i < mg) {
+              YVec<T, CPL> r;
+#pragma unroll
+              for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(yreg[u][i].e[j]) + out[j][i]);
+              store_y<T, CPL>(yrow[u][i] + c, r, nt);
+            }
           }
         }
       }
@@ -418,27 +458,33 @@ void launch_shrink_rank(const ShrinkLaunch& l, int kr) {
   }
 }
 
-template <typename T>
-void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, int big_cap, dim3 grid, int ksplit, int cpl, const ExpandSplits& sp) {
+template <typename T, int R>
+void launch_expand_group(const MloraAddArgs* a, const PlanLayout& lay, int big_units, dim3 grid, int ksplit, int cpl, int group,
+                         const ExpandSplits& sp) {
   hipStream_t st = static_cast<hipStream_t>(a->stream);
   const float* h = static_cast<const float*>(a->workspace);
   const int nt = env_int("MLORA_SGMV_NT_HINT", 0);
-#define MLORA_EXPAND(RR)                                                                                                     \
-  if (cpl == 4)                                                                                                              \
-    hipLaunchKernelGGL((sgmv_expand_kernel<T, RR, 4, 4>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y,          \
-                       a->y_stride, lay.big_off, lay.small_off, big_cap, lay.sorted_off, a->num_tokens, a->num_slots,        \
-                       a->num_slices, ksplit, a->scaling, nt, sp);                                                           \
-  else                                                                                                                       \
-    hipLaunchKernelGGL((sgmv_expand_kernel<T, RR, 8, 2>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, a->y_stride, \
-                     lay.big_off, lay.small_off, big_cap, lay.sorted_off, a->num_tokens, a->num_slots, a->num_slices, ksplit,    \
-                     a->scaling, nt, sp)
-  switch (a->r) {
-    case 8: MLORA_EXPAND(8); break;
-    case 16: MLORA_EXPAND(16); break;
-    case 32: MLORA_EXPAND(32); break;
-    default: MLORA_EXPAND(64); break;
+#define MLORA_EXPAND(CPL_, TPF_, G_)                                                                                       \
+  hipLaunchKernelGGL((sgmv_expand_kernel<T, R, CPL_, TPF_, G_>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, \
+                     a->y_stride, lay.big_off, lay.small_off, big_units, lay.sorted_off, a->num_tokens, a->num_slots,      \
+                     a->num_slices, ksplit, a->scaling, nt, sp)
+  if (cpl == 4) {
+    if (group == 4) MLORA_EXPAND(4, 4, 4); else if (group == 2) MLORA_EXPAND(4, 4, 2); else MLORA_EXPAND(4, 4, 1);
+  } else {
+    if (group == 4) MLORA_EXPAND(8, 2, 4); else if (group == 2) MLORA_EXPAND(8, 2, 2); else MLORA_EXPAND(8, 2, 1);
   }
 #undef MLORA_EXPAND
+}
+
+template <typename T>
+void launch_expand_rank(const MloraAddArgs* a, const PlanLayout& lay, int big_units, dim3 grid, int ksplit, int cpl, int group,
+                        const ExpandSplits& sp) {
+  switch (a->r) {
+    case 8: launch_expand_group<T, 8>(a, lay, big_units, grid, ksplit, cpl, group, sp); break;
+    case 16: launch_expand_group<T, 16>(a, lay, big_units, grid, ksplit, cpl, group, sp); break;
+    case 32: launch_expand_group<T, 32>(a, lay, big_units, grid, ksplit, cpl, group, sp); break;
+    default: launch_expand_group<T, 64>(a, lay, big_units, grid, ksplit, cpl, group, sp); break;
+  }
 }
 
 // Column ranges of about `nt` columns (a multiple of 512: four wavefronts of 128 columns).
@@ -542,19 +588,24 @@ int launch_sgmv(const MloraAddArgs* a) {
   int rc = check_launch("mlora_add_lora(sgmv shrink)");
   if (rc) return rc;
 
-  // expand: tiles x column ranges of about 2048 workgroups
+  // expand: consecutive tiles per workgroup (they share their B rows when they share their
+  // slot), then column ranges so that the grid has about 2048 workgroups
   ExpandSplits splits;
+  int group = env_int("MLORA_SGMV_GROUP", 0);
+  if (group != 1 && group != 2 && group != 4) group = (cols >= 4096 && est_tiles >= 64) ? 4 : 1;  // wide projections only: narrow ones need the workgroups
   const int target = env_int("MLORA_SGMV_WGS", 2048);
   int nt = env_int("MLORA_SGMV_NT", 0);
   if (nt <= 0) {
-    const long long want = static_cast<long long>(cols) * est_tiles / (target > 0 ? target : 1);
+    const long long want = static_cast<long long>(cols) * (est_tiles / group + 1) / (target > 0 ? target : 1);
     nt = want > 8192 ? 8192 : static_cast<int>(want);
   }
   const int nsplit = fill_splits(a, nt, splits.split);
   const int cpl = env_int("MLORA_SGMV_CPL", 8) == 4 ? 4 : 8;
-  dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(l.tiles8));
-  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, l.big_cap, grid, ksplit, cpl, splits);
-  else launch_expand_rank<_Float16>(a, l.lay, l.big_cap, grid, ksplit, cpl, splits);
+  const int big_units = l.big_cap / group;  // big_cap is a multiple of 32: a multiple of 8 again
+  const int units = big_units + (l.tiles8 * 8 - l.big_cap);
+  dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(units / 8));
+  if (a->dtype == MLORA_DTYPE_BF16) launch_expand_rank<__bf16>(a, l.lay, big_units, grid, ksplit, cpl, group, splits);
+  else launch_expand_rank<_Float16>(a, l.lay, big_units, grid, ksplit, cpl, group, splits);
   return check_launch("mlora_add_lora(sgmv expand)");
 }
 

@@ -561,7 +561,7 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     small_off = (offsets_off + r4(L + 2) + 31) & ~31
     cap_small = ((T + 15) // 16 + min(L, T) + 7) & ~7
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
-    coop_off = big_off + 4 * ((T // 64 + min(L, T) + 7) & ~7)
+    coop_off = big_off + 4 * ((T // 64 + min(L, T) + 31) & ~31)
     assert len(ws) == coop_off + 8 * cap_small
     assert ws[coop_off:] == [0] * (8 * cap_small)  # arrival counters rest at zero
     assert ws[sorted_off : sorted_off + len(s)] == s
