@@ -70,10 +70,13 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   const int beg = wave * span;
   const int end = beg + span < T ? beg + span : T;
 
+  // (the slot id of the next step is requested before the current one is counted)
+  int s_next = beg + lane < end ? p.tts[beg + lane] : -1;
   for (int base = beg; base < end; base += kWave) {
-    int t = base + lane;
+    const int t = base + lane;
+    const int s = s_next;
+    if (t + kWave < end) s_next = p.tts[t + kWave];
     if (t < end) {
-      int s = p.tts[t];
       int key = (s >= 0 && s < L) ? s + 1 : 0;
       if (s >= L) s_bad = 1;
       atomicAdd(&hist[wave * NB + key], 1);
@@ -224,42 +227,47 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   __syncthreads();
 
   // Stable scatter: every wave walks its span again in token order.  The rank of a token
-  // among the equal keys of its 64-token step comes from a ballot; the running cursor of
-  // (wave, key) lives in hist and is advanced once per distinct key per step.
+  // among the equal keys of its 64-token step is counted lane against lane; the running cursor
+  // of (wave, key) lives in hist and is advanced once per distinct key per step.
   int32_t* plan_sorted = p.plan ? p.plan + lay.sorted_off : nullptr;
-  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+  s_next = beg + lane < end ? p.tts[beg + lane] : -1;
   for (int base = beg; base < end; base += kWave) {
     const int t = base + lane;
+    const int s = s_next;
+    if (t + kWave < end) s_next = p.tts[t + kWave];
     int key = -1;
-    if (t < end) {
-      int s = p.tts[t];
-      key = (s >= 0 && s < L) ? s + 1 : 0;
-    }
+    if (t < end) key = (s >= 0 && s < L) ? s + 1 : 0;
     const bool take = key >= 1 || (key == 0 && p.no_lora_bucket && !reset_only);
-    uint64_t remaining = __ballot(take);
-    while (remaining) {
-      const int leader = __ffsll(static_cast<unsigned long long>(remaining)) - 1;
-      const int k = __shfl(key, leader, kWave);
-      const uint64_t group = __ballot(take && key == k);
-      int cursor = 0;
-      if (lane == leader) cursor = atomicAdd(&hist[wave * NB + k], __popcll(group));
-      cursor = __shfl(cursor, leader, kWave);
-      if (take && key == k) {
-        const int r = cursor + __popcll(group & lt_mask);
-        if (k >= 1) {
-          if (plan_sorted) {
-            plan_sorted[off[k] + r] = t;
-            const int c = total[k];
-            const int q = (c < MLORA_SEGMENT_THRESHOLD ? ts_short[k] : n_short + ts_long[k]) + r / MLORA_TILE_SMALL;
-            p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (r % MLORA_TILE_SMALL)] = t;
-          }
-          if (p.sorted_idx) p.sorted_idx[n_neg + off[k] + r] = t;
-        } else if (p.sorted_idx) {
-          p.sorted_idx[r] = t;
-        }
-      }
-      remaining &= ~group;
+    // Rank of this token among the equal keys of its 64-token step, and the size of that group:
+    // every lane compares its key with each lane's key in turn (a fixed 64 broadcasts, however
+    // many distinct keys the step holds).  Lanes that take no part get keys nobody else has.
+    const int mine = take ? key : -1 - lane;
+    int before = 0, group = 0;
+#pragma unroll
+    for (int j = 0; j < kWave; ++j) {
+      const int eq = __builtin_amdgcn_readlane(mine, j) == mine;
+      group += eq;
+      before += eq & int(j < lane);
     }
+    if (take) {
+      const int cursor = hist[wave * NB + key];
+      const int r = cursor + before;
+      if (key >= 1) {
+        if (plan_sorted) {
+          plan_sorted[off[key] + r] = t;
+          const int c = total[key];
+          const int q = (c < MLORA_SEGMENT_THRESHOLD ? ts_short[key] : n_short + ts_long[key]) + r / MLORA_TILE_SMALL;
+          p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (r % MLORA_TILE_SMALL)] = t;
+        }
+        if (p.sorted_idx) p.sorted_idx[n_neg + off[key] + r] = t;
+      } else if (p.sorted_idx) {
+        p.sorted_idx[r] = t;
+      }
+      // the last lane of a group moves the group's cursor on (one writer per key; the wavefront's
+      // LDS accesses execute in order, so the next step reads the new value)
+      if (before == group - 1) hist[wave * NB + key] = cursor + group;
+    }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
