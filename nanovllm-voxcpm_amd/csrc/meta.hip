@@ -231,6 +231,8 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   // of (wave, key) lives in hist and is advanced once per distinct key per step.
   int32_t* plan_sorted = p.plan ? p.plan + lay.sorted_off : nullptr;
   s_next = beg + lane < end ? p.tts[beg + lane] : -1;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+  const int key_bits = 32 - __builtin_clz(NB);  // keys are 0 .. NB - 1
   for (int base = beg; base < end; base += kWave) {
     const int t = base + lane;
     const int s = s_next;
@@ -239,16 +241,14 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
     if (t < end) key = (s >= 0 && s < L) ? s + 1 : 0;
     const bool take = key >= 1 || (key == 0 && p.no_lora_bucket && !reset_only);
     // Rank of this token among the equal keys of its 64-token step, and the size of that group:
-    // every lane compares its key with each lane's key in turn (a fixed 64 broadcasts, however
-    // many distinct keys the step holds).  Lanes that take no part get keys nobody else has.
-    const int mine = take ? key : -1 - lane;
-    int before = 0, group = 0;
-#pragma unroll
-    for (int j = 0; j < kWave; ++j) {
-      const int eq = __builtin_amdgcn_readlane(mine, j) == mine;
-      group += eq;
-      before += eq & int(j < lane);
+    // the set of lanes holding the same key is narrowed down one key bit at a time with ballots
+    // (a fixed handful of steps, however many distinct keys the step holds).
+    uint64_t peers = __ballot(take);
+    for (int bit = 0; bit < key_bits; ++bit) {
+      const uint64_t set = __ballot((key >> bit) & 1);
+      peers &= ((key >> bit) & 1) ? set : ~set;
     }
+    const int before = __popcll(peers & lt_mask), group = __popcll(peers);
     if (take) {
       const int cursor = hist[wave * NB + key];
       const int r = cursor + before;
