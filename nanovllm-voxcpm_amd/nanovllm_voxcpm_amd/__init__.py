@@ -6,6 +6,9 @@ Modules mirror the reference package paths they stand in for:
   layers.lora       the four LoRA-wrapped linears
   utils.context     per-domain LoRAContext and its on-device builder
   engine.lora_manager, engine.graph_meta   batch plan -> context, graph-buffer refresh
+  engine.lora_runtime   adapter lifecycle, reference counts, LRU slot residency
+  lora_checkpoint   checkpoint directory -> payloads -> resident slot
+  synthetic, backbone   seeded workloads and the synthetic decoder of the benchmark configurations
   _hip              ctypes binding of the C-ABI library (include/mlora.h)
 """
 

@@ -4,7 +4,8 @@ Counterpart of the index builders of the reference's ``nanovllm_voxcpm/engine/lo
 (:67-180).  The reference sorts the tokens by slot in Python for every step and domain
 (:77-91) and uploads five packed arrays (:118-176); here only the slot-id vector crosses PCIe
 (one pinned copy) and one launch of the on-device counting sort produces the rest.  The
-adapter lifecycle / LRU residency half of that file is host bookkeeping outside this path.
+adapter lifecycle / LRU residency half of that file lives in ``lora_runtime.py`` and is
+re-exported here under the reference's import path.
 """
 
 from __future__ import annotations
@@ -31,6 +32,24 @@ class LoRABatchPlan:
     @property
     def active_slot_ids(self) -> list[int]:
         return sorted({s for s in self.token_to_slot if s >= 0})
+
+    # The remaining host-side views of the reference's plan (lora_manager.py:67-91) are derived
+    # on demand; the device path never reads them (the GPU sorts the tokens itself).
+    @property
+    def num_tokens_per_slot(self) -> list[int]:
+        return [sum(1 for s in self.token_to_slot if s == slot) for slot in self.active_slot_ids]
+
+    @property
+    def slot_start_offsets(self) -> list[int]:
+        offsets = [0]
+        for count in self.num_tokens_per_slot:
+            offsets.append(offsets[-1] + count)
+        return offsets
+
+    @property
+    def token_indices_sorted_by_slot(self) -> list[int]:
+        keyed = [(s, t) for t, s in enumerate(self.token_to_slot) if s >= 0]
+        return [t for _, t in sorted(keyed)]
 
 
 def build_lora_batch_plan_from_token_to_slot(
@@ -107,3 +126,16 @@ def build_lora_context_from_slot_list(
     return build_lora_context_from_batch_plan(
         build_lora_batch_plan_from_token_to_slot({}, token_to_slot), max_slots=max_slots, device=device
     )
+
+
+from nanovllm_voxcpm_amd.engine.lora_runtime import (  # noqa: E402  (re-export under the reference's module path)
+    LoRAControlEntry,
+    LoRALifecycleState,
+    LoRAManager,
+    LoRAModelPayload,
+    LoRAModulePayload,
+    LoRAResidentState,
+    LoRARuntime,
+    LoRARuntimeEntry,
+    LoRASlot,
+)
