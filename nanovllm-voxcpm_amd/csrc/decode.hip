@@ -68,7 +68,15 @@ struct DecodeSplits {
 // exchanged words are written and read with device-scope atomic accesses, which are performed
 // at the level of the memory system that all compute units share, so no cache has to be
 // flushed.  The counter is back at zero when the launch ends.
-template <typename T, int R, int KSPW>
+//
+// TR (needs KSPW == 4): a compute unit's vector L1 handles a 128-bit load whose consecutive
+// lanes touch different rows (what the MFMA operand layout asks for) at about a quarter of the
+// rate of one whose lanes walk along a row, and even cache-resident operands showed up as
+// 3-4 us per launch.  With TR the x rows and A rows of a wavefront's K range are fetched
+// row-contiguously (sixteen lanes per 256 bytes of a row) and turned into operand layout through
+// a private LDS block per wavefront, and the expand runs with the tokens as MFMA rows, so that
+// sixteen consecutive lanes cover 128 contiguous bytes of one y row.
+template <typename T, int R, int KSPW, bool TR>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
@@ -84,6 +92,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
   __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
   __shared__ int s_arrived;
+  constexpr int kStageRow = 17;  // 16 chunks of 16 bytes + one of padding: operand reads hit every bank once
+  __shared__ __attribute__((aligned(16))) i32x4 s_stage[TR ? kNW * (1 + RB) * 16 * kStageRow : 1];
+  static_assert(!TR || KSPW == 4, "the staged form covers four k-steps per wavefront");
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
@@ -98,6 +109,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // ---- round trip 1 ---------------------------------------------------------------------------
   const int32_t* rec = plan + small_off + tile * MLORA_SMALL_TILE_WORDS;  // tile < capacity: in bounds
   const int row = rec[MLORA_SMALL_TILE_ROWS + lr];
+  const i32x4 rows4 = *reinterpret_cast<const i32x4*>(rec + MLORA_SMALL_TILE_ROWS + 4 * lg);  // tokens 4*lg .. 4*lg+3
   const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);       // slot, count, start, 0
   const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);      // magic, T, L, ...
   const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
@@ -131,35 +143,73 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   const int ks0 = kpart * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
   const int ks1 = KSPW > 0 ? ks0 + KSPW : kpart * nks + (wave + 1) * nks / kNW;
   Pack8 xa[CH], aw[RB][CH];
+  i32x4 xst[TR ? 4 : 1], ast[TR ? RB : 1][TR ? 4 : 1];
+  if constexpr (TR) {
+    // row-contiguous: lane = (row group lane/16, 16-byte chunk lane%16 of the 256-byte K range)
+    const int64_t koff = static_cast<int64_t>(ks0) * 32 + (lane & 15) * 8;
 #pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int ks = ks0 + i;
-    if (KSPW > 0 || ks < ks1) {
-      xa[i].raw = load128(xrow + ks * 32);  // absent tokens read row 0; their results are never stored
+    for (int i = 0; i < 4; ++i) {
+      xst[i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = load128(arow[rb] + ks * 32);
+      for (int rb = 0; rb < RB; ++rb) {
+        const int rr = rb * 16 + 4 * lg + i;
+        ast[rb][i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int ks = ks0 + i;
+      if (KSPW > 0 || ks < ks1) {
+        xa[i].raw = load128(xrow + ks * 32);  // absent tokens read row 0; their results are never stored
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = load128(arow[rb] + ks * 32);
+      }
     }
   }
   Pack8 bop[kSpansAhead][4][KSTEPS], yreg[kSpansAhead][2];
+  uint2 yq[TR ? kSpansAhead : 1][TR ? 4 : 1];  // TR: four columns of four tokens per lane and span
+  T* const ycols = static_cast<T*>(yv_) + sp.y_col;
+  // TR span: MFMA j takes column c0 + 4 * (lane % 16) + j, so a lane ends up with four consecutive
+  // columns of tokens 4 * (lane / 16) .. + 3
+  auto load_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int n = c0 + 4 * lr + j;
+      n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = (lg + 4 * ks) & (R / 8 - 1);
+        bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+      }
+    }
+    const int c = c0 + 4 * lr < sp.n1 ? c0 + 4 * lr : sp.n1 - 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) yy[i] = *reinterpret_cast<const uint2*>(ycols + static_cast<int64_t>(rows4[i]) * ys + c);
+  };
 #pragma unroll
   for (int s = 0; s < kSpansAhead; ++s) {
     const int c0 = sp.n0 + (wave + s * kNW) * 64;
     if (c0 < sp.n1) {
+      if constexpr (TR) {
+        load_span_tr(c0, bop[s], yq[s]);
+      } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
-        n = n < sp.n1 ? n : sp.n1 - 1;
+        for (int j = 0; j < 4; ++j) {
+          int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
+          n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          // lanes whose chunk lies beyond the rank fetch a valid chunk anyway: their H operand is
-          // zero, and an unconditional load keeps the whole batch of loads in flight together
-          const int kc = (lg + 4 * ks) & (R / 8 - 1);
-          bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            // lanes whose chunk lies beyond the rank fetch a valid chunk anyway: their H operand is
+            // zero, and an unconditional load keeps the whole batch of loads in flight together
+            const int kc = (lg + 4 * ks) & (R / 8 - 1);
+            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          }
         }
-      }
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-        if (live && c0 + 16 * lg + 8 * half < sp.n1) yreg[s][half].raw = load128(yrow + c0 + 8 * half);
+        for (int half = 0; half < 2; ++half)
+          if (live && c0 + 16 * lg + 8 * half < sp.n1) yreg[s][half].raw = load128(yrow + c0 + 8 * half);
+      }
     }
   }
 
@@ -167,6 +217,24 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   f32x4 acc[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if constexpr (TR) {
+    // through the wavefront's LDS block: written row-contiguously, read in operand layout
+    // (k-step i of lane group g is chunk 4 * i + g, the same elements the direct loads take)
+    i32x4* stage = s_stage + wave * (1 + RB) * 16 * kStageRow;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[i];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) stage[((1 + rb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = ast[rb][i];
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = stage[((1 + rb) * 16 + lr) * kStageRow + 4 * i + lg];
+    }
+  }
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     if (KSPW > 0 || ks0 + i < ks1) {
@@ -366,43 +434,78 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       }
     }
   };
+  // tokens as MFMA rows: lane holds out[token 4 * lg + i][column c0 + 4 * lr + j]
+  auto finish_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
+    f32x4 out[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        out[j] = Mma<T>::run(hlo[ks], bo[j][ks], out[j]);
+        out[j] = Mma<T>::run(hop[ks], bo[j][ks], out[j]);
+      }
+    }
+    const int c = c0 + 4 * lr;
+    if (c < sp.n1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (4 * lg + i < m) {
+          union { uint2 raw; T e[4]; } v;
+          v.raw = yy[i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v.e[j] = from_f32<T>(to_f32(v.e[j]) + out[j][i]);
+          *reinterpret_cast<uint2*>(ycols + static_cast<int64_t>(rows4[i]) * ys + c) = v.raw;
+        }
+      }
+    }
+  };
 
 #pragma unroll
   for (int s = 0; s < kSpansAhead; ++s) {
     const int c0 = sp.n0 + (wave + s * kNW) * 64;
-    if (c0 < sp.n1) finish_span(c0, bop[s], yreg[s]);
+    if (c0 < sp.n1) {
+      if constexpr (TR) finish_span_tr(c0, bop[s], yq[s]);
+      else finish_span(c0, bop[s], yreg[s]);
+    }
   }
   for (int c0 = sp.n0 + (wave + kSpansAhead * kNW) * 64; c0 < sp.n1; c0 += kNW * 64) {  // wide ranges
     Pack8 bo[4][KSTEPS], yy[2];
+    if constexpr (TR) {
+      uint2 yt[4];
+      load_span_tr(c0, bo, yt);
+      finish_span_tr(c0, bo, yt);
+    } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
-      n = n < sp.n1 ? n : sp.n1 - 1;
+      for (int j = 0; j < 4; ++j) {
+        int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
+        n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = (lg + 4 * ks) & (R / 8 - 1);
-        bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = (lg + 4 * ks) & (R / 8 - 1);
+          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        }
       }
-    }
 #pragma unroll
-    for (int half = 0; half < 2; ++half)
-      if (live && c0 + 16 * lg + 8 * half < sp.n1) yy[half].raw = load128(yrow + c0 + 8 * half);
-    finish_span(c0, bo, yy);
+      for (int half = 0; half < 2; ++half)
+        if (live && c0 + 16 * lg + 8 * half < sp.n1) yy[half].raw = load128(yrow + c0 + 8 * half);
+      finish_span(c0, bo, yy);
+    }
   }
 }
 
 struct Launch {
   const MloraAddArgs* a;
-  int small_off, include_long, kshift, mode, spin_ticks;
+  int small_off, include_long, kshift, mode, spin_ticks, staged;
   int32_t* counters;
   dim3 grid;
   const DecodeSplits* splits;
 };
 
-template <typename T, int R, int KSPW>
+template <typename T, int R, int KSPW, bool TR = false>
 void launch_one(const Launch& l) {
   const MloraAddArgs* a = l.a;
-  hipLaunchKernelGGL((decode_kernel<T, R, KSPW>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+  hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
                      a->num_slots, a->scaling, l.kshift, l.mode, l.spin_ticks, l.counters, static_cast<float*>(a->workspace),
                      *l.splits);
@@ -412,7 +515,13 @@ void launch_one(const Launch& l) {
 // for every rank and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
-  if (kspw == 4) return launch_one<T, R, 4>(l);
+  if (kspw == 4) {
+    // staged operands: LDS for the A rows of ranks up to 32 (rank 64 would need 174 KB)
+    if constexpr (R <= 32) {
+      if (l.staged) return launch_one<T, R, 4, true>(l);
+    }
+    return launch_one<T, R, 4>(l);
+  }
   if (kspw == 2) return launch_one<T, R, 2>(l);
   if (kspw == 1) return launch_one<T, R, 1>(l);
   if constexpr (R <= 16) {
@@ -473,6 +582,7 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
   l.spin_ticks = env_int("MLORA_DECODE_SPIN_TICKS", 20000);  // 200 us of the 100 MHz clock
   l.kshift = 0;
   l.mode = 0;
+  l.staged = env_int("MLORA_DECODE_STAGED", 1);
   int total = 0;
 
   // Mode 2: the workgroups of a (tile, slice) each take one part of K and one part of the columns.
@@ -503,10 +613,23 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
     }
   }
   if (l.mode == 0) {
-    // Column range per workgroup: every range repeats the shrink of its tile, so ranges are kept
-    // wide enough (default 1024 columns: two 64-column spans per wavefront) for the expand to
-    // outweigh that repeat.
-    int nt = env_int("MLORA_DECODE_NT", 1024);
+    // Column range per workgroup.  Every range repeats the shrink of its tile, but a compute unit
+    // takes in only 30-60 bytes per cycle even from the L2, so a launch is fastest when its
+    // bytes are spread over 150-250 workgroups: ranges shrink down to 128 columns for narrow
+    // projections and stay at 1024 (two 64-column spans per wavefront, all loads still in
+    // registers) for wide ones.  Measured per launch at 32 tiles: o 6.2 us at 1024 columns,
+    // 5.1 at 512, 4.7 at 256; gate_up 8.2 / 8.9 / 11.1.
+    int nt = env_int("MLORA_DECODE_NT", 0);
+    if (nt <= 0) {
+      long long cols = 0;
+      for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+      const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
+      const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
+      const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
+      nt = static_cast<int>(cols * tiles / 160);
+      if (nt > 1024) nt = 1024;
+      if (nt < 128) nt = 128;
+    }
     if (nt < 64) nt = 64;
     nt = (nt + 63) & ~63;
     for (;;) {
