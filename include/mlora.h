@@ -36,8 +36,8 @@ extern "C" {
 #define MLORA_FORM_AUTO 0  /* library chooses from shapes and the plan */
 #define MLORA_FORM_TOKEN 1 /* one workgroup per token, any shape or dtype; needs no plan */
 #define MLORA_FORM_BGMV 2  /* small tiles (<= 16 tokens of one slot), packed dot2 + wave64 reductions */
-#define MLORA_FORM_SGMV 3  /* 64-token MFMA tiles for segments >= threshold (shrink launch + expand launch through
-                              the workspace), small MFMA tiles for the rest */
+#define MLORA_FORM_SGMV 3  /* shrink launch + expand launch through the workspace: 64-token MFMA tiles for
+                              segments >= threshold, one short tile each for the rest */
 #define MLORA_FORM_MFMA 4  /* small tiles for every segment, both products on the matrix cores */
 
 /* error codes (negative) */

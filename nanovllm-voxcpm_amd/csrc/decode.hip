@@ -1,22 +1,24 @@
 // Small-tile form: one workgroup per (small tile, slice, column range).  A small tile is up
 // to sixteen tokens of one slot, described by a self-contained 128-byte record.
 //
-// A launch of this size (a few MB) is bound by memory latency, not bandwidth, so the kernel
-// is built around the number of dependent round trips to memory:
+// A launch of this size (a few MB) is bound by fixed latencies and by how fast one compute
+// unit takes data in (about 20 bytes per cycle, cache-resident or not), not by HBM bandwidth,
+// so the kernel is built around the number of dependent round trips to memory and the launch
+// around the number of workgroups:
 //   0. the scalar launch arguments arrive preloaded in SGPRs (the kernel takes them as plain
 //      leading arguments for that purpose), so no fetch of the argument block comes first;
-//   1. the plan header, the tile record, this lane's token index and the column-range entry
-//      are fetched together — their addresses depend on nothing but the workgroup index — and
-//      one branch-free test decides whether the workgroup has work;
+//   1. the plan header, the tile record, the token indices and the column-range entry are
+//      fetched together — their addresses depend on nothing but the workgroup index — and one
+//      branch-free test decides whether the workgroup has work;
 //   2. every global load the workgroup needs — its K-range of the x rows and of A[slot], the
-//      B[slot] rows and the y rows of its output spans — is issued before any arithmetic.
+//      B[slot] rows and the y rows of its output spans — is issued before any arithmetic;
+//   3. column ranges are sized on the host so that a launch spreads over 150-250 workgroups.
 // Both products run on the matrix cores (v_mfma_f32_16x16x32, fp32 accumulate): the sixteen
-// token rows are the MFMA's N (shrink: M) dimension, so a half-empty tile costs nothing but
-// idle multiplier lanes.  The eight wavefronts split K for the shrink, sum their partial tiles
-// through LDS, keep the rank-r intermediate there as a hi + lo pair of operand-precision
-// values, and then each take 64-column spans of the expand; the B rows of a span are
-// interleaved across its four MFMAs so that a lane owns 16 consecutive columns of one token
-// and y is updated with 128-bit accesses.
+// token rows are one MFMA dimension, so a half-empty tile costs nothing but idle multiplier
+// lanes.  The eight wavefronts split K for the shrink, sum their partial tiles through LDS,
+// keep the rank-r intermediate there as a hi + lo pair of operand-precision values, and then
+// each take 64-column spans of the expand; the B rows of a span are interleaved across its
+// four MFMAs so that a lane owns consecutive columns and y is updated with wide accesses.
 #include "common.h"
 #include "launch.h"
 

@@ -1,28 +1,31 @@
-// SGMV form for the 64-token tiles of long segments: two launches that meet in a small
-// workspace, both on the matrix cores (v_mfma_f32_16x16x32 bf16 / f16, fp32 accumulate).
+// SGMV form for batches above the small-batch limit: two launches that meet in a small
+// workspace, both on the matrix cores (v_mfma_f32_16x16x32 bf16 / f16, fp32 accumulate).  Work
+// units are the 64-token tiles of the long segments and, behind them in the same grids, the
+// short segments (one small-tile record each).
 //
 //   shrink — H^T[rank x tokens] = A[slot] . X_tile^T for a (tile, slice, K part).  What bounds
-//            this product is the number of bytes a compute unit pulls through its vector L1
-//            (hits cost as much as misses there), so each operand element passes through it once
-//            per workgroup: the A[slot] slab of the workgroup's K part is copied to LDS with
-//            row-contiguous 128-bit loads and shared by the four wavefronts, each of which owns
-//            sixteen tokens of the tile and streams their x rows straight from global memory
-//            into the MFMA operand layout, a whole batch of k-steps in flight at a time.  No
-//            wavefront shares a sum with another, so the accumulators go straight to the
+//            this product is the number of bytes a compute unit takes in (cache hits cost about
+//            as much as misses: the limit is requests in flight), so each operand element is
+//            fetched once per workgroup: the A[slot] slab of the workgroup's K part is copied to
+//            LDS with row-contiguous 128-bit loads and shared by the four wavefronts, each of
+//            which owns sixteen tokens of the tile and streams their x rows straight from global
+//            memory into the MFMA operand layout, a whole batch of k-steps in flight at a time.
+//            No wavefront shares a sum with another, so the accumulators go straight to the
 //            workspace as fp32; when K is split across workgroups each part writes its own
-//            partial.  x is read from HBM once per slice.
-//   expand — OUT^T[cols x tokens] = B[slot] . H^T for a (tile, column range).  The H tile is
-//            staged in LDS once (K partials summed, scaled, and split into a hi + lo pair of
-//            operand-precision values, about 16 significant bits: the expand loses nothing that
-//            would show after the final rounding of y); a wavefront owns 64-column spans: it
-//            fetches the span's B rows and the y rows of all four 16-token blocks up front, then
-//            runs the MFMAs block by block and writes y back.  The B rows fed to the four MFMAs
-//            of a span are interleaved (row rho of MFMA j is column 16*(rho/4) + 4j + rho%4) so
-//            that a lane ends up with 16 consecutive output columns of one token: y moves in
-//            128-bit accesses, a full 128-byte line per token per wavefront, with no
-//            transposition pass.
+//            partial.  For three or more slices one workgroup walks all of them with the x rows
+//            it holds.
+//   expand — OUT[tokens x cols] = H . B[slot]^T for a (group of tiles, column range).  The H
+//            tiles are staged in LDS once (K partials summed, scaled, and split into a hi + lo
+//            pair of operand-precision values, about 16 significant bits: the expand loses
+//            nothing that would show after the final rounding of y).  A wavefront owns spans of
+//            64 or 128 columns: it fetches the span's B rows once per slot, then for every tile
+//            of the group the y rows of two or four 16-token blocks at a time, runs the MFMAs
+//            and writes y back.  Tokens are the MFMA rows and the B rows fed to the MFMAs of a
+//            span are interleaved, so a lane ends up with consecutive output columns of four
+//            tokens and sixteen consecutive lanes cover a contiguous piece of one y row: y moves
+//            in fully coalesced accesses with no transposition pass.
 // Splitting the two products means no column range repeats the shrink of its tile, and each
-// kernel keeps only its own operands in registers (more wavefronts per SIMD to hide latency).
+// kernel keeps only its own operands in registers.
 #include "common.h"
 #include "launch.h"
 
