@@ -42,6 +42,22 @@ template <> struct Mma<_Float16> {
   }
 };
 
+// 16x16x16 variant (four operand elements per lane): for rank 16 the contraction of the
+// expand is exactly sixteen long, so no lane fetches B elements it would multiply by zero.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+template <typename T> struct Mma16;
+template <> struct Mma16<__bf16> {
+  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<_Float16> {
+  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h16x4, a), __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
+  }
+};
+
 struct DecodeSplit {
   const void* a;
   const void* b;
@@ -174,15 +190,21 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   T* const ycols = static_cast<T*>(yv_) + sp.y_col;
   // TR span: MFMA j takes column c0 + 4 * (lane % 16) + j, so a lane ends up with four consecutive
   // columns of tokens 4 * (lane / 16) .. + 3
+  constexpr bool K16 = TR && R == 16;  // expand on the 16x16x16 MFMA: 64-bit operand pieces
   auto load_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int n = c0 + 4 * lr + j;
       n = n < sp.n1 ? n : sp.n1 - 1;
+      if constexpr (K16) {
+        const uint2 piece = *reinterpret_cast<const uint2*>(B + static_cast<int64_t>(n) * R + 4 * lg);  // ranks 4*lg .. 4*lg+3
+        bo[j][0].raw = i32x4{static_cast<int>(piece.x), static_cast<int>(piece.y), 0, 0};
+      } else {
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = (lg + 4 * ks) & (R / 8 - 1);
-        bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = (lg + 4 * ks) & (R / 8 - 1);
+          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        }
       }
     }
     const int c = c0 + 4 * lr < sp.n1 ? c0 + 4 * lr : sp.n1 - 4;
@@ -437,15 +459,26 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     }
   };
   // tokens as MFMA rows: lane holds out[token 4 * lg + i][column c0 + 4 * lr + j]
+  uint2 hop16 = {0, 0}, hlo16 = {0, 0};
+  if constexpr (K16) {
+    hop16 = *reinterpret_cast<const uint2*>(&s_hi[lr * HSTRIDE + 4 * lg]);
+    hlo16 = *reinterpret_cast<const uint2*>(&s_lo[lr * HSTRIDE + 4 * lg]);
+  }
   auto finish_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
     f32x4 out[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (K16) {
+        const uint2 piece = {static_cast<uint32_t>(bo[j][0].raw[0]), static_cast<uint32_t>(bo[j][0].raw[1])};
+        out[j] = Mma16<T>::run(hlo16, piece, out[j]);
+        out[j] = Mma16<T>::run(hop16, piece, out[j]);
+      } else {
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        out[j] = Mma<T>::run(hlo[ks], bo[j][ks], out[j]);
-        out[j] = Mma<T>::run(hop[ks], bo[j][ks], out[j]);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          out[j] = Mma<T>::run(hlo[ks], bo[j][ks], out[j]);
+          out[j] = Mma<T>::run(hop[ks], bo[j][ks], out[j]);
+        }
       }
     }
     const int c = c0 + 4 * lr;
