@@ -40,6 +40,9 @@ using namespace mlora;
 
 namespace {
 
+// Both matrix-core forms step through K in units of 32.
+bool mfma_supported(const MloraAddArgs* a) { return a->k % 32 == 0 && a->k >= 32; }
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // The vectorised kernels move eight 16-bit elements per lane: every row they touch has to
@@ -93,11 +96,11 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
     // tiles for the long segments and 16-token tiles for the rest.
     if (!vec) form = MLORA_FORM_TOKEN;
-    else if (!sgmv_supported(a)) form = MLORA_FORM_BGMV;
-    else if (a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
+    else if (!mfma_supported(a)) form = MLORA_FORM_BGMV;
+    else if (a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) || !sgmv_supported(a) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
     else form = MLORA_FORM_SGMV;
   }
-  if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && vec && sgmv_supported(a) && !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
+  if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && vec && mfma_supported(a) && !(sgmv_supported(a) && sgmv_workspace_ok(a))) form = MLORA_FORM_MFMA;
   switch (form) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
@@ -106,8 +109,9 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
       return launch_bgmv(a, /*include_long=*/true);
     case MLORA_FORM_SGMV:
     case MLORA_FORM_MFMA: {
-      if (!vec || !sgmv_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
+      if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
+      if (!sgmv_supported(a)) { set_error("mlora_add_lora: SGMV form needs K %% 128 == 0"); return MLORA_E_UNSUPPORTED; }
       if (!sgmv_workspace_ok(a)) {
         set_error("mlora_add_lora: SGMV form needs a 16-byte aligned workspace of %zu bytes and no empty slice",
                   sgmv_workspace_bytes(a->num_tokens, a->num_slices, a->r, a->dtype));

@@ -209,6 +209,35 @@ def test_ranks_and_dtypes_small(rank, dtype, form):
     _check(got, y0, exact, mag, slots, f"rank{rank}/{dtype}/{form}")
 
 
+@pytest.mark.parametrize("staged", ["1", "0"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [8, 16, 32, 64])
+def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
+    """The small-tile kernel at the K values that select its specialisations (1024: four k-steps
+    per wavefront, staged operands for ranks up to 32; 4096: K shared between workgroups; 512 and
+    160: two k-steps / run-time split), with ragged slice widths, narrow and wide column ranges,
+    row-strided x and y views, rows without adapter and a segment longer than one tile."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"small tiles r={rank} {dtype} staged={staged}", flush=True)
+    monkeypatch.setenv("MLORA_DECODE_STAGED", staged)
+    shapes = {"a": (1024, [72, 200, 8]), "b": (4096, [328]), "c": (512, [1096, 64]), "d": (160, [24])}
+    g = torch.Generator().manual_seed(40 + rank)
+    T = 77
+    slots = torch.randint(-1, 9, (T,), generator=g, dtype=torch.int32)
+    slots[5:30] = 4
+    slots = slots.cuda()
+    for name in shapes:
+        proj = synthetic.make_projection(name, 9, rank, dtype, seed=950 + rank, device="cuda", shapes=shapes)
+        xw, yw = synthetic.make_activations(T, proj.k + 16, sum(proj.widths) + 24, dtype, seed=951, device="cuda")
+        x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 8 : 8 + sum(proj.widths)]
+        y = yw.clone()[:, 8 : 8 + sum(proj.widths)]
+        got = _apply("mfma", proj, x, y, slots, scaling=1.25)
+        exact, mag = _exact(proj, x, y0, slots, scaling=1.25)
+        _check(got, y0, exact, mag, slots, f"small/{name}/r{rank}/{dtype}/staged{staged}")
+        assert torch.equal(y._base[:, :8], yw[:, :8]) and torch.equal(y._base[:, 8 + sum(proj.widths):], yw[:, 8 + sum(proj.widths):])
+
+
 @pytest.mark.parametrize("form", ["auto", "token"])
 def test_odd_shapes_take_the_scalar_path(form):
     """K, widths and rank that are not multiples of eight, unaligned column offsets, fp32."""
@@ -251,6 +280,37 @@ def test_config3_prefill_bf16(name, form):
     got = _apply(form, proj, x, y0.clone(), slots)
     exact, mag = _exact(proj, x, y0, slots)
     _check(got, y0, exact, mag, slots, f"config3/{name}/{form}")
+
+
+@pytest.mark.parametrize("knobs", [{}, {"MLORA_SGMV_KSPLIT": "1", "MLORA_SGMV_GROUP": "2"}, {"MLORA_SGMV_KR": "128", "MLORA_SGMV_KSPLIT": "4", "MLORA_SGMV_GROUP": "4", "MLORA_SGMV_CPL": "4"},
+                                   {"MLORA_SGMV_ALL_SLICES": "2", "MLORA_SGMV_KR": "256", "MLORA_SGMV_NT": "512"}])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [8, 16, 32, 64])
+def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
+    """The two-launch form on segments of 1..130 tokens (short ones, exact tile multiples, tails),
+    rows without adapter, ragged slice widths (not multiples of a span), row-strided x and y
+    views, every rank and both 16-bit types, and the launch shapes the knobs select (K parts,
+    slab width, tile groups, span width, slice walk)."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"long form r={rank} {dtype} {knobs}", flush=True)
+    for key, value in knobs.items():
+        monkeypatch.setenv(key, value)
+    shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520])}
+    lengths = [130, 1, 64, 15, 16, 65, 3, 128, 17, 7]
+    slot_of = [2, 0, 5, 1, 3, -1, 4, 2, -1, 6]  # slot 2 twice: two segments merge into one of 258
+    slots = torch.cat([torch.full((n,), s, dtype=torch.int32) for n, s in zip(lengths, slot_of)])
+    slots = slots[torch.randperm(slots.numel(), generator=torch.Generator().manual_seed(9))].cuda()
+    T = slots.numel()
+    for name in ("p", "q"):
+        proj = synthetic.make_projection(name, 7, rank, dtype, seed=900 + rank, device="cuda", shapes=shapes)
+        xw, yw = synthetic.make_activations(T, proj.k + 24, sum(proj.widths) + 40, dtype, seed=901, device="cuda")
+        x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 16 : 16 + sum(proj.widths)]  # 16-byte aligned views of wider buffers
+        y = yw.clone()[:, 16 : 16 + sum(proj.widths)]
+        got = _apply("sgmv", proj, x, y, slots, scaling=0.75)
+        exact, mag = _exact(proj, x, y0, slots, scaling=0.75)
+        _check(got, y0, exact, mag, slots, f"long/{name}/r{rank}/{dtype}/{knobs}")
+        assert torch.equal(y._base[:, :16], yw[:, :16]) and torch.equal(y._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
 
 
 # ---- config 4: mixed batch, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity ----
