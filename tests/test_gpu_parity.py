@@ -709,3 +709,52 @@ def test_graph_capture_replays_follow_new_slots_inputs_and_weights():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_buf, want), f"replay {step} differs from eager"
+
+
+@pytest.mark.parametrize("name,tokens,rank", [("down", 256, 16), ("gate_up", 1500, 64), ("down", 1500, 32)])
+def test_graph_replays_of_the_shared_and_the_two_launch_forms(name, tokens, rank):
+    """Backend call captured once (K = 4096 at decode size: workgroups exchanging partial sums
+    through the scratch and the plan's counters; 1500 tokens: the two-launch form with its scratch
+    allocated inside the capture) and replayed with new activations, base outputs and slot ids in
+    the same buffers; every replay is checked against the fp64 evaluation and against an eager
+    call on the same inputs, with eager work and synchronisations between the replays."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"graph {name} T={tokens} r={rank}", flush=True)
+    slots_n = 8
+    proj = _make(name, slots_n, rank, torch.bfloat16, seed=600 + rank)
+    x_buf = torch.zeros(tokens, proj.k, dtype=torch.bfloat16, device="cuda")
+    y_buf = torch.zeros(tokens, sum(proj.widths), dtype=torch.bfloat16, device="cuda")
+    s_buf = torch.zeros(tokens, dtype=torch.int32, device="cuda")
+    backend = _backend()
+    blocks = list(y_buf.split(proj.widths, dim=-1))
+    packed = y_buf if len(blocks) > 1 else None
+
+    def call(meta):
+        backend.add_lora(blocks, x_buf, proj.a, proj.b, indices=s_buf, metadata=meta, scaling=1.0, y_packed=packed)
+
+    call(_metadata(s_buf))  # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(_metadata(s_buf))  # a fresh metadata object: the plan launch is part of the graph
+
+    g = torch.Generator().manual_seed(61)
+    for step in range(4):
+        x, y0 = synthetic.make_activations(tokens, proj.k, sum(proj.widths), torch.bfloat16, seed=610 + step, device="cuda")
+        if tokens <= 1024:
+            slots = torch.randint(-1, slots_n, (tokens,), generator=g, dtype=torch.int32)
+        else:
+            slots, _ = synthetic.prefill_slots(12, slots_n, seed=620 + step, min_len=40, max_len=200)
+            slots = torch.nn.functional.pad(slots, (0, max(0, tokens - slots.numel())), value=-1)[:tokens]
+        slots = slots.cuda()
+        x_buf.copy_(x); y_buf.copy_(y0); s_buf.copy_(slots)
+        call(_metadata(s_buf))  # eager call on the same buffers
+        eager = y_buf.clone()
+        torch.cuda.synchronize()
+        y_buf.copy_(y0)
+        graph.replay()
+        torch.cuda.synchronize()
+        exact, mag = _exact(proj, x, y0, slots)
+        _check(y_buf, y0, exact, mag, slots, f"graph/{name}/T{tokens}/step{step}")
+        assert torch.equal(y_buf, eager), f"replay {step} differs from the eager call"
