@@ -177,15 +177,33 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
             views = list(y.split(proj.widths, dim=-1))
             oracle.per_token_add_lora(views, x, a, b, indices=slots_cpu, scaling=1.0, y_packed=y)
 
-    one_layer()  # warm-up
-    times = []
-    t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
-        t0 = time.perf_counter()
-        one_layer()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    def timed(fn, budget):
+        fn()  # warm-up
+        samples = []
+        t_end = time.perf_counter() + budget
+        while len(samples) < 3 or (time.perf_counter() < t_end and len(samples) < 20):
+            t0 = time.perf_counter()
+            fn()
+            samples.append(time.perf_counter() - t0)
+        samples.sort()
+        return samples[len(samples) // 2], len(samples)
+
+    med, runs = timed(one_layer, budget_s * 0.5)
+    times = [0.0] * runs
+
+    # two more views of the same layer, a few seconds each: the loop on one thread, and the
+    # vectorised restatement (gather + two batched matmuls per slice) on all threads
+    def one_layer_vectorised():
+        for proj, x, y, a, b in work:
+            for a_i, b_i in zip(a, b):
+                oracle.fused_delta(x, a_i, b_i, slots_cpu, 1.0)
+
+    vec_med, _ = timed(one_layer_vectorised, budget_s * 0.2)
+    torch.set_num_threads(1)
+    try:
+        one_med, _ = timed(one_layer, budget_s * 0.3)
+    finally:
+        torch.set_num_threads(threads)
     model = ""
     try:
         for line in Path("/proc/cpuinfo").read_text().splitlines():
@@ -202,6 +220,8 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
         "sample": f"1 of {NUM_LAYERS} layers of the same step (4 projections, {num_tokens} tokens, rank {rank}), fp32, "
                   f"per-token torch loop, median of {len(times)} runs",
         "us_per_layer": round(med * 1e6, 1),
+        "variants_us_per_layer": {"per_token_loop_1_thread": round(one_med * 1e6, 1),
+                                  f"gather_bmm_{threads}_threads": round(vec_med * 1e6, 1)},
         "us_per_step_extrapolated": round(med * 1e6 * NUM_LAYERS, 1),
         "cpu_model": model,
         "host_cpus": os.cpu_count(),
