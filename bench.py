@@ -410,7 +410,7 @@ def main() -> None:
             # HBM bytes per average launch from the two rocprofv3 --pmc runs of the default workload
             # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 256 MiB copy in the same runs);
             # only quoted for the configuration those runs covered
-            "traffic": 9824051 if default_run else None,
+            "traffic": 9823027 if default_run else None,
             "bytes_per_launch": round(launch_bytes),
             "us_per_launch": round(launch_us, 3),
         },
