@@ -192,14 +192,21 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // columns of tokens 4 * (lane / 16) .. + 3
   constexpr bool K16 = TR && R == 16;  // expand on the 16x16x16 MFMA: 64-bit operand pieces
   auto load_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
+    if constexpr (K16) {
+      // A span's 64 B rows of 32 bytes are 2 KB of contiguous memory: fetched as such (lane l takes
+      // 16 bytes of row c0 + l / 2 and of row c0 + 32 + l / 2, eight cache lines per instruction
+      // instead of sixteen quarter-used ones); finish_span_tr turns them into operand pieces.
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int n = c0 + 4 * lr + j;
-      n = n < sp.n1 ? n : sp.n1 - 1;
-      if constexpr (K16) {
-        const uint2 piece = *reinterpret_cast<const uint2*>(B + static_cast<int64_t>(n) * R + 4 * lg);  // ranks 4*lg .. 4*lg+3
-        bo[j][0].raw = i32x4{static_cast<int>(piece.x), static_cast<int>(piece.y), 0, 0};
-      } else {
+      for (int h = 0; h < 2; ++h) {
+        int n = c0 + 32 * h + (lane >> 1);
+        n = n < sp.n1 ? n : sp.n1 - 1;
+        bo[h][0].raw = load128(B + static_cast<int64_t>(n) * R + (lane & 1) * 8);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int n = c0 + 4 * lr + j;
+        n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
@@ -466,11 +473,24 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   }
   auto finish_span_tr = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
     f32x4 out[4];
+    uint2 pieces[4];
+    if constexpr (K16) {
+      // B rows -> operand pieces through the wavefront's LDS block: four rows (128 bytes) per
+      // group, groups 144 bytes apart so that the sixteen lanes of a piece read hit every bank
+      // once.  MFMA j of lane (lr, lg) takes ranks 4*lg .. 4*lg+3 of column c0 + 4*lr + j.
+      char* blk = reinterpret_cast<char*>(s_stage + wave * (1 + RB) * 16 * kStageRow);
+      *reinterpret_cast<i32x4*>(blk + (lane >> 3) * 144 + (lane & 7) * 16) = bo[0][0].raw;
+      *reinterpret_cast<i32x4*>(blk + ((lane >> 3) + 8) * 144 + (lane & 7) * 16) = bo[1][0].raw;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pieces[j] = *reinterpret_cast<const uint2*>(blk + lr * 144 + j * 32 + lg * 8);
+      __builtin_amdgcn_wave_barrier();
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       if constexpr (K16) {
-        const uint2 piece = {static_cast<uint32_t>(bo[j][0].raw[0]), static_cast<uint32_t>(bo[j][0].raw[1])};
+        const uint2 piece = pieces[j];
         out[j] = Mma16<T>::run(hlo16, piece, out[j]);
         out[j] = Mma16<T>::run(hop16, piece, out[j]);
       } else {

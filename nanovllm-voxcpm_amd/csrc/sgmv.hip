@@ -35,6 +35,7 @@ namespace {
 
 constexpr int kMaxSplits = 64;
 constexpr int kExpandWaves = 4;
+constexpr int kMaxKSplit = 4;  // most K parts the shrink ever uses (the workspace has room for them)
 
 template <typename T> struct Mma;
 template <> struct Mma<__bf16> {
@@ -92,26 +93,32 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
 }
 
 // ---- shrink -------------------------------------------------------------------------------------
-// grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  KR: columns of
-// K per LDS slab (the workgroup's K part is a whole number of slabs).
+// grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  The workgroup's
+// K part is walked in x batches of XW columns (a wavefront holds the batch of its sixteen token
+// rows in registers) and, inside a batch, in A slabs of KR columns that pass through LDS.  Both
+// streams run one step ahead of the MFMAs: the next slab sits in registers and the next x batch
+// is in flight while the current slab is multiplied, so that a compute unit keeps requesting
+// data for the whole life of the workgroup instead of in bursts between barriers.  DB: a second
+// register buffer for the x batches (without it a K part of several batches fetches each batch
+// after the previous one has been consumed; the launcher gives such parts the DB form).
 constexpr int kShrinkWaves = 4;
 
-template <typename T, int R, int KR>
-__global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
-                                                                          float* __restrict__ hws, int64_t xs, int big_off,
-                                                                          int small_off, int big_cap, int sorted_off, int T_, int K,
-                                                                          int num_slots, int num_slices, int ksplit, int krange,
-                                                                          int all_slices, ShrinkSlices sl) {
+template <typename T, int R, int KR, int XW, bool DB>
+__global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                                                             float* __restrict__ hws, int64_t xs, int big_off,
+                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
+                                                                             int num_slots, int num_slices, int ksplit, int krange,
+                                                                             int all_slices, ShrinkSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
   constexpr int CPR = KR / 8;            // 16-byte chunks per slab row
   constexpr int TOTAL = R * CPR;         // chunks per slab
   constexpr int CHUNKS = (TOTAL + NT - 1) / NT;  // chunks each thread copies per slab
-  constexpr int SB = CHUNKS < 8 ? CHUNKS : 8;    // chunks in flight together
   constexpr int KS = KR / 32;            // k-steps per slab
-  constexpr int XB = KS < 16 ? KS : 16;  // x loads in flight together
-  static_assert(CHUNKS % SB == 0 && KS % XB == 0, "slab shape");
+  constexpr int XK = XW / 32;            // k-steps per x batch
+  constexpr int SPB = XW / KR;           // slabs per x batch
+  static_assert(XW % KR == 0 && XK <= 16, "batch shape");
 
   __shared__ __attribute__((aligned(16))) T s_a[R * ASTRIDE];
 
@@ -128,78 +135,91 @@ __global__ __launch_bounds__(kShrinkWaves* kWave) void sgmv_shrink_kernel(const 
   const int slot = tr.slot, start = tr.start, m = tr.m;
 
   const int k0 = kpart * krange;
-  const int nslab = krange / KR;
+  const int nbatch = krange / XW;
   const bool active = wave * 16 < m;  // this wavefront's token block exists
   // token row of this lane (lanes past the end of the tile repeat its last token: they feed the
   // MFMA harmlessly and are never written back)
   const int ti = wave * 16 + lr;
   const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
   const T* xptr = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + k0 + lg * 8;
-  Pack8 xa[XB];
- for (int si = 0; si < nsl; ++si) {
-  const int slice = slice0 + si;
-  const T* A = static_cast<const T*>(sl.a[slice]) + static_cast<int64_t>(slot) * R * K + k0;
+  const int64_t aoff = static_cast<int64_t>(slot) * R * K + k0;
 
+  i32x4 v[CHUNKS];
+  auto request_slab = [&](const T* Aslab) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int c = i * NT + tid;
+      if (TOTAL % NT == 0 || c < TOTAL) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
+    }
+  };
+  auto store_slab = [&]() {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int c = i * NT + tid;
+      if (TOTAL % NT == 0 || c < TOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
+    }
+  };
+  auto request_x = [&](Pack8(&buf)[XK], int kc) {
+#pragma unroll
+    for (int i = 0; i < XK; ++i) buf[i].raw = load128(xptr + kc + i * 32);
+  };
+
+  Pack8 xa[XK], xb[DB ? XK : 1];
   f32x4 acc[RB];
+  bool first = true;
+  // One x batch: `cur` holds it (or is about to), `nxt` receives the following one meanwhile.
+  auto run_batch = [&](Pack8(&cur)[XK], Pack8(&nxt)[XK], int si, int b) {
+    const T* A = static_cast<const T*>(sl.a[slice0 + si]) + aoff;
+    if (DB && active && b + 1 < nbatch) request_x(nxt, (b + 1) * XW);
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  for (int slab = 0; slab < nslab; ++slab) {
-    const T* Aslab = A + slab * KR;
-    const T* xslab = xptr + slab * KR;
-    // the first batch of x loads goes out together with the slab copy (later slices of an
-    // all-slices walk already hold it)
-    if (active && si == 0) {
+    for (int s = 0; s < SPB; ++s) {
+      if (!first) __syncthreads();  // everyone is done reading the previous slab
+      first = false;
+      store_slab();
+      __syncthreads();
+      // the slab after this one: same batch, next batch, or the first of the next slice
+      if (s + 1 < SPB) request_slab(A + b * XW + (s + 1) * KR);
+      else if (b + 1 < nbatch) request_slab(A + (b + 1) * XW);
+      else if (si + 1 < nsl) request_slab(static_cast<const T*>(sl.a[slice0 + si + 1]) + aoff);
+      if (active) {
 #pragma unroll
-      for (int i = 0; i < XB; ++i) xa[i].raw = load128(xslab + i * 32);
-    }
-    if (slab > 0 || si > 0) __syncthreads();  // everyone is done reading the previous slab
-#pragma unroll
-    for (int c0 = 0; c0 < CHUNKS; c0 += SB) {
-      i32x4 v[SB];
-#pragma unroll
-      for (int i = 0; i < SB; ++i) {
-        const int c = (c0 + i) * NT + tid;
-        if (TOTAL % NT == 0 || c < TOTAL) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
-      }
-#pragma unroll
-      for (int i = 0; i < SB; ++i) {
-        const int c = (c0 + i) * NT + tid;
-        if (TOTAL % NT == 0 || c < TOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
-      }
-    }
-    __syncthreads();
-    if (active) {
-#pragma unroll
-      for (int kb = 0; kb < KS; kb += XB) {
-        if (kb > 0) {
-#pragma unroll
-          for (int i = 0; i < XB; ++i) xa[i].raw = load128(xslab + (kb + i) * 32);
-        }
-#pragma unroll
-        for (int i = 0; i < XB; ++i) {
+        for (int i = 0; i < KS; ++i) {
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
             const int rr = rb * 16 + lr;
             Pack8 aw;
-            aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + (kb + i) * 32 + lg * 8]);
-            acc[rb] = Mma<T>::run(aw, xa[i], acc[rb]);
+            aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + i * 32 + lg * 8]);
+            acc[rb] = Mma<T>::run(aw, cur[s * KS + i], acc[rb]);
           }
         }
       }
     }
-  }
+    if (!DB && active && b + 1 < nbatch) request_x(cur, (b + 1) * XW);
+  };
 
-  // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
-  if (active && ti < m) {
-    float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice) * R;
+  request_slab(static_cast<const T*>(sl.a[slice0]) + aoff);
+  if (active) request_x(xa, 0);
+  for (int si = 0; si < nsl; ++si) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const int r0 = rb * 16 + 4 * lg;
-      if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
+    for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (DB) {
+      for (int b = 0; b < nbatch; b += 2) {
+        run_batch(xa, xb, si, b);
+        if (b + 1 < nbatch) run_batch(xb, xa, si, b + 1);
+      }
+    } else {
+      for (int b = 0; b < nbatch; ++b) run_batch(xa, xa, si, b);
+    }
+    // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
+    if (active && ti < m) {
+      float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice0 + si) * R;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int r0 = rb * 16 + 4 * lg;
+        if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
+      }
     }
   }
- }
 }
 
 // ---- expand -------------------------------------------------------------------------------------
@@ -242,16 +262,19 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
 }
 
 template <typename T, int R, int CPL, int TPF, int G>
-__global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
-                                                                          void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
-                                                                          int big_units, int sorted_off, int T_, int num_slots,
-                                                                          int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
+__global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
+                                                                             void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
+                                                                             int big_units, int sorted_off, int T_, int num_slots,
+                                                                             int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
+  constexpr int NB = TB / TPF;           // y batches per tile
+  constexpr int STEPS = G * NB;          // (tile, batch) steps of a span
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps
   constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
   constexpr int NT = kExpandWaves * kWave;
   constexpr int CPR = R / 8;             // groups of eight ranks per token
   constexpr int SPAN = 16 * CPL;         // columns of one span
+  constexpr int HC = (MLORA_TILE_BIG * CPR + NT - 1) / NT;  // H chunks per thread and tile
 
   __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
   __shared__ __attribute__((aligned(16))) int s_row[G * MLORA_TILE_BIG];
@@ -290,136 +313,194 @@ __global__ __launch_bounds__(kExpandWaves* kWave) void sgmv_expand_kernel(const 
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
   if (!usable) return;
 
-  // token rows (entries past the end of a tile repeat its last token: a valid row to read, never
-  // written) and the H tiles -> LDS: K partials summed, scaled, split into leading part and
-  // remainder (absent tokens get zeros)
+  // token rows -> LDS (entries past the end of a tile repeat its last token: a valid row to read,
+  // never written)
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; }
+    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
+  }
+  __syncthreads();
+
+  // A wavefront's work is a sequence of items: for each of its spans of 16 * CPL columns, the
+  // (tile, y batch) steps that hold tokens.  The y rows of the item after the current one are
+  // always in flight, and those of the first item (and its B rows) go out before the H tiles
+  // are staged, so that the stream of y never waits for anything but itself.
+  T* const ybase = static_cast<T*>(yv_) + sp.y_col;
+  auto next_step = [&](int st) {
+    for (++st; st < STEPS; ++st)
+      if (s_m[st / NB] > (st % NB) * TPF * 16) break;
+    return st;
+  };
+  const int first_step = next_step(-1);  // exists: some tile holds tokens
+  auto column = [&](int c0) {  // first of this lane's CPL columns, clamped into the range
+    const int c = c0 + CPL * lr;
+    return c < sp.n1 ? c : sp.n1 - 8;
+  };
+  auto issue_y = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+    const int g = st / NB, tp = (st % NB) * TPF, cl = column(c0);
+#pragma unroll
+    for (int u = 0; u < TPF; ++u) {
+      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + (tp + u) * 16 + 4 * lg]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) buf[u][i] = load_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + cl, nt);
+    }
+  };
+  Pack8 bop[CPL][KSTEPS];
+  int b_slot = -1, b_c0 = -1;  // what bop holds
+  auto load_b = [&](int c0, int sg) {
+    // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
+    // their H operand is zero; columns past the range repeat the last one and are never stored)
+    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) {
+      int n = c0 + CPL * lr + j;
+      n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = (lg + 4 * ks) & (R / 8 - 1);
+        bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+      }
+    }
+    b_slot = sg;
+    b_c0 = c0;
+  };
+  auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+    const int g = st / NB, tp = (st % NB) * TPF;
+    const int mg = s_m[g], sg = s_slot[g];
+    if (sg != b_slot || c0 != b_c0) load_b(c0, sg);
+    const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
+    const int c = c0 + CPL * lr;
+    const bool col_ok = c < sp.n1;
+#pragma unroll
+    for (int u = 0; u < TPF; ++u) {
+      const int tb = tp + u;
+      if (tb * 16 >= mg) continue;
+      Pack8 hop[KSTEPS], hlo[KSTEPS];
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = lg + 4 * ks;
+        if (kc * 8 < R) {
+          hop[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+          hlo[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
+        } else {
+          hop[ks].raw = i32x4{0, 0, 0, 0};
+          hlo[ks].raw = i32x4{0, 0, 0, 0};
+        }
+      }
+      f32x4 out[CPL];
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
+          out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
+        }
+      }
+      // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
+      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + tb * 16 + 4 * lg]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (col_ok && tb * 16 + 4 * lg + i < mg) {
+          YVec<T, CPL> r;
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(buf[u][i].e[j]) + out[j][i]);
+          store_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + c, r, nt);
+        }
+      }
+    }
+  };
+
+  YVec<T, CPL> ya[TPF][4], yb[TPF][4];
+  int c0 = sp.n0 + wave * SPAN, st = first_step;
+  const bool has_work = c0 < sp.n1;
+  if (has_work) {
+    load_b(c0, s_slot[st / NB]);
+    issue_y(ya, c0, st);
+  }
+
+  // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
+  // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
   {
     const int64_t hrow = static_cast<int64_t>(num_slices) * R;
     const int64_t part = static_cast<int64_t>(T_) * hrow;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; }
       if (m[g] == 0) continue;
-      if (tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
       const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
-      for (int c = tid; c < MLORA_TILE_BIG * CPR; c += NT) {
-        const int tok = c / CPR, ch = c % CPR;
-        Pack8 hi, lo;
-        hi.raw = i32x4{0, 0, 0, 0};
-        lo.raw = i32x4{0, 0, 0, 0};
-        if (tok < m[g]) {
-          const float* q = src + tok * hrow + ch * 8;
-          f32x4 s0 = *reinterpret_cast<const f32x4*>(q), s1 = *reinterpret_cast<const f32x4*>(q + 4);
-          for (int kp = 1; kp < ksplit; ++kp) {
-            const f32x4 t0 = *reinterpret_cast<const f32x4*>(q + kp * part), t1 = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
-            s0[0] += t0[0]; s0[1] += t0[1]; s0[2] += t0[2]; s0[3] += t0[3];
-            s1[0] += t1[0]; s1[1] += t1[1]; s1[2] += t1[2]; s1[3] += t1[3];
-          }
-          float v[8], rem[8];
+      f32x4 t[HC][kMaxKSplit][2];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            v[i] = s0[i] * scaling;
-            v[4 + i] = s1[i] * scaling;
-          }
-          pack8<T>(v, hi);
-          float back[8];
-          unpack8<T>(hi, back);
+      for (int h = 0; h < HC; ++h) {
+        const int c = h * NT + tid;
+        int tok = c / CPR;
+        tok = tok < m[g] ? tok : m[g] - 1;
+        const float* q = src + tok * hrow + (c % CPR) * 8;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
-          pack8<T>(rem, lo);
+        for (int kp = 0; kp < kMaxKSplit; ++kp) {
+          if (kp < ksplit) {
+            t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
+            t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+          }
         }
+      }
+#pragma unroll
+      for (int h = 0; h < HC; ++h) {
+        const int c = h * NT + tid, tok = c / CPR, ch = c % CPR;
+        if ((MLORA_TILE_BIG * CPR) % NT != 0 && c >= MLORA_TILE_BIG * CPR) continue;
+        f32x4 s0 = t[h][0][0], s1 = t[h][0][1];
+#pragma unroll
+        for (int kp = 1; kp < kMaxKSplit; ++kp) {
+          if (kp < ksplit) {
+            s0[0] += t[h][kp][0][0]; s0[1] += t[h][kp][0][1]; s0[2] += t[h][kp][0][2]; s0[3] += t[h][kp][0][3];
+            s1[0] += t[h][kp][1][0]; s1[1] += t[h][kp][1][1]; s1[2] += t[h][kp][1][2]; s1[3] += t[h][kp][1][3];
+          }
+        }
+        Pack8 hi, lo;
+        float v[8], back[8], rem[8];
+        const float live = tok < m[g] ? scaling : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = s0[i] * live;
+          v[4 + i] = s1[i] * live;
+        }
+        pack8<T>(v, hi);
+        unpack8<T>(hi, back);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
+        pack8<T>(rem, lo);
         *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
         *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
       }
     }
   }
   __syncthreads();
+  if (!has_work) return;
 
-  T* ybase = static_cast<T*>(yv_) + sp.y_col;
-
-  for (int c0 = sp.n0 + wave * SPAN; c0 < sp.n1; c0 += kExpandWaves * SPAN) {
-    Pack8 bop[CPL][KSTEPS];
-    int loaded = -1;  // slot whose B rows are in bop
-    const int c = c0 + CPL * lr;
-    const bool col_ok = c < sp.n1;
-    const int cl = col_ok ? c : sp.n1 - 8;
-
-    for (int g = 0; g < G; ++g) {
-      const int mg = s_m[g];
-      if (mg == 0) continue;
-      const int sg = s_slot[g];
-      if (sg != loaded) {
-        // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
-        // their H operand is zero; columns past the range repeat the last one and are never stored)
-        const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
-#pragma unroll
-        for (int j = 0; j < CPL; ++j) {
-          int n = c0 + CPL * lr + j;
-          n = n < sp.n1 ? n : sp.n1 - 1;
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int kc = (lg + 4 * ks) & (R / 8 - 1);
-            bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-          }
-        }
-        loaded = sg;
-      }
-      const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
-      const int* rowg = s_row + g * MLORA_TILE_BIG;
-
-#pragma unroll
-      for (int tp = 0; tp < TB; tp += TPF) {  // TPF token blocks at a time: their y rows are in flight together
-        if (tp * 16 >= mg) continue;
-        YVec<T, CPL> yreg[TPF][4];
-        T* yrow[TPF][4];
-#pragma unroll
-        for (int u = 0; u < TPF; ++u) {
-          const i32x4 rows = *reinterpret_cast<const i32x4*>(&rowg[(tp + u) * 16 + 4 * lg]);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            yrow[u][i] = ybase + static_cast<int64_t>(rows[i]) * ys;
-            yreg[u][i] = load_y<T, CPL>(yrow[u][i] + cl, nt);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < TPF; ++u) {
-          const int tb = tp + u;
-          if (tb * 16 >= mg) continue;
-          Pack8 hop[KSTEPS], hlo[KSTEPS];
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int kc = lg + 4 * ks;
-            if (kc * 8 < R) {
-              hop[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-              hlo[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
-            } else {
-              hop[ks].raw = i32x4{0, 0, 0, 0};
-              hlo[ks].raw = i32x4{0, 0, 0, 0};
-            }
-          }
-          f32x4 out[CPL];
-#pragma unroll
-          for (int j = 0; j < CPL; ++j) {
-            out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-              out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
-              out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
-            }
-          }
-          // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (col_ok && tb * 16 + 4 * lg + i < mg) {
-              YVec<T, CPL> r;
-#pragma unroll
-              for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(yreg[u][i].e[j]) + out[j][i]);
-              store_y<T, CPL>(yrow[u][i] + c, r, nt);
-            }
-          }
-        }
-      }
+  // two y buffers, used in turn
+  auto advance = [&](int& nc0, int& nst) {  // item after (c0, st); false when there is none
+    nst = next_step(st);
+    nc0 = c0;
+    if (nst >= STEPS) {
+      nst = first_step;
+      nc0 = c0 + kExpandWaves * SPAN;
     }
+    return nc0 < sp.n1;
+  };
+  for (;;) {
+    int nc0, nst;
+    bool more = advance(nc0, nst);
+    if (more) issue_y(yb, nc0, nst);
+    process(ya, c0, st);
+    if (!more) break;
+    c0 = nc0;
+    st = nst;
+    more = advance(nc0, nst);
+    if (more) issue_y(ya, nc0, nst);
+    process(yb, c0, st);
+    if (!more) break;
+    c0 = nc0;
+    st = nst;
   }
 }
 
@@ -432,32 +513,31 @@ struct ShrinkLaunch {
   int ksplit, krange, all_slices;
 };
 
-template <typename T, int R, int KR>
+template <typename T, int R, int KR, int XW, bool DB>
 void launch_shrink_one(const ShrinkLaunch& l) {
   const MloraAddArgs* a = l.a;
   dim3 grid(8, static_cast<unsigned>(l.all_slices ? l.ksplit : a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
-  hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
+  hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR, XW, DB>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
                      l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, l.sl);
 }
 
+// (slab width, x batch width): 128/128 and 256/256 with two x buffers, 256/512 and 512/512 with one
 template <typename T, int R>
-void launch_shrink_slab(const ShrinkLaunch& l, int kr) {
-  switch (kr) {
-    case 128: launch_shrink_one<T, R, 128>(l); break;
-    case 256: launch_shrink_one<T, R, 256>(l); break;
-    case 512: launch_shrink_one<T, R, 512>(l); break;
-    default: launch_shrink_one<T, R, 1024>(l); break;
-  }
+void launch_shrink_slab(const ShrinkLaunch& l, int kr, int xw) {
+  if (kr == 128) launch_shrink_one<T, R, 128, 128, true>(l);
+  else if (kr == 256 && xw == 256) launch_shrink_one<T, R, 256, 256, true>(l);
+  else if (kr == 256) launch_shrink_one<T, R, 256, 512, false>(l);
+  else launch_shrink_one<T, R, 512, 512, false>(l);
 }
 
 template <typename T>
-void launch_shrink_rank(const ShrinkLaunch& l, int kr) {
+void launch_shrink_rank(const ShrinkLaunch& l, int kr, int xw) {
   switch (l.a->r) {
-    case 8: launch_shrink_slab<T, 8>(l, kr); break;
-    case 16: launch_shrink_slab<T, 16>(l, kr); break;
-    case 32: launch_shrink_slab<T, 32>(l, kr); break;
-    default: launch_shrink_slab<T, 64>(l, kr); break;
+    case 8: launch_shrink_slab<T, 8>(l, kr, xw); break;
+    case 16: launch_shrink_slab<T, 16>(l, kr, xw); break;
+    case 32: launch_shrink_slab<T, 32>(l, kr, xw); break;
+    default: launch_shrink_slab<T, 64>(l, kr, xw); break;
   }
 }
 
@@ -520,9 +600,6 @@ static size_t partial_bytes(int num_tokens, int num_slices, int r) {
   return static_cast<size_t>(num_tokens) * static_cast<size_t>(num_slices) * static_cast<size_t>(r) * sizeof(float);
 }
 
-// Room for the most K parts the shrink ever uses.
-constexpr int kMaxKSplit = 4;
-
 size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype) {
   (void)dtype;
   if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
@@ -559,26 +636,31 @@ int launch_sgmv(const MloraAddArgs* a) {
   if (cols == 0) return 0;
   const int est_tiles = a->num_tokens / MLORA_TILE_BIG + 1;
 
-  // shrink: LDS slab width (the A slab of r rows has to fit next to nothing else), then K parts
-  // so that the grid has a few workgroups per compute unit
+  // shrink: x batch width (what a wavefront holds in registers: 512 columns when K allows), A
+  // slab width (a whole batch: on the prefill and the mixed batch 128-, 256- and 512-column
+  // slabs measured within 2 % of each other), then K parts so that the grid has a few
+  // workgroups per compute unit
+  int xw = 512;
+  while (xw > 128 && a->k % xw != 0) xw /= 2;
   int kr = env_int("MLORA_SGMV_KR", 0);
-  if (kr != 128 && kr != 256 && kr != 512 && kr != 1024) kr = 512;
-  while (kr > 128 && (a->k % kr != 0)) kr /= 2;
+  if (kr != 128 && kr != 256 && kr != 512) kr = xw;
+  if (kr > xw) kr = xw;
+  if (kr == 128) xw = 128;  // 128-column slabs come with 128-column batches only
   const int max_parts = static_cast<int>(static_cast<size_t>(a->workspace_bytes) / partial_bytes(a->num_tokens, a->num_slices, a->r));
   int ksplit = env_int("MLORA_SGMV_KSPLIT", 0);
   if (ksplit <= 0) {
     ksplit = 1;
-    while (ksplit < kMaxKSplit && static_cast<long long>(est_tiles) * a->num_slices * ksplit < 512 && a->k % (kr * ksplit * 2) == 0) ksplit *= 2;
+    while (ksplit < kMaxKSplit && static_cast<long long>(est_tiles) * a->num_slices * ksplit < 512 && a->k % (xw * ksplit * 2) == 0) ksplit *= 2;
   }
   if (ksplit > max_parts) ksplit = max_parts;
   if (ksplit > kMaxKSplit) ksplit = kMaxKSplit;
-  while (ksplit > 1 && a->k % (kr * ksplit) != 0) --ksplit;
+  while (ksplit > 1 && a->k % (xw * ksplit) != 0) --ksplit;
   // three or more slices: one workgroup walks them all with the x rows it already holds, when
-  // its K part is a single batch of loads (measured on the prefill batch: qkv 31.9 -> 29.6 us per
-  // call; with two slices the shorter chain of separate workgroups wins, gate_up 76.6 vs 77.8)
+  // its K part is a single batch (measured on the prefill batch: qkv 31.9 -> 29.6 us per call;
+  // with two slices the shorter chain of separate workgroups wins, gate_up 76.6 vs 77.8)
   l.all_slices = 0;
-  if (a->num_slices >= env_int("MLORA_SGMV_ALL_SLICES", 3) && kr <= 512) {
-    const int parts = a->k / kr;
+  if (a->num_slices >= env_int("MLORA_SGMV_ALL_SLICES", 3)) {
+    const int parts = a->k / xw;
     if (parts <= kMaxKSplit && parts <= max_parts) {
       ksplit = parts;
       l.all_slices = 1;
@@ -586,8 +668,10 @@ int launch_sgmv(const MloraAddArgs* a) {
   }
   l.ksplit = ksplit;
   l.krange = a->k / ksplit;
-  if (a->dtype == MLORA_DTYPE_BF16) launch_shrink_rank<__bf16>(l, kr);
-  else launch_shrink_rank<_Float16>(l, kr);
+  // a K part of several batches: the form with two x buffers (256-column batches)
+  if (xw == 512 && l.krange > xw && env_int("MLORA_SGMV_XDB", 1)) { xw = 256; kr = 256; }
+  if (a->dtype == MLORA_DTYPE_BF16) launch_shrink_rank<__bf16>(l, kr, xw);
+  else launch_shrink_rank<_Float16>(l, kr, xw);
   int rc = check_launch("mlora_add_lora(sgmv shrink)");
   if (rc) return rc;
 
