@@ -296,13 +296,14 @@ def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
     print(f"long form r={rank} {dtype} {knobs}", flush=True)
     for key, value in knobs.items():
         monkeypatch.setenv(key, value)
-    shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520])}
+    # K = 640 and 768 take 128- and 256-column x batches, 1536 and 2048 several batches per K part
+    shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520]), "s": (640, [64, 72]), "t": (768, [264]), "u": (1536, [136]), "v": (2048, [64])}
     lengths = [130, 1, 64, 15, 16, 65, 3, 128, 17, 7]
     slot_of = [2, 0, 5, 1, 3, -1, 4, 2, -1, 6]  # slot 2 twice: two segments merge into one of 258
     slots = torch.cat([torch.full((n,), s, dtype=torch.int32) for n, s in zip(lengths, slot_of)])
     slots = slots[torch.randperm(slots.numel(), generator=torch.Generator().manual_seed(9))].cuda()
     T = slots.numel()
-    for name in ("p", "q"):
+    for name in shapes:
         proj = synthetic.make_projection(name, 7, rank, dtype, seed=900 + rank, device="cuda", shapes=shapes)
         xw, yw = synthetic.make_activations(T, proj.k + 24, sum(proj.widths) + 40, dtype, seed=901, device="cuda")
         x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 16 : 16 + sum(proj.widths)]  # 16-byte aligned views of wider buffers
