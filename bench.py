@@ -366,8 +366,8 @@ def main() -> None:
     launch_us = ms * 1e3 / launches
     achieved = launch_bytes / (launch_us * 1e-6) / 1e9
     default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers
-    kernel = {"decode": "decode_kernel<bf16,16>", "prefill": "sgmv_kernel<bf16,64,64>",
-              "mixed": "sgmv_kernel<bf16,64,64> + decode_kernel<bf16,64>"}[args.workload]
+    kernel = {"decode": "decode_kernel<bf16,16>", "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
+              "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>"}[args.workload]
     if args.form == "bgmv":
         kernel = "bgmv_kernel<bf16>"
     out = {
@@ -410,7 +410,7 @@ def main() -> None:
             # HBM bytes per average launch from the two rocprofv3 --pmc runs of the default workload
             # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 256 MiB copy in the same runs);
             # only quoted for the configuration those runs covered
-            "traffic": 9823027 if default_run else None,
+            "traffic": 9824051 if default_run else None,
             "bytes_per_launch": round(launch_bytes),
             "us_per_launch": round(launch_us, 3),
         },
