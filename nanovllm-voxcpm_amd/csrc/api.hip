@@ -62,6 +62,22 @@ bool vector_ok(const MloraAddArgs* a) {
 
 }  // namespace
 
+// Where the one-launch form over 16-token tiles stops paying.  Its cost per token grows with the
+// rank (every tile fetches A[slot] again, every column range repeats its tile's shrink) while the
+// two-launch form pays about 10 us up front; measured per projection shape, single- and
+// multi-adapter batches of 512..16384 tokens, the two meet where tokens x (slices x K + columns)
+// reaches 8.4e7 for ranks up to 16, 1.7e7 for rank 32 and 0.86e7 for rank 64 (rank 64: 840
+// tokens for gate_up, 4200 for o; rank 16: 8200 for gate_up, never below 16384 for o and qkv).
+// MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
+static bool small_batch(const MloraAddArgs* a) {
+  const int fixed = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
+  if (fixed > 0) return a->num_tokens <= fixed;
+  long long width = static_cast<long long>(a->num_slices) * a->k;
+  for (int i = 0; i < a->num_slices; ++i) width += a->slices[i].n;
+  const long long limit = a->r <= 16 ? 84000000LL : a->r <= 32 ? 17000000LL : 8600000LL;
+  return static_cast<long long>(a->num_tokens) * width <= limit;
+}
+
 extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   if (!a) { set_error("mlora_add_lora: NULL args"); return MLORA_E_INVALID; }
   if (a->num_tokens < 0 || a->k < 0 || a->r < 0 || a->num_slots < 0 || a->num_slices < 0) {
@@ -94,10 +110,10 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   }
   if (form == MLORA_FORM_AUTO) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
-    // tiles for the long segments and 16-token tiles for the rest.
+    // tiles for the long segments and 16-token tiles for the rest, as two launches.
     if (!vec) form = MLORA_FORM_TOKEN;
     else if (!mfma_supported(a)) form = MLORA_FORM_BGMV;
-    else if (a->num_tokens <= env_int("MLORA_SMALL_BATCH_TOKENS", 1024) || !sgmv_supported(a) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
+    else if (small_batch(a) || !sgmv_supported(a) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
     else form = MLORA_FORM_SGMV;
   }
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && vec && mfma_supported(a) && !(sgmv_supported(a) && sgmv_workspace_ok(a))) form = MLORA_FORM_MFMA;

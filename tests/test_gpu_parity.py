@@ -314,6 +314,26 @@ def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
         assert torch.equal(y._base[:, :16], yw[:, :16]) and torch.equal(y._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
 
 
+@pytest.mark.parametrize("rank,expected", [(16, "mfma"), (64, "sgmv")])
+def test_auto_form_follows_rank_and_width(rank, expected):
+    """A 3000-token prefill of three sequences through the o projection: at rank 16 the one-launch
+    small-tile form is the faster one up to far larger batches, at rank 64 the two-launch form
+    takes over near 4000 tokens x (K + N) / 2048.  AUTO gives the oracle's result in both cases
+    and exactly what the form it is meant to pick gives."""
+    print(f"auto form r={rank}", flush=True)
+    T = 3000 if rank == 16 else 5000
+    proj = _make("o", 4, rank, torch.bfloat16, seed=330 + rank)
+    slots = torch.cat([torch.full((T // 2,), 1, dtype=torch.int32), torch.full((T // 4,), -1, dtype=torch.int32),
+                       torch.full((T - T // 2 - T // 4,), 3, dtype=torch.int32)]).cuda()
+    from nanovllm_voxcpm_amd import synthetic
+
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=331, device="cuda")
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"auto/r{rank}")
+    assert torch.equal(got, _apply(expected, proj, x, y0.clone(), slots))
+
+
 # ---- config 4: mixed batch, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity ----
 
 
