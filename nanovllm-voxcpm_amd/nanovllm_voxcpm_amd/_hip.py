@@ -243,7 +243,15 @@ def dtype_code(dtype: torch.dtype) -> int:
 
 
 def _stream(device: torch.device) -> int:
+    """Handle of torch's current stream on ``device`` (the raw-handle query is several times
+    cheaper than building a ``torch.cuda.Stream`` object, and this runs on every call)."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        return raw(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+current_stream_handle = _stream
 
 
 def _require_cuda(t: torch.Tensor, name: str) -> None:
@@ -271,14 +279,16 @@ def add_lora(
     scaling: float,
     form: int = FORM_AUTO,
     workspace: torch.Tensor | None = None,
+    stream: int | None = None,
 ) -> None:
-    """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice."""
+    """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice.
+    ``stream``: handle of the stream to launch on, torch's current one when omitted."""
     lib = load()
     _require_cuda(x, "x")
     if len(a_slices) > MAX_SLICES:
         raise ValueError(f"at most {MAX_SLICES} slices per call, got {len(a_slices)}")
     args = MloraAddArgs()
-    args.stream = _stream(x.device)
+    args.stream = _stream(x.device) if stream is None else stream
     args.x = x.data_ptr()
     args.y = y.data_ptr()
     args.x_stride = x.stride(0)
@@ -435,9 +445,10 @@ def install_slot(
     _check(lib.mlora_install_slot(C.byref(args)), "mlora_install_slot")
 
 
-def stream_capture_id(device: torch.device) -> int:
-    """Identifier of the graph capture in progress on torch's current stream, 0 when none."""
-    return int(load().mlora_stream_capture_id(_stream(device)))
+def stream_capture_id(device: torch.device, stream: int | None = None) -> int:
+    """Identifier of the graph capture in progress on ``stream`` (torch's current stream on
+    ``device`` when omitted), 0 when none."""
+    return int(load().mlora_stream_capture_id(_stream(device) if stream is None else stream))
 
 
 def build_info() -> str:

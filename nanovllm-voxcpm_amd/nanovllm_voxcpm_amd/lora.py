@@ -129,7 +129,7 @@ class HipLoRABackend:
 
     # -- segment plan ---------------------------------------------------------------------
     @staticmethod
-    def _plan_for(metadata: LoRAMetadata, tts: torch.Tensor, max_slots: int) -> SegmentPlan:
+    def _plan_for(metadata: LoRAMetadata, tts: torch.Tensor, max_slots: int, capture: int | None = None) -> SegmentPlan:
         """One metadata launch per batch: every LoRA layer of a step shares the metadata
         object, so the plan is cached on it.
 
@@ -145,7 +145,9 @@ class HipLoRABackend:
             version = own._version
         except RuntimeError:  # inference tensors carry no version counter
             version = None
-        key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, _hip.stream_capture_id(tts.device))
+        if capture is None:
+            capture = _hip.stream_capture_id(tts.device)
+        key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, capture)
         cache = getattr(metadata, _PLAN_ATTR, None)
         if cache is None:
             cache = {}
@@ -160,16 +162,19 @@ class HipLoRABackend:
             plan = cache[key] = build_segment_plan(tts, max_slots)
         return plan
 
-    def _scratch_for(self, x: torch.Tensor, num_slices: int, rank: int) -> torch.Tensor:
+    def _scratch_for(self, x: torch.Tensor, num_slices: int, rank: int, stream: int | None = None,
+                     capture: int | None = None) -> torch.Tensor:
         """Device scratch for the rank-r intermediate (between the two launches of the
         long-segment form, or between workgroups sharing one shrink).  One buffer per
         (device, stream), grown on demand: calls on one stream are ordered, so they can share
         it; a buffer first created while a graph is being captured belongs to that graph's
         memory pool and is not kept for later eager calls."""
         nbytes = _hip.add_workspace_bytes(x.size(0), num_slices, rank, x.dtype)
-        stream = torch.cuda.current_stream(x.device)
-        capture = _hip.stream_capture_id(x.device)
-        key = (x.device, stream.cuda_stream, capture)
+        if stream is None:
+            stream = _hip.current_stream_handle(x.device)
+        if capture is None:
+            capture = _hip.stream_capture_id(x.device, stream)
+        key = (x.device, stream, capture)
         buf = self._scratch.get(key)
         if buf is None or buf.numel() < nbytes:
             if len(self._scratch) >= 8:
@@ -259,6 +264,8 @@ class HipLoRABackend:
 
         # Slices are launched together when they share (rank, K); shapes that differ (never
         # the case for the stacked projections) simply take one launch each.
+        stream = _hip.current_stream_handle(x2.device)  # looked up once per call
+        capture = None
         groups: dict[tuple[int, int], list[int]] = {}
         for i in live:
             a = lora_a_slices[i]
@@ -272,9 +279,11 @@ class HipLoRABackend:
                 plan = scratch = None
                 form = _hip.FORMS[self.form]
                 if form != _hip.FORM_TOKEN and self._vectorisable(x2, target, a_list, b_list, c_list):
-                    plan = self._plan_for(metadata, tts, a_list[0].size(0)).workspace
-                    scratch = self._scratch_for(x2, len(chunk), a_list[0].size(-2))
-                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch)
+                    if capture is None:
+                        capture = _hip.stream_capture_id(x2.device, stream)
+                    plan = self._plan_for(metadata, tts, a_list[0].size(0), capture).workspace
+                    scratch = self._scratch_for(x2, len(chunk), a_list[0].size(-2), stream, capture)
+                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch, stream)
         if staged is not None:
             staged.copy_(target)
         return outputs
