@@ -1,3 +1,8 @@
+// Entry points declared in include/mlora.h.  mlora_add_lora stands where the reference's backend
+// method stands (nanovllm_voxcpm/lora.py:241-381); its slice grouping plan (lora.py:65-90, 195-239)
+// and pointer tables (lora_ops/triton_ops/utils.py:15-116) have no counterpart: one launch takes a
+// table of slices with their own widths, and pointers travel by value.
+//
 // C-ABI front door: argument checks, form selection, error text.
 #include <stdarg.h>
 #include <stdio.h>

@@ -1,3 +1,6 @@
+// Vector-ALU alternative to decode.hip for the same computation (reference:
+// nanovllm_voxcpm/lora.py:291-381, lora_ops/triton_ops/lora_shrink_op.py:104-210).
+//
 // BGMV form (vector ALU): one workgroup per (small tile, slice, column range).  A small tile is
 // up to sixteen tokens that share a slot; the workgroup takes them eight at a time.
 //   shrink  — every lane takes one 128-bit chunk of K, forms the partial dot products of its

@@ -1,3 +1,9 @@
+// Computes, for decode-sized batches, what the reference computes with a shrink launch, a
+// temporary [slices, T, r] tensor and one or two expand launches
+// (nanovllm_voxcpm/lora.py:291-381 driving lora_ops/triton_ops/lora_shrink_op.py:16-173,
+// lora_expand_op.py:11-91 and kernel_utils.py:7-228; its small-batch dispatch:
+// lora_shrink_op.py:10-13, 176-210): y_i[t] += (x[t] . A_i[s_t]^T) . B_i[s_t]^T * scaling.
+//
 // Small-tile form: one workgroup per (small tile, slice, column range).  A small tile is up
 // to sixteen tokens of one slot, described by a self-contained 128-byte record.
 //

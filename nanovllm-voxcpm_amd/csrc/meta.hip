@@ -1,6 +1,9 @@
 // On-device segment metadata: a stable counting sort of the tokens by slot id, run by one
 // workgroup, that emits (a) the plan workspace the apply kernels walk and (b) any of the
-// three index layouts the reference builds on the host.
+// three index layouts the reference builds on the host: the engine's (slots ascending, -1
+// left out: nanovllm_voxcpm/engine/lora_manager.py:77-91, utils/context.py:77-116), the kernel
+// metadata's (-1 bucket first: lora_ops/triton_ops/lora_kernel_metadata.py:46-68) and the graph
+// buffers' (fixed ids -1 .. L-1, counts scattered: engine/model_runner.py:727-797).
 #include "common.h"
 
 namespace mlora {

@@ -1,3 +1,8 @@
+// Computes, for prefill-sized batches, what the reference computes with its segment-grouped
+// shrink and expand kernels (nanovllm_voxcpm/lora_ops/triton_ops/lora_shrink_op.py:16-101, 257-341,
+// lora_expand_op.py:11-170, kernel_utils.py:7-228, launched from nanovllm_voxcpm/lora.py:291-381):
+// y_i[t] += (x[t] . A_i[s_t]^T) . B_i[s_t]^T * scaling, tokens grouped by slot.
+//
 // SGMV form for batches above the small-batch limit: two launches that meet in a small
 // workspace, both on the matrix cores (v_mfma_f32_16x16x32 bf16 / f16, fp32 accumulate).  Work
 // units are the 64-token tiles of the long segments and, behind them in the same grids, the

@@ -1,7 +1,10 @@
 // Shape- and dtype-agnostic kernels: one workgroup per token, scalar loads.  They carry the
 // fp32 / odd-shape cases of the fused apply, the unfused shrink and expand of the low-level
 // API, and the slot install.  Nothing here needs segment metadata: a token's slot id is all
-// a workgroup reads.
+// a workgroup reads.  Reference semantics followed: lora_shrink (zero-filled output, scaling in
+// the shrink: lora_ops/triton_ops/lora_shrink_op.py:257-341), lora_expand (offset_start,
+// add_inputs, product rounded to B's type first: lora_expand_op.py:94-170), set_slot_lora
+// (slot zeroed, rank-limited copy, alpha / r folded into B: nanovllm_voxcpm/layers/lora.py:395-417).
 #include "common.h"
 
 namespace mlora {
