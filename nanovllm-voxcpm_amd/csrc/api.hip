@@ -102,8 +102,14 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
     const MloraSlice& s = a->slices[i];
     if (s.n < 0 || s.y_col < 0) { set_error("mlora_add_lora: slice %d has negative extent", i); return MLORA_E_INVALID; }
     if (s.n > 0 && (!s.a || !s.b)) { set_error("mlora_add_lora: slice %d has NULL weights", i); return MLORA_E_INVALID; }
+    if (static_cast<int64_t>(s.y_col) + s.n > a->y_stride) {
+      set_error("mlora_add_lora: slice %d ends at column %lld, beyond the y row stride %lld", i, static_cast<long long>(s.y_col) + s.n,
+                static_cast<long long>(a->y_stride));
+      return MLORA_E_INVALID;
+    }
     any |= s.n > 0;
   }
+  if (a->x_stride < a->k) { set_error("mlora_add_lora: x row stride %lld is below K = %d", static_cast<long long>(a->x_stride), a->k); return MLORA_E_INVALID; }
   if (!any) return 0;
   if (reinterpret_cast<uintptr_t>(a->plan) & 15) { set_error("mlora_add_lora: plan must be 16-byte aligned"); return MLORA_E_INVALID; }
 

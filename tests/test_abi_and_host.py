@@ -87,6 +87,13 @@ def test_arguments_are_rejected_before_any_launch():
     assert lib.mlora_add_lora(C.byref(args)) == -3
     args.num_slots = 2  # valid sizes, NULL tensors
     assert lib.mlora_add_lora(C.byref(args)) == -1 and b"NULL tensor" in lib.mlora_last_error()
+    # rows that would overlap or run past their stride (dummy addresses: rejected before any use)
+    args.x, args.y, args.token_to_slot = 0x1000, 0x2000, 0x3000
+    args.x_stride, args.y_stride = 8, 8
+    args.slices[0].a, args.slices[0].b, args.slices[0].n, args.slices[0].y_col = 0x4000, 0x5000, 16, 0
+    assert lib.mlora_add_lora(C.byref(args)) == -1 and b"y row stride" in lib.mlora_last_error()
+    args.y_stride, args.x_stride = 16, 4
+    assert lib.mlora_add_lora(C.byref(args)) == -1 and b"x row stride" in lib.mlora_last_error()
     args.num_tokens = 0  # nothing to do is success
     assert lib.mlora_add_lora(C.byref(args)) == 0
     meta = _hip.MloraMetaArgs()
