@@ -97,34 +97,6 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
   return t;
 }
 
-// The fp32 partial sums travel through memory between workgroups.  Between two launches plain
-// accesses do; inside one launch (the fused form) the writer and the reader may sit on different
-// XCDs with their own L2s, so every word is written and read with device-scope atomic accesses,
-// which are performed where all compute units meet and need no cache flushed.
-template <bool COH>
-__device__ __forceinline__ void store_partial(float* p, const f32x4& v) {
-  if constexpr (COH) {
-    const uint64_t lo = static_cast<uint64_t>(__float_as_uint(v[0])) | (static_cast<uint64_t>(__float_as_uint(v[1])) << 32);
-    const uint64_t hi = static_cast<uint64_t>(__float_as_uint(v[2])) | (static_cast<uint64_t>(__float_as_uint(v[3])) << 32);
-    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(reinterpret_cast<uint64_t*>(p) + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  } else {
-    *reinterpret_cast<f32x4*>(p) = v;
-  }
-}
-template <bool COH>
-__device__ __forceinline__ f32x4 load_partial(const float* p) {
-  if constexpr (COH) {
-    uint64_t* q = reinterpret_cast<uint64_t*>(const_cast<float*>(p));
-    const uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return f32x4{__uint_as_float(static_cast<uint32_t>(lo)), __uint_as_float(static_cast<uint32_t>(lo >> 32)),
-                 __uint_as_float(static_cast<uint32_t>(hi)), __uint_as_float(static_cast<uint32_t>(hi >> 32))};
-  } else {
-    return *reinterpret_cast<const f32x4*>(p);
-  }
-}
-
 // ---- shrink -------------------------------------------------------------------------------------
 // grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  The workgroup's
 // K part is walked in x batches of XW columns (a wavefront holds the batch of its sixteen token
@@ -136,16 +108,12 @@ __device__ __forceinline__ f32x4 load_partial(const float* p) {
 // after the previous one has been consumed; the launcher gives such parts the DB form).
 constexpr int kShrinkWaves = 4;
 
-template <int R, int KR>
-constexpr int shrink_lds_bytes() { return R * (KR + 8) * 2; }
-
-// The work of one workgroup on one tile (slot, start, m): slices slice0 .. slice0 + nsl - 1, K part
-// kpart.  `after_slice(slice)` runs, in uniform control flow, once that slice's partial sums have
-// been stored.
-template <typename T, int R, int KR, int XW, bool DB, bool COH, typename AfterSlice>
-__device__ __forceinline__ void shrink_body(T* s_a, const int32_t* __restrict__ plan, const void* __restrict__ xv, float* __restrict__ hws,
-                                            int64_t xs, int sorted_off, int T_, int K, int num_slices, int krange, const ShrinkSlices& sl,
-                                            int slot, int start, int m, int slice0, int nsl, int kpart, AfterSlice after_slice) {
+template <typename T, int R, int KR, int XW, bool DB>
+__global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                                                             float* __restrict__ hws, int64_t xs, int big_off,
+                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
+                                                                             int num_slots, int num_slices, int ksplit, int krange,
+                                                                             int all_slices, ShrinkSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -157,8 +125,19 @@ __device__ __forceinline__ void shrink_body(T* s_a, const int32_t* __restrict__ 
   constexpr int SPB = XW / KR;           // slabs per x batch
   static_assert(XW % KR == 0 && XK <= 16, "batch shape");
 
+  __shared__ __attribute__((aligned(16))) T s_a[R * ASTRIDE];
+
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
+  // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
+  // registers (its K part is a single batch then), instead of one workgroup per slice
+  const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
+  const int nsl = all_slices ? num_slices : 1;
+  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+
+  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
+  if (!tr.ok) return;
+  const int slot = tr.slot, start = tr.start, m = tr.m;
 
   const int k0 = kpart * krange;
   const int nbatch = krange / XW;
@@ -242,29 +221,10 @@ __device__ __forceinline__ void shrink_body(T* s_a, const int32_t* __restrict__ 
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const int r0 = rb * 16 + 4 * lg;
-        if (r0 < R) store_partial<COH>(dst + r0, acc[rb]);
+        if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
       }
     }
-    after_slice(slice0 + si);
   }
-}
-
-template <typename T, int R, int KR, int XW, bool DB>
-__global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
-                                                                             float* __restrict__ hws, int64_t xs, int big_off,
-                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
-                                                                             int num_slots, int num_slices, int ksplit, int krange,
-                                                                             int all_slices, ShrinkSlices sl) {
-  __shared__ __attribute__((aligned(16))) char s_a[shrink_lds_bytes<R, KR>()];
-  // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
-  // registers (its K part is a single batch then), instead of one workgroup per slice
-  const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
-  const int nsl = all_slices ? num_slices : 1;
-  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
-  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
-  if (!tr.ok) return;
-  shrink_body<T, R, KR, XW, DB, false>(reinterpret_cast<T*>(s_a), plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, sl, tr.slot,
-                                       tr.start, tr.m, slice0, nsl, kpart, [](int) {});
 }
 
 // ---- expand -------------------------------------------------------------------------------------
@@ -306,14 +266,11 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
   else *reinterpret_cast<Raw*>(p) = r;
 }
 
-template <typename T, int R, int G>
-constexpr int expand_lds_bytes() { return G * MLORA_TILE_BIG * (2 * R + 8) * static_cast<int>(sizeof(T)) + G * MLORA_TILE_BIG * 4 + 2 * G * 4; }
-
-// The work of one workgroup on G tiles (slot, start, m; m = 0: no tile) and one column range.
-template <typename T, int R, int CPL, int TPF, int G, bool COH>
-__device__ __forceinline__ void expand_body(char* smem, const int32_t* __restrict__ plan, const float* __restrict__ hws, void* __restrict__ yv_,
-                                            int64_t ys, int sorted_off, int T_, int num_slices, int ksplit, float scaling, int nt,
-                                            const ExpandSplit& sp, const int (&slot)[G], const int (&start)[G], const int (&m)[G]) {
+template <typename T, int R, int CPL, int TPF, int G>
+__global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
+                                                                             void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
+                                                                             int big_units, int sorted_off, int T_, int num_slots,
+                                                                             int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int NB = TB / TPF;           // y batches per tile
   constexpr int STEPS = G * NB;          // (tile, batch) steps of a span
@@ -324,13 +281,42 @@ __device__ __forceinline__ void expand_body(char* smem, const int32_t* __restric
   constexpr int SPAN = 16 * CPL;         // columns of one span
   constexpr int HC = (MLORA_TILE_BIG * CPR + NT - 1) / NT;  // H chunks per thread and tile
 
-  T* const s_h = reinterpret_cast<T*>(smem);                                      // [G * 64][HSTRIDE]
-  int* const s_row = reinterpret_cast<int*>(smem + G * MLORA_TILE_BIG * HSTRIDE * sizeof(T));  // [G * 64]
-  int* const s_slot = s_row + G * MLORA_TILE_BIG;                                // [G]
-  int* const s_m = s_slot + G;                                                   // [G]
+  __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) int s_row[G * MLORA_TILE_BIG];
+  __shared__ int s_slot[G], s_m[G];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
+  // A workgroup takes G consecutive 64-token tiles (consecutive tiles mostly belong to one slot,
+  // whose B rows then stay in registers across them), or, past `big_units`, one short segment.
+  const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const bool is_big = unit < big_units;
+  const int sidx = is_big ? 0 : unit - big_units;
+
+  // header and every candidate record are requested together (all addresses are in bounds for
+  // the whole grid)
+  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
+  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);
+  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);
+  const i32x4 small = *reinterpret_cast<const i32x4*>(plan + small_off + sidx * MLORA_SMALL_TILE_WORDS);
+  i32x4 big[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) big[g] = reinterpret_cast<const i32x4*>(plan + big_off)[is_big ? unit * G + g : 0];
+  const ExpandSplit sp = splits.split[blockIdx.y];
+  const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
+  int slot[G], start[G], m[G], any = 0;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const bool have = is_big ? unit * G + g < n_big : (g == 0 && sidx < n_short);
+    slot[g] = is_big ? big[g][0] : small[0];
+    start[g] = is_big ? big[g][1] : small[2];
+    m[g] = is_big ? big[g][2] : small[1];
+    if (!have || m[g] <= 0 || slot[g] < 0 || slot[g] >= num_slots) m[g] = 0;
+    any |= m[g];
+  }
+  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
+  if (!usable) return;
 
   // token rows -> LDS (entries past the end of a tile repeat its last token: a valid row to read,
   // never written)
@@ -458,8 +444,8 @@ __device__ __forceinline__ void expand_body(char* smem, const int32_t* __restric
 #pragma unroll
         for (int kp = 0; kp < kMaxKSplit; ++kp) {
           if (kp < ksplit) {
-            t[h][kp][0] = load_partial<COH>(q + kp * part);
-            t[h][kp][1] = load_partial<COH>(q + kp * part + 4);
+            t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
+            t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
           }
         }
       }
@@ -521,45 +507,6 @@ __device__ __forceinline__ void expand_body(char* smem, const int32_t* __restric
     c0 = nc0;
     st = nst;
   }
-}
-
-template <typename T, int R, int CPL, int TPF, int G>
-__global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
-                                                                             void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
-                                                                             int big_units, int sorted_off, int T_, int num_slots,
-                                                                             int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
-  __shared__ __attribute__((aligned(16))) char smem[expand_lds_bytes<T, R, G>()];
-  // A workgroup takes G consecutive 64-token tiles (consecutive tiles mostly belong to one slot,
-  // whose B rows then stay in registers across them), or, past `big_units`, one short segment.
-  const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
-  const bool is_big = unit < big_units;
-  const int sidx = is_big ? 0 : unit - big_units;
-
-  // header and every candidate record are requested together (all addresses are in bounds for
-  // the whole grid)
-  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);
-  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);
-  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);
-  const i32x4 small = *reinterpret_cast<const i32x4*>(plan + small_off + sidx * MLORA_SMALL_TILE_WORDS);
-  i32x4 big[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) big[g] = reinterpret_cast<const i32x4*>(plan + big_off)[is_big ? unit * G + g : 0];
-  const ExpandSplit sp = splits.split[blockIdx.y];
-  const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
-  int slot[G], start[G], m[G], any = 0;
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const bool have = is_big ? unit * G + g < n_big : (g == 0 && sidx < n_short);
-    slot[g] = is_big ? big[g][0] : small[0];
-    start[g] = is_big ? big[g][1] : small[2];
-    m[g] = is_big ? big[g][2] : small[1];
-    if (!have || m[g] <= 0 || slot[g] < 0 || slot[g] >= num_slots) m[g] = 0;
-    any |= m[g];
-  }
-  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
-                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
-  if (!usable) return;
-  expand_body<T, R, CPL, TPF, G, false>(smem, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt, sp, slot, start, m);
 }
 
 struct ShrinkLaunch {
