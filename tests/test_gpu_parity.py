@@ -334,6 +334,44 @@ def test_auto_form_follows_rank_and_width(rank, expected):
     assert torch.equal(got, _apply(expected, proj, x, y0.clone(), slots))
 
 
+@pytest.mark.parametrize("seed", list(range(32)))
+def test_seeded_random_shapes_all_forms_agree_with_the_oracle(seed):
+    """Shapes nobody picked by hand: token counts 1..2500, 1..40 slots, K a multiple of 32 (so
+    also of 64 and 128 in some draws, which decides which kernels may run), one to three slices
+    of ragged widths, a random share of rows without adapter, random segment structure (sorted
+    runs or fully shuffled), views of wider buffers.  Every form that accepts the shape gives the
+    oracle's result."""
+    g = torch.Generator().manual_seed(7000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    rank = (8, 16, 32, 64)[ri(0, 3)]
+    dtype = (torch.bfloat16, torch.float16)[ri(0, 1)]
+    T, L = (1, 7, 40, 300, 1100, 2500)[ri(0, 5)], (1, 3, 9, 40)[ri(0, 3)]
+    K = 32 * ri(1, 40) if ri(0, 1) else 128 * ri(1, 16)
+    widths = [8 * ri(1, 96) for _ in range(ri(1, 3))]
+    print(f"random seed={seed} r={rank} {dtype} T={T} L={L} K={K} widths={widths}", flush=True)
+    slots = torch.randint(0, L, (T,), generator=g, dtype=torch.int32)
+    if ri(0, 1):
+        slots = torch.sort(slots).values  # long runs, as a prefill batch has them
+    slots[torch.rand(T, generator=g) < (0.0, 0.2, 0.7)[ri(0, 2)]] = -1
+    slots = slots.cuda()
+    a = [(torch.randn(L, rank, K, generator=g) * 0.05).to(dtype).cuda() for _ in widths]
+    b = [(torch.randn(L, n, rank, generator=g) * 0.05).to(dtype).cuda() for n in widths]
+    from nanovllm_voxcpm_amd import synthetic
+
+    proj = synthetic.ProjectionWeights("random", K, widths, a, b)
+    pad_x, pad_y = 8 * ri(0, 2), 8 * ri(0, 2)
+    xw = torch.randn(T, K + 2 * pad_x, generator=g).to(dtype).cuda()
+    yw = torch.randn(T, sum(widths) + 2 * pad_y, generator=g).to(dtype).cuda()
+    x, y0 = xw[:, pad_x : pad_x + K], yw[:, pad_y : pad_y + sum(widths)]
+    exact, mag = _exact(proj, x, y0, slots, scaling=0.5)
+    forms = ["auto", "token", "bgmv", "mfma"] + (["sgmv"] if K % 128 == 0 else [])
+    for form in forms:
+        y = yw.clone()[:, pad_y : pad_y + sum(widths)]
+        got = _apply(form, proj, x, y, slots, scaling=0.5)
+        _check(got, y0, exact, mag, slots, f"random/{seed}/{form}")
+        assert torch.equal(y._base[:, :pad_y], yw[:, :pad_y]) and torch.equal(y._base[:, pad_y + sum(widths):], yw[:, pad_y + sum(widths):])
+
+
 # ---- config 4: mixed batch, 128 adapters of ranks {8,16,32,64} padded to 64, Zipf popularity ----
 
 
