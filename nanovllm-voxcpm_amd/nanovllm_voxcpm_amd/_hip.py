@@ -7,6 +7,7 @@ torch's current stream.  A missing library is an error, never a silent fallback.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
 from pathlib import Path
@@ -253,6 +254,18 @@ def _stream(device: torch.device) -> int:
 
 current_stream_handle = _stream
 
+_SAME_DEVICE = contextlib.nullcontext()
+
+
+def _on(device: torch.device):
+    """Context in which ``device`` is the calling thread's current device: a kernel launch goes to
+    the current device, whatever stream it names, so a tensor on another GPU of the process has
+    to make its device current for the call.  One process per GPU (the reference's deployment)
+    never switches."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(device.index)
+
 
 def _require_cuda(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
@@ -312,7 +325,8 @@ def add_lora(
     if workspace is not None:
         args.workspace = workspace.data_ptr()
         args.workspace_bytes = workspace.numel() * workspace.element_size()
-    _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
+    with _on(x.device):
+        _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
 
 
 def shrink(
@@ -336,7 +350,8 @@ def shrink(
     args.scaling = scaling
     for i, a in enumerate(a_slices):
         args.a[i] = a.data_ptr()
-    _check(lib.mlora_shrink(C.byref(args)), "mlora_shrink")
+    with _on(x.device):
+        _check(lib.mlora_shrink(C.byref(args)), "mlora_shrink")
 
 
 def expand(
@@ -366,7 +381,8 @@ def expand(
     for i, b in enumerate(b_slices):
         args.b[i] = b.data_ptr()
         args.n[i] = b.size(1)
-    _check(lib.mlora_expand(C.byref(args)), "mlora_expand")
+    with _on(h.device):
+        _check(lib.mlora_expand(C.byref(args)), "mlora_expand")
 
 
 def _ptr(t: torch.Tensor | None) -> int | None:
@@ -411,7 +427,8 @@ def meta_build(
     args.padded_token_to_slot = _ptr(padded_token_to_slot)
     args.padded_len = padded_token_to_slot.numel() if padded_token_to_slot is not None else 0
     args.scalars = _ptr(scalars)
-    _check(lib.mlora_meta_build(C.byref(args)), "mlora_meta_build")
+    with _on(token_to_slot.device):
+        _check(lib.mlora_meta_build(C.byref(args)), "mlora_meta_build")
 
 
 def install_slot(
@@ -442,7 +459,8 @@ def install_slot(
     args.dtype = dtype_code(a_dst.dtype)
     args.src_dtype = dtype_code(a_src.dtype)
     args.scaling = scaling
-    _check(lib.mlora_install_slot(C.byref(args)), "mlora_install_slot")
+    with _on(a_dst.device):
+        _check(lib.mlora_install_slot(C.byref(args)), "mlora_install_slot")
 
 
 def stream_capture_id(device: torch.device, stream: int | None = None) -> int:
