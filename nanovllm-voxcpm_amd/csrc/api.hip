@@ -71,15 +71,16 @@ bool vector_ok(const MloraAddArgs* a) {
 // rank (every tile fetches A[slot] again, every column range repeats its tile's shrink) while the
 // two-launch form pays about 10 us up front; measured per projection shape, single- and
 // multi-adapter batches of 512..16384 tokens, the two meet where tokens x (slices x K + columns)
-// reaches 8.4e7 for ranks up to 16, 1.7e7 for rank 32 and 0.86e7 for rank 64 (rank 64: 840
-// tokens for gate_up, 4200 for o; rank 16: 8200 for gate_up, never below 16384 for o and qkv).
+// reaches 8.4e7 for ranks up to 16, 1.7e7 for rank 32 and about 1.2e7 for rank 64 (rank 64: 850
+// tokens for gate_up, 2200 for down, 3500 for qkv, 7500 for o; rank 16: 8200 for gate_up, never
+// below 16384 for o and qkv).
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
 static bool small_batch(const MloraAddArgs* a) {
   const int fixed = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
   if (fixed > 0) return a->num_tokens <= fixed;
   long long width = static_cast<long long>(a->num_slices) * a->k;
   for (int i = 0; i < a->num_slices; ++i) width += a->slices[i].n;
-  const long long limit = a->r <= 16 ? 84000000LL : a->r <= 32 ? 17000000LL : 8600000LL;
+  const long long limit = a->r <= 16 ? 84000000LL : a->r <= 32 ? 17000000LL : 12000000LL;
   return static_cast<long long>(a->num_tokens) * width <= limit;
 }
 

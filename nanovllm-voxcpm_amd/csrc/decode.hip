@@ -117,7 +117,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
   __shared__ int s_arrived;
   constexpr int kStageRow = 17;  // 16 chunks of 16 bytes + one of padding: operand reads hit every bank once
-  __shared__ __attribute__((aligned(16))) i32x4 s_stage[TR ? kNW * (1 + RB) * 16 * kStageRow : 1];
+  constexpr int SB = RB < 2 ? RB : 2;  // 16-rank blocks of A staged together (rank 64 goes through in two passes)
+  __shared__ __attribute__((aligned(16))) i32x4 s_stage[TR ? kNW * (1 + SB) * 16 * kStageRow : 1];
   static_assert(!TR || KSPW == 4, "the staged form covers four k-steps per wavefront");
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -257,19 +258,24 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   if constexpr (TR) {
     // through the wavefront's LDS block: written row-contiguously, read in operand layout
     // (k-step i of lane group g is chunk 4 * i + g, the same elements the direct loads take)
-    i32x4* stage = s_stage + wave * (1 + RB) * 16 * kStageRow;
+    i32x4* stage = s_stage + wave * (1 + SB) * 16 * kStageRow;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[i];
+    for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[i];
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) stage[((1 + rb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = ast[rb][i];
-    }
-    __builtin_amdgcn_wave_barrier();
+    for (int p = 0; p < RB / SB; ++p) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+      for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) aw[rb][i].raw = stage[((1 + rb) * 16 + lr) * kStageRow + 4 * i + lg];
+        for (int sb = 0; sb < SB; ++sb) stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = ast[p * SB + sb][i];
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+#pragma unroll
+        for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
+      }
+      __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass (and later by the expand)
     }
   }
 #pragma unroll
@@ -484,7 +490,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       // B rows -> operand pieces through the wavefront's LDS block: four rows (128 bytes) per
       // group, groups 144 bytes apart so that the sixteen lanes of a piece read hit every bank
       // once.  MFMA j of lane (lr, lg) takes ranks 4*lg .. 4*lg+3 of column c0 + 4*lr + j.
-      char* blk = reinterpret_cast<char*>(s_stage + wave * (1 + RB) * 16 * kStageRow);
+      char* blk = reinterpret_cast<char*>(s_stage + wave * (1 + SB) * 16 * kStageRow);
       *reinterpret_cast<i32x4*>(blk + (lane >> 3) * 144 + (lane & 7) * 16) = bo[0][0].raw;
       *reinterpret_cast<i32x4*>(blk + ((lane >> 3) + 8) * 144 + (lane & 7) * 16) = bo[1][0].raw;
       __builtin_amdgcn_wave_barrier();
@@ -577,10 +583,8 @@ void launch_one(const Launch& l) {
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
   if (kspw == 4) {
-    // staged operands: LDS for the A rows of ranks up to 32 (rank 64 would need 174 KB)
-    if constexpr (R <= 32) {
-      if (l.staged) return launch_one<T, R, 4, true>(l);
-    }
+    // staged operands (rank 64 in two passes of 32 ranks through the same LDS block)
+    if (l.staged) return launch_one<T, R, 4, true>(l);
     return launch_one<T, R, 4>(l);
   }
   if (kspw == 2) return launch_one<T, R, 2>(l);
