@@ -652,10 +652,14 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
 
   // Mode 2: the workgroups of a (tile, slice) each take one part of K and one part of the columns.
   // The exchange costs a few trips through memory (about 2 us measured), which pays when K is
-  // long (4096: 8.9 -> 7.9 us per launch at 32 tiles) and does not at K = 1024.
+  // long (4096: 8.9 -> 7.9 us per launch at 32 tiles; 3072: 7.0 -> 6.8) and does not at K = 1024;
+  // at K = 2048 it pays for wide outputs only (2 x 8192 columns: 10.4 -> 9.7 us, but 2048 columns
+  // 5.5 -> 6.0 and three slices of 3072 columns 6.2 -> 8.8).
   int mode = env_int("MLORA_DECODE_MODE", -1);
   const int want = env_int("MLORA_DECODE_KPARTS", 0);
-  if (mode == 2 || (mode < 0 && a->k >= 2048)) {
+  long long all_cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) all_cols += a->slices[i].n;
+  if (mode == 2 || (mode < 0 && (a->k >= 3072 || (a->k >= 2048 && all_cols >= 8192)))) {
     int parts = 1;
     if (live == a->num_slices && live <= MLORA_COOP_SPLITS) parts = usable_parts(a, want > 0 ? want : 4, static_cast<long long>(cap) * live);
     if (parts > 1 && (mode == 2 || static_cast<long long>(cap) * live * parts <= 1024)) {
