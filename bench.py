@@ -67,7 +67,7 @@ def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int) -> int:
     return 2 * t_lora * rank * (len(widths) * k + sum(widths))
 
 
-def build_workload(name: str, device: str):
+def build_workload(name: str, device: str, rank: int | None = None):
     """Per-layer (projection weights, x, y) for the distinct layers of the workload and the
     batch's slot vector.  Layers beyond the distinct ones reuse buffers round-robin (the distinct
     set alone exceeds the 256 MB last-level cache)."""
@@ -76,6 +76,7 @@ def build_workload(name: str, device: str):
     from nanovllm_voxcpm_amd import synthetic
 
     spec = WORKLOADS[name]
+    rank = rank or spec["rank"]
     if name == "decode":
         slots = synthetic.decode_slots(256, spec["slots"], seed=7)
         ranks = None
@@ -90,7 +91,7 @@ def build_workload(name: str, device: str):
     for layer in range(spec["distinct_layers"]):
         entry = {}
         for j, proj_name in enumerate(ORDER):
-            proj = synthetic.make_projection(proj_name, spec["slots"], spec["rank"], torch.bfloat16,
+            proj = synthetic.make_projection(proj_name, spec["slots"], rank, torch.bfloat16,
                                              seed=1000 + 16 * layer + j, device=device, true_ranks=ranks)
             x, y = synthetic.make_activations(num_tokens, proj.k, sum(proj.widths), torch.bfloat16,
                                               seed=5000 + 16 * layer + j, device=device)
@@ -295,6 +296,8 @@ def main() -> None:
     ap.add_argument("--hot-layers", type=int, default=0,
                     help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
                          "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
+    ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
+                    help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
                          "that rocprof byte counters of the same run are scaled by")
@@ -313,7 +316,9 @@ def main() -> None:
     if args.workload == "backbone":
         run_backbone(args)
         return
-    layers, slots = build_workload(args.workload, device)
+    if args.rank and args.workload in ("decode", "prefill"):
+        rank = args.rank
+    layers, slots = build_workload(args.workload, device, rank)
     if args.hot_layers > 0:
         layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
     step, launches = make_step(layers, slots, args.form, args.only)
@@ -365,7 +370,7 @@ def main() -> None:
     launch_bytes = step_bytes / launches
     launch_us = ms * 1e3 / launches
     achieved = launch_bytes / (launch_us * 1e-6) / 1e9
-    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers
+    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers and rank == spec["rank"]
     kernel = {"decode": "decode_kernel<bf16,16>", "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
               "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>"}[args.workload]
     if args.form == "bgmv":
@@ -384,7 +389,7 @@ def main() -> None:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": spec["text"],
+            "workload": spec["text"] if rank == spec["rank"] else spec["text"] + f" -- run at rank {rank} instead",
             "tokens": num_tokens, "tokens_with_adapter": t_lora, "adapters": spec["slots"], "adapters_in_batch": used,
             "rank": rank, "layers": NUM_LAYERS, "projections": names, "form": args.form,
             "launch": "eager" if args.eager else "graph replay",
