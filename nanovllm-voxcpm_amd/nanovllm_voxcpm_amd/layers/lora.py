@@ -221,12 +221,18 @@ class _LoRALayerBase(nn.Module):
         b_dst[slot_id, :, :rank].copy_(b_src[:, :rank] * scaling)
 
     def _record_slot(self, slot_id: int, effective_rank: int, scaling: float) -> None:
-        self.effective_lora_rank[slot_id] = effective_rank
-        self.lora_scaling[slot_id] = scaling
-        self.lora_base_scaling[slot_id] = scaling
-        self._effective_lora_rank_values[slot_id] = effective_rank
-        self._lora_scaling_values[slot_id] = scaling
-        self._lora_base_scaling_values[slot_id] = scaling
+        # The device buffers follow the host mirrors; an element is rewritten (one small launch
+        # each) only when it changes, and adapters that replace each other in a slot mostly share
+        # rank and scaling.
+        if self._effective_lora_rank_values[slot_id] != effective_rank:
+            self.effective_lora_rank[slot_id] = effective_rank
+            self._effective_lora_rank_values[slot_id] = effective_rank
+        if self._lora_scaling_values[slot_id] != scaling:
+            self.lora_scaling[slot_id] = scaling
+            self._lora_scaling_values[slot_id] = scaling
+        if self._lora_base_scaling_values[slot_id] != scaling:
+            self.lora_base_scaling[slot_id] = scaling
+            self._lora_base_scaling_values[slot_id] = scaling
 
     def set_slot_lora(self, slot_id: int, lora_a, lora_b, effective_rank: int, scaling: float) -> None:
         """Make slot ``slot_id`` hold this adapter.  Multi-target layers take ``lora_a`` as

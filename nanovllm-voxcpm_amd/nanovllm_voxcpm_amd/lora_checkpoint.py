@@ -193,11 +193,11 @@ def install_lora_payload(model: torch.nn.Module, slot_id: int, payload: LoRAMode
     ``loaded`` (slot id -> module names, kept by the caller across calls) limits the clearing
     of the previous occupant to the modules it actually populated; without it every
     LoRA-capable module not named in the payload is cleared."""
-    modules = {name: m for name, m in model.named_modules() if hasattr(m, "set_slot_lora")}
-    unknown = [name for name in payload.modules if name not in dict(model.named_modules())]
-    if unknown:
-        raise ValueError(f"Unknown LoRA target module '{unknown[0]}'")
+    every = dict(model.named_modules())  # one walk over the model per admission
+    modules = {name: m for name, m in every.items() if hasattr(m, "set_slot_lora")}
     for name in payload.modules:
+        if name not in every:
+            raise ValueError(f"Unknown LoRA target module '{name}'")
         if name not in modules:
             raise ValueError(f"Module '{name}' does not support LoRA slots")
     previous = loaded.get(slot_id) if loaded is not None and slot_id in loaded else list(modules)
