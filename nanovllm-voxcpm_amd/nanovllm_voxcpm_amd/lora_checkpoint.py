@@ -148,20 +148,34 @@ def _shard(name: str, module: LoRAModulePayload, tp_rank: int, tp_size: int) -> 
 
 
 def _pinned(payload: LoRAModelPayload) -> LoRAModelPayload:
-    """Host staging tensors in pinned memory when a GPU is present, so that the slot load's
-    ``.to("cuda", non_blocking=True)`` is an asynchronous copy."""
-    if not torch.cuda.is_available():
+    """All tensors of the payload as views of one host buffer (``payload.packed``), pinned when a GPU
+    is present: a slot load then moves the adapter with one asynchronous copy instead of one per
+    tensor."""
+    tensors: list[torch.Tensor] = []
+    for m in payload.modules.values():
+        tensors.append(m.lora_a)
+        tensors.extend(m.lora_b if isinstance(m.lora_b, list) else [m.lora_b])
+    if not tensors or any(t.dtype != torch.float32 for t in tensors):
         return payload
+    flat = torch.empty(sum(t.numel() for t in tensors), dtype=torch.float32, pin_memory=torch.cuda.is_available())
+    offset = 0
 
-    def pin(t: torch.Tensor) -> torch.Tensor:
-        return t if t.is_pinned() else t.pin_memory()
+    def view_of(t: torch.Tensor) -> torch.Tensor:
+        nonlocal offset
+        v = flat[offset : offset + t.numel()].view(t.shape)
+        v.copy_(t)
+        offset += t.numel()
+        return v
 
     modules = {
-        name: LoRAModulePayload(lora_a=pin(m.lora_a), lora_b=[pin(t) for t in m.lora_b] if isinstance(m.lora_b, list) else pin(m.lora_b),
+        name: LoRAModulePayload(lora_a=view_of(m.lora_a),
+                                lora_b=[view_of(t) for t in m.lora_b] if isinstance(m.lora_b, list) else view_of(m.lora_b),
                                 effective_rank=m.effective_rank, scaling=m.scaling)
         for name, m in payload.modules.items()
     }
-    return LoRAModelPayload(modules=modules, rank=payload.rank, alpha=payload.alpha)
+    packed = LoRAModelPayload(modules=modules, rank=payload.rank, alpha=payload.alpha)
+    packed.packed = flat  # type: ignore[attr-defined]
+    return packed
 
 
 def load_voxcpm_lora_checkpoint(path: str, *, tp_size: int = 1) -> LoRAModelPayload | list[LoRAModelPayload]:
@@ -204,10 +218,19 @@ def install_lora_payload(model: torch.nn.Module, slot_id: int, payload: LoRAMode
     for name in previous:
         if name not in payload.modules and name in modules:
             modules[name].clear_slot_lora(slot_id)
+    staged: dict = {}  # device -> copy of the payload's packed host buffer
+
     for name, m in payload.modules.items():
         device = next(modules[name].parameters()).device
 
         def put(t: torch.Tensor) -> torch.Tensor:
+            packed = getattr(payload, "packed", None)
+            if packed is not None and device.type == "cuda" and t.is_contiguous():
+                first = (t.data_ptr() - packed.data_ptr()) // packed.element_size()
+                if t.dtype == packed.dtype and 0 <= first and first + t.numel() <= packed.numel():
+                    if device not in staged:
+                        staged[device] = packed.to(device=device, non_blocking=True)
+                    return staged[device][first : first + t.numel()].view(t.shape)
             return t.to(device=device, non_blocking=True)
 
         modules[name].set_slot_lora(slot_id=slot_id, lora_a=put(m.lora_a),
