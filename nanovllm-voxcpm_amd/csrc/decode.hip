@@ -93,7 +93,7 @@ struct DecodeSplits {
 // at the level of the memory system that all compute units share, so no cache has to be
 // flushed.  The counter is back at zero when the launch ends.
 //
-// TR (needs KSPW == 4): a compute unit's vector L1 handles a 128-bit load whose consecutive
+// TR (KSPW a multiple of four): a compute unit's vector L1 handles a 128-bit load whose consecutive
 // lanes touch different rows (what the MFMA operand layout asks for) at about a quarter of the
 // rate of one whose lanes walk along a row, and even cache-resident operands showed up as
 // 3-4 us per launch.  With TR the x rows and A rows of a wavefront's K range are fetched
@@ -110,7 +110,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
   constexpr int NT = kNW * kWave;
-  constexpr int CH = KSPW > 0 ? KSPW : 4;  // k-steps whose loads are in flight together
+  constexpr int CH = TR ? 4 : KSPW > 0 ? KSPW : 4;  // k-steps whose operands are in registers together
+  constexpr int ROUNDS = TR ? KSPW / 4 : 1;          // staged form: groups of four k-steps per wavefront
 
   __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
   __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   constexpr int kStageRow = 17;  // 16 chunks of 16 bytes + one of padding: operand reads hit every bank once
   constexpr int SB = RB < 2 ? RB : 2;  // 16-rank blocks of A staged together (rank 64 goes through in two passes)
   __shared__ __attribute__((aligned(16))) i32x4 s_stage[TR ? kNW * (1 + SB) * 16 * kStageRow : 1];
-  static_assert(!TR || KSPW == 4, "the staged form covers four k-steps per wavefront");
+  static_assert(!TR || (KSPW >= 4 && KSPW % 4 == 0), "the staged form takes the k-steps of a wavefront four at a time");
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
@@ -168,17 +169,21 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   const int ks0 = kpart * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
   const int ks1 = KSPW > 0 ? ks0 + KSPW : kpart * nks + (wave + 1) * nks / kNW;
   Pack8 xa[CH], aw[RB][CH];
-  i32x4 xst[TR ? 4 : 1], ast[TR ? RB : 1][TR ? 4 : 1];
+  i32x4 xst[TR ? 4 * ROUNDS : 1], ast[TR ? RB : 1][TR ? 4 * ROUNDS : 1];
   if constexpr (TR) {
-    // row-contiguous: lane = (row group lane/16, 16-byte chunk lane%16 of the 256-byte K range)
-    const int64_t koff = static_cast<int64_t>(ks0) * 32 + (lane & 15) * 8;
+    // row-contiguous: lane = (row group lane/16, 16-byte chunk lane%16 of a 256-byte K range);
+    // one such range (four k-steps) per round
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xst[i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int64_t koff = static_cast<int64_t>(ks0 + 4 * r) * 32 + (lane & 15) * 8;
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int rr = rb * 16 + 4 * lg + i;
-        ast[rb][i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+      for (int i = 0; i < 4; ++i) {
+        xst[4 * r + i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const int rr = rb * 16 + 4 * lg + i;
+          ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+        }
       }
     }
   } else {
@@ -260,29 +265,39 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     // (k-step i of lane group g is chunk 4 * i + g, the same elements the direct loads take)
     i32x4* stage = s_stage + wave * (1 + SB) * 16 * kStageRow;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[i];
+    for (int r = 0; r < ROUNDS; ++r) {
 #pragma unroll
-    for (int p = 0; p < RB / SB; ++p) {
+      for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[4 * r + i];
+#pragma unroll
+      for (int p = 0; p < RB / SB; ++p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+          for (int sb = 0; sb < SB; ++sb) stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = ast[p * SB + sb][4 * r + i];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+#pragma unroll
+          for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
+        }
+        __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass or round (and later by the expand)
+      }
+      // this round's k-steps, in ascending order as the direct form takes them
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int sb = 0; sb < SB; ++sb) stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = ast[p * SB + sb][i];
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
       }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
-#pragma unroll
-        for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
-      }
-      __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass (and later by the expand)
     }
-  }
+  } else {
 #pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    if (KSPW > 0 || ks0 + i < ks1) {
+    for (int i = 0; i < CH; ++i) {
+      if (KSPW > 0 || ks0 + i < ks1) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+      }
     }
   }
   if (KSPW == 0) {
@@ -582,11 +597,20 @@ void launch_one(const Launch& l) {
 // for every rank and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
-  if (kspw == 4) {
-    // staged operands (rank 64 in two passes of 32 ranks through the same LDS block)
-    if (l.staged) return launch_one<T, R, 4, true>(l);
-    return launch_one<T, R, 4>(l);
+  if (l.staged) {
+    // staged operands, the k-steps of a wavefront four at a time (rank 64 in two passes of 32 ranks
+    // through the same LDS block); how many k-steps fit is a matter of registers: every load of
+    // the workgroup's K part is issued before the first is used
+    if (kspw == 4) return launch_one<T, R, 4, true>(l);
+    if constexpr (R <= 32) {
+      if (kspw == 8) return launch_one<T, R, 8, true>(l);
+    }
+    if constexpr (R <= 16) {
+      if (kspw == 12) return launch_one<T, R, 12, true>(l);
+      if (kspw == 16) return launch_one<T, R, 16, true>(l);
+    }
   }
+  if (kspw == 4) return launch_one<T, R, 4>(l);
   if (kspw == 2) return launch_one<T, R, 2>(l);
   if (kspw == 1) return launch_one<T, R, 1>(l);
   if constexpr (R <= 16) {
@@ -652,14 +676,16 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
 
   // Mode 2: the workgroups of a (tile, slice) each take one part of K and one part of the columns.
   // The exchange costs a few trips through memory (about 2 us measured), which pays when K is
-  // long (4096: 8.9 -> 7.9 us per launch at 32 tiles; 3072: 7.0 -> 6.8) and does not at K = 1024;
-  // at K = 2048 it pays for wide outputs only (2 x 8192 columns: 10.4 -> 9.7 us, but 2048 columns
-  // 5.5 -> 6.0 and three slices of 3072 columns 6.2 -> 8.8).
+  // long (6144 x 1536: 10.4 -> 7.7 us per launch at 32 tiles, 8192 x 2048: 12.9 -> 7.5; at 4096 x 1024
+  // the two are level since the staged loads reach sixteen k-steps per wavefront) and does not at
+  // K = 1024; at K = 2048 and 3072 it pays for wide outputs only (2048 -> 2 x 8192 columns:
+  // 11.1 -> 9.6 us, but 2048 -> 2048 4.7 -> 6.0, 3072 -> 3072 5.9 -> 6.8, and three slices of 3072
+  // columns 5.5 -> 8.6).
   int mode = env_int("MLORA_DECODE_MODE", -1);
   const int want = env_int("MLORA_DECODE_KPARTS", 0);
   long long all_cols = 0;
   for (int i = 0; i < a->num_slices; ++i) all_cols += a->slices[i].n;
-  if (mode == 2 || (mode < 0 && (a->k >= 3072 || (a->k >= 2048 && all_cols >= 8192)))) {
+  if (mode == 2 || (mode < 0 && (a->k >= 4096 || (a->k >= 2048 && all_cols >= 8192)))) {
     int parts = 1;
     if (live == a->num_slices && live <= MLORA_COOP_SPLITS) parts = usable_parts(a, want > 0 ? want : 4, static_cast<long long>(cap) * live);
     if (parts > 1 && (mode == 2 || static_cast<long long>(cap) * live * parts <= 1024)) {

@@ -221,7 +221,8 @@ def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
 
     print(f"small tiles r={rank} {dtype} staged={staged}", flush=True)
     monkeypatch.setenv("MLORA_DECODE_STAGED", staged)
-    shapes = {"a": (1024, [72, 200, 8]), "b": (4096, [328]), "c": (512, [1096, 64]), "d": (160, [24])}
+    shapes = {"a": (1024, [72, 200, 8]), "b": (4096, [328]), "c": (512, [1096, 64]), "d": (160, [24]),
+              "e": (2048, [136, 64]), "f": (3072, [72]), "b0": (4096, [328])}  # 8, 12 (and, unshared, 16) k-steps per wavefront
     g = torch.Generator().manual_seed(40 + rank)
     T = 77
     slots = torch.randint(-1, 9, (T,), generator=g, dtype=torch.int32)
@@ -232,7 +233,10 @@ def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
         xw, yw = synthetic.make_activations(T, proj.k + 16, sum(proj.widths) + 24, dtype, seed=951, device="cuda")
         x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 8 : 8 + sum(proj.widths)]
         y = yw.clone()[:, 8 : 8 + sum(proj.widths)]
+        if name == "b0":
+            monkeypatch.setenv("MLORA_DECODE_MODE", "0")  # all of K = 4096 in one workgroup
         got = _apply("mfma", proj, x, y, slots, scaling=1.25)
+        monkeypatch.delenv("MLORA_DECODE_MODE", raising=False)
         exact, mag = _exact(proj, x, y0, slots, scaling=1.25)
         _check(got, y0, exact, mag, slots, f"small/{name}/r{rank}/{dtype}/staged{staged}")
         assert torch.equal(y._base[:, :8], yw[:, :8]) and torch.equal(y._base[:, 8 + sum(proj.widths):], yw[:, 8 + sum(proj.widths):])
