@@ -213,9 +213,10 @@ def test_ranks_and_dtypes_small(rank, dtype, form):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rank", [8, 16, 32, 64])
 def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
-    """The small-tile kernel at the K values that select its specialisations (1024: four k-steps
-    per wavefront, staged operands for ranks up to 32; 4096: K shared between workgroups; 512 and
-    160: two k-steps / run-time split), with ragged slice widths, narrow and wide column ranges,
+    """The small-tile kernel at the K values that select its specialisations (1024, 2048, 3072:
+    four, eight, twelve k-steps per wavefront with staged operands; 4096: K shared between
+    workgroups, or sixteen k-steps when it is not; 512 and 160: two k-steps / run-time split),
+    with ragged slice widths, narrow and wide column ranges,
     row-strided x and y views, rows without adapter and a segment longer than one tile."""
     from nanovllm_voxcpm_amd import synthetic
 
