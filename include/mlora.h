@@ -97,6 +97,17 @@ typedef struct MloraAddArgs {
 
 int mlora_add_lora(const MloraAddArgs* args);
 
+/* The same fused apply for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  args->workspace and args->workspace_bytes are ignored: the scratch is an array of
+ * MLORA_STATIC_SCRATCH_BYTES bytes that lives in the library's device image, one copy per GPU, held
+ * until the process ends.  The call allocates and frees nothing.  It returns MLORA_E_TOO_LARGE when
+ * one fp32 copy of the rank-r intermediate (num_tokens x num_slices x r x 4 bytes) does not fit the
+ * array.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it and must be ordered by the caller. */
+#define MLORA_STATIC_SCRATCH_BYTES (16u << 20)
+int mlora_add_lora_static(const MloraAddArgs* args);
+
 /* Bytes of MloraAddArgs.workspace that let mlora_add_lora use every form it has for this shape
  * (a smaller workspace is legal: the library then splits K less, or not at all). */
 size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);

@@ -8,6 +8,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "common.h"
 #include "launch.h"
 
@@ -150,6 +152,58 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   }
   set_error("mlora_add_lora: unreachable form %d", form);
   return MLORA_E_INVALID;
+}
+
+// ---- the entry point that allocates nothing --------------------------------------------------
+// Scratch of mlora_add_lora_static: part of the library's device image, so every GPU the
+// library runs on holds its own copy at its own address from module load until the process ends.
+// In host code the name `scratch` is only a handle for hipGetSymbolAddress; the address kernels
+// and copies may use is the one that call returns, looked up once per device.
+static __device__ __align__(256) unsigned char scratch[MLORA_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU (nullptr: not looked up yet)
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`; nullptr (and the error text set) on failure.
+void* static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("mlora_add_lora_static: cannot identify the current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      set_error("mlora_add_lora_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int mlora_add_lora_static(const MloraAddArgs* a) {
+  if (!a) { set_error("mlora_add_lora_static: NULL args"); return MLORA_E_INVALID; }
+  if (a->num_tokens < 0 || a->num_slices < 0 || a->r < 0) { set_error("mlora_add_lora_static: negative size"); return MLORA_E_INVALID; }
+  const unsigned long long one_copy = 4ull * static_cast<unsigned long long>(a->num_tokens) * static_cast<unsigned long long>(a->num_slices) *
+                                      static_cast<unsigned long long>(a->r);
+  if (one_copy > MLORA_STATIC_SCRATCH_BYTES) {
+    set_error("mlora_add_lora_static: num_tokens x num_slices x r x 4 = %llu bytes exceed the static scratch of %u bytes (use mlora_add_lora with a workspace)",
+              one_copy, static_cast<unsigned>(MLORA_STATIC_SCRATCH_BYTES));
+    return MLORA_E_TOO_LARGE;
+  }
+  void* ptr = static_scratch();
+  if (!ptr) return MLORA_E_INVALID;
+  MloraAddArgs b = *a;
+  b.workspace = ptr;
+  b.workspace_bytes = MLORA_STATIC_SCRATCH_BYTES;
+  return mlora_add_lora(&b);
 }
 
 extern "C" size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype) {

@@ -42,11 +42,13 @@ PLAN_HEADER_WORDS = 16
 PLAN_MAGIC_VALUE = 0x4D4C5031
 SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 16, 64
 SMALL_TILE_WORDS, SMALL_TILE_ROWS, BIG_TILE_WORDS = 32, 4, 4
+STATIC_SCRATCH_BYTES = 16 << 20
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 
 EXPORTS = (
     "mlora_add_lora",
+    "mlora_add_lora_static",
     "mlora_add_workspace_bytes",
     "mlora_shrink",
     "mlora_expand",
@@ -197,6 +199,7 @@ def load() -> C.CDLL:
         raise RuntimeError(_LOAD_ERROR) from exc
     for name, args in (
         ("mlora_add_lora", MloraAddArgs),
+        ("mlora_add_lora_static", MloraAddArgs),
         ("mlora_shrink", MloraShrinkArgs),
         ("mlora_expand", MloraExpandArgs),
         ("mlora_meta_build", MloraMetaArgs),
@@ -293,9 +296,12 @@ def add_lora(
     form: int = FORM_AUTO,
     workspace: torch.Tensor | None = None,
     stream: int | None = None,
+    static_scratch: bool = False,
 ) -> None:
     """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice.
-    ``stream``: handle of the stream to launch on, torch's current one when omitted."""
+    ``stream``: handle of the stream to launch on, torch's current one when omitted.
+    ``static_scratch``: call the entry point that allocates nothing and keeps its scratch in the
+    library's own device image (``workspace`` is ignored then)."""
     lib = load()
     _require_cuda(x, "x")
     if len(a_slices) > MAX_SLICES:
@@ -326,7 +332,10 @@ def add_lora(
         args.workspace = workspace.data_ptr()
         args.workspace_bytes = workspace.numel() * workspace.element_size()
     with _on(x.device):
-        _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
+        if static_scratch:
+            _check(lib.mlora_add_lora_static(C.byref(args)), "mlora_add_lora_static")
+        else:
+            _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
 
 
 def shrink(
