@@ -124,6 +124,7 @@ def make_step(layers, slots, form: str, only: str | None = None):
         for blocks, x, a, b, packed in calls:
             backend.add_lora(blocks, x, a, b, indices=slots, metadata=meta, scaling=1.0, y_packed=packed)
 
+    step.backend = backend
     return step, len(calls)
 
 
@@ -229,6 +230,56 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
     }
 
 
+STAMPS = {
+    "decode_kernel": ["entry", "record here", "loads issued", "wave 0 shrink done", "partials in LDS", "intermediate in LDS",
+                      "wave 0 first spans stored", "wave 0 stores acknowledged", "all waves done"],
+    "split_kernel producer": ["entry", "record here", "K part summed", "partials published"],
+    "split_kernel consumer": ["entry", "record here", None, None, "loads issued", "wait over", "intermediate in LDS",
+                              "wave 0 first spans stored", "wave 0 stores acknowledged", "all waves done"],
+}
+
+
+def run_timeline(args) -> None:
+    """In-kernel timeline of the last launch of a step restricted to one projection (24 launches on
+    24 layers' own buffers, so the traced launch reads cold data): readings of the 100 MHz clock
+    taken by thread 0 of every workgroup at fixed points of the kernel, reported in ns after the
+    earliest workgroup entered the kernel (min / median / max over the workgroups that had work).
+    Needs the trace build of the library (make -C nanovllm-voxcpm_amd/csrc trace)."""
+    import torch
+
+    from nanovllm_voxcpm_amd import _hip
+
+    device = "cuda:0"
+    layers, slots = build_workload("decode", device, args.rank or None)
+    step, launches = make_step(layers, slots, args.form, args.timeline)
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    buf = torch.zeros(8192, 16, dtype=torch.int64, device=device)
+    _hip.trace_set(buf)
+    step()
+    torch.cuda.synchronize()
+    _hip.trace_set(None)
+    t = buf.cpu()
+    rows = t[t[:, 1] != 0]  # workgroups that found a tile
+    t0 = int(t[t[:, 0] != 0][:, 0].min())
+    out = {"timeline_of": args.timeline, "form": args.form, "workgroups_launched": int((t[:, 0] != 0).sum()),
+           "workgroups_with_work": int(rows.size(0)), "unit": "ns after the first workgroup entered", "kernels": {}}
+    groups = {"decode_kernel": rows[rows[:, 15] == 0]} if int((rows[:, 15] != 0).sum()) == 0 else {
+        "split_kernel producer": rows[rows[:, 15] != 0], "split_kernel consumer": rows[rows[:, 15] == 0]}
+    for name, g in groups.items():
+        entry = {}
+        for i, label in enumerate(STAMPS[name]):
+            if label is None:
+                continue
+            col = g[:, i]
+            col = (col[col != 0] - t0) * 10
+            if col.numel():
+                entry[label] = [int(col.min()), int(col.median()), int(col.max())]
+        out["kernels"][name] = {"workgroups": int(g.size(0)), "min_median_max": entry}
+    print(json.dumps(out))
+
+
 def run_backbone(args) -> None:
     """BASELINE configs[4]: decode-step latency of a synthetic 24-layer decoder (hidden 1024, 16 query /
     2 KV heads of 64, SwiGLU 4096, RMSNorm; 64 streams with context lengths U[128, 2048]; 32 rank-32
@@ -298,12 +349,18 @@ def main() -> None:
                          "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
     ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
                     help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
+    ap.add_argument("--timeline", default=None, choices=ORDER,
+                    help="diagnostic: in-kernel timeline of one projection's launch on the decode workload "
+                         "(needs the trace build of the library)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
                          "that rocprof byte counters of the same run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; every box in this pool has one (use --gpus 1)")
+
+    if args.timeline:
+        os.environ.setdefault("MLORA_LIBRARY", str(ROOT / "nanovllm-voxcpm_amd" / "nanovllm_voxcpm_amd" / "libmlora_gfx950_trace.so"))
 
     import torch
 
@@ -313,6 +370,9 @@ def main() -> None:
     torch.cuda.set_device(0)
     spec = WORKLOADS[args.workload]
     rank = spec["rank"]
+    if args.timeline:
+        run_timeline(args)
+        return
     if args.workload == "backbone":
         run_backbone(args)
         return
@@ -420,6 +480,14 @@ def main() -> None:
             "us_per_launch": round(launch_us, 3),
         },
     }
+    # waits of the split form that ran out during everything above (0 in a healthy run: a consumer
+    # workgroup that gives up computes its intermediate itself, which is correct but slow)
+    from nanovllm_voxcpm_amd import _hip
+
+    torch.cuda.synchronize()
+    out["split_waits_run_out"] = sum(
+        int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
+        for buf in step.backend._scratch.values())
     if not args.no_cpu_baseline and args.workload == "decode":
         out["cpu_baseline"] = cpu_baseline(layers, slots, rank)
     print(json.dumps(out))

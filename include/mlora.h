@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MLORA_ABI_VERSION 2
+#define MLORA_ABI_VERSION 3
 
 /* element types of x / y / A / B */
 #define MLORA_DTYPE_F32 0
@@ -38,7 +38,11 @@ extern "C" {
 #define MLORA_FORM_BGMV 2  /* small tiles (<= 16 tokens of one slot), packed dot2 + wave64 reductions */
 #define MLORA_FORM_SGMV 3  /* shrink launch + expand launch through the workspace: 64-token MFMA tiles for
                               segments >= threshold, one short tile each for the rest */
-#define MLORA_FORM_MFMA 4  /* small tiles for every segment, both products on the matrix cores */
+#define MLORA_FORM_MFMA 4  /* small tiles for every segment, both products on the matrix cores; one workgroup
+                              per (tile, column range), each repeating its tile's shrink */
+#define MLORA_FORM_SPLIT 5 /* small tiles, one launch: producer workgroups compute the rank-r intermediate of a
+                              (tile, slice, K part) and publish it in the workspace, consumer workgroups take a
+                              column range each, pick the intermediate up and expand; needs an initialised workspace */
 
 /* error codes (negative) */
 #define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
@@ -73,9 +77,9 @@ typedef struct MloraAddArgs {
   int64_t x_stride;
   int64_t y_stride;
   const int32_t* token_to_slot; /* [T] on device */
-  int32_t* plan;          /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
+  const int32_t* plan;    /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
                              (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it).  Read-only
-                             for the caller; launches keep transient arrival counters in it */
+                             for mlora_add_lora too: calls on any number of streams may share one plan */
   int32_t num_tokens;     /* T */
   int32_t k;              /* K, input features */
   int32_t r;              /* rank dimension of the A/B buffers (max_lora_rank) */
@@ -85,14 +89,22 @@ typedef struct MloraAddArgs {
   int32_t form;           /* MLORA_FORM_* */
   float scaling;
   MloraSlice slices[MLORA_MAX_SLICES];
-  void* workspace;        /* device scratch for the rank-r intermediate: between the two launches of
-                             MLORA_FORM_SGMV, and between workgroups that share one shrink in the
-                             small-tile form; 16-byte aligned, or NULL (AUTO then keeps to the
-                             small-tile form, one workgroup per shrink).  Counterpart of
-                             the [S, T, r] buffer the reference allocates between its two kernels
-                             (reference: nanovllm_voxcpm/lora.py:299-381).  Contents need not be kept
-                             between calls; calls that share it must be ordered on one stream. */
-  int64_t workspace_bytes; /* >= mlora_add_workspace_bytes(T, num_slices, r, dtype) to be used */
+  void* workspace;        /* device scratch for the rank-r intermediate: between the producer and the
+                             consumer workgroups of MLORA_FORM_SPLIT and between the two launches of
+                             MLORA_FORM_SGMV; 256-byte aligned and at least MLORA_WORKSPACE_HEAD_BYTES
+                             long, or NULL (AUTO then keeps to MLORA_FORM_MFMA).  Counterpart of the
+                             [S, T, r] buffer the reference allocates between its two kernels
+                             (reference: nanovllm_voxcpm/lora.py:299-381).  Pass it to
+                             mlora_workspace_init once after allocating it; calls that share a
+                             workspace must be ordered on one stream. */
+  int64_t workspace_bytes; /* >= mlora_add_workspace_bytes(T, num_slices, r, dtype) lets every form be used */
+  const int32_t* effective_rank; /* [num_slots] on device, or NULL: rank of the adapter resident in each slot
+                             of THESE buffers (0: none).  Rows of A_i[s] and columns of B_i[s] at or
+                             above effective_rank[s] are then neither read nor multiplied, so a slot
+                             costs what its own rank costs, not what the padded rank costs.  The
+                             reference keeps this vector per layer
+                             (reference: nanovllm_voxcpm/layers/lora.py:409-417) and relies on the
+                             padding being zero; with NULL this library does the same. */
 } MloraAddArgs;
 
 int mlora_add_lora(const MloraAddArgs* args);
@@ -109,8 +121,20 @@ int mlora_add_lora(const MloraAddArgs* args);
 int mlora_add_lora_static(const MloraAddArgs* args);
 
 /* Bytes of MloraAddArgs.workspace that let mlora_add_lora use every form it has for this shape
- * (a smaller workspace is legal: the library then splits K less, or not at all). */
+ * (a smaller workspace of at least MLORA_WORKSPACE_HEAD_BYTES is legal: the two-launch form then
+ * splits K less, or AUTO does not choose it). */
 size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);
+
+/* A workspace starts with a head of MLORA_WORKSPACE_HEAD_BYTES bytes: a signature word, one
+ * {generation, arrivals} pair per small tile and the area in which producer workgroups of
+ * MLORA_FORM_SPLIT leave the intermediate for the consumers, every word tagged with its tile's
+ * generation.  mlora_workspace_init enqueues one kernel that clears the head and writes the
+ * signature; call it once after allocation (it is a kernel, not a memset, so it may be recorded
+ * into a graph).  Launches leave the head ready for the next launch.  A workspace whose head
+ * does not carry the signature is still safe to pass: the kernels then compute every
+ * intermediate locally and never read the exchange area.  No counterpart in the reference. */
+#define MLORA_WORKSPACE_HEAD_BYTES (16384 + (1 << 20))
+int mlora_workspace_init(void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0
  * for rows with s_t < 0 (the reference zero-fills the buffer first).
@@ -178,16 +202,13 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
 #define MLORA_TILE_SMALL 16
 #define MLORA_TILE_BIG 64
 /* A small tile is a self-contained 128-byte record, so that a workgroup learns everything it
- * needs from one load: words {slot, token count, first position in sorted_idx, 0}, then the 16
- * token indices of the tile (entries past the count are 0, a valid row), then padding.
+ * needs from one load: words {slot, token count, first position in sorted_idx, 0}, then 16
+ * token indices (the tile's tokens in order; entries past the count repeat them cyclically, so
+ * all sixteen name rows of the tile itself), then padding.
  * A big tile is four words {slot, first position in sorted_idx, token count, 0}. */
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
 #define MLORA_BIG_TILE_WORDS 4
-/* Behind the tile lists the plan holds MLORA_COOP_SPLITS int32 counters per small tile: when
- * several workgroups share the shrink of one tile they count their arrivals there.  They are
- * zero whenever no launch is in flight, so calls that share a plan must be ordered on one stream. */
-#define MLORA_COOP_SPLITS 8
 
 /* Arguments of the on-device metadata build: a stable counting sort of the tokens by
  * slot id.  The plan workspace (always written when non-NULL) feeds mlora_add_lora; the
@@ -238,6 +259,7 @@ typedef struct MloraInstallArgs {
   int32_t dtype;          /* of the destination buffers */
   int32_t src_dtype;      /* of a_src and b_src */
   float scaling;
+  int32_t num_slots;      /* first dimension of a_dst / b_dst: slot >= num_slots is rejected */
 } MloraInstallArgs;
 
 int mlora_install_slot(const MloraInstallArgs* args);
@@ -246,6 +268,17 @@ int mlora_install_slot(const MloraInstallArgs* args);
  * capturing.  No counterpart in the reference: lets a host-side cache tell work recorded
  * into one capture from work run eagerly or recorded into another capture. */
 uint64_t mlora_stream_capture_id(void* stream);
+
+/* Diagnostic knobs (the MLORA_* environment variables) are read once per process and kept;
+ * this makes the next call read them again.  No counterpart in the reference. */
+void mlora_reload_knobs(void);
+
+/* In-kernel timelines (diagnostic, no counterpart in the reference).  The library variant built
+ * with `make trace` (libmlora_gfx950_trace.so) records, per workgroup of the small-tile kernels,
+ * up to 16 readings of the 100 MHz clock at fixed points of the kernel into `buf` (uint64
+ * [workgroups][16], device memory the caller zeroes; NULL switches recording off).  The regular
+ * library returns MLORA_E_UNSUPPORTED. */
+int mlora_trace_set(void* buf);
 
 /* Library identification and diagnostics. */
 int mlora_abi_version(void);

@@ -35,6 +35,11 @@ int check_launch(const char* what) {
   return 0;
 }
 
+namespace {
+int g_knob_generation = 0;
+}
+int knob_generation() { return g_knob_generation; }
+
 int env_int(const char* name, int fallback) {
   const char* v = getenv(name);
   if (!v || !*v) return fallback;
@@ -69,6 +74,27 @@ bool vector_ok(const MloraAddArgs* a) {
 
 }  // namespace
 
+namespace {
+
+// Diagnostic knobs, read from the environment once per process.
+struct ApiKnobs {
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_k;
+  void read() {
+    generation = knob_generation();
+    small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
+    force_form = env_int("MLORA_FORCE_FORM", 0);
+    no_split = env_int("MLORA_NO_SPLIT", 0);
+    split_min_k = env_int("MLORA_SPLIT_MIN_K", 2048);
+  }
+};
+const ApiKnobs& knobs() {
+  static ApiKnobs k;
+  if (k.generation != knob_generation()) k.read();
+  return k;
+}
+
+}  // namespace
+
 // Where the one-launch form over 16-token tiles stops paying.  Its cost per token grows with the
 // rank (every tile fetches A[slot] again, every column range repeats its tile's shrink) while the
 // two-launch form pays about 10 us up front; measured per projection shape, single- and
@@ -78,7 +104,7 @@ bool vector_ok(const MloraAddArgs* a) {
 // below 16384 for o and qkv).
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
 static bool small_batch(const MloraAddArgs* a) {
-  const int fixed = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
+  const int fixed = knobs().small_batch_tokens;
   if (fixed > 0) return a->num_tokens <= fixed;
   long long width = static_cast<long long>(a->num_slices) * a->k;
   for (int i = 0; i < a->num_slices; ++i) width += a->slices[i].n;
@@ -86,7 +112,17 @@ static bool small_batch(const MloraAddArgs* a) {
   return static_cast<long long>(a->num_tokens) * width <= limit;
 }
 
-extern "C" int mlora_add_lora(const MloraAddArgs* a) {
+namespace {
+
+int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace);
+
+}  // namespace
+
+extern "C" int mlora_add_lora(const MloraAddArgs* a) { return add_lora_impl(a, false); }
+
+namespace {
+
+int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (!a) { set_error("mlora_add_lora: NULL args"); return MLORA_E_INVALID; }
   if (a->num_tokens < 0 || a->k < 0 || a->r < 0 || a->num_slots < 0 || a->num_slices < 0) {
     set_error("mlora_add_lora: negative size"); return MLORA_E_INVALID;
@@ -94,7 +130,7 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   if (a->dtype != MLORA_DTYPE_F32 && a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) {
     set_error("mlora_add_lora: unknown dtype %d", a->dtype); return MLORA_E_INVALID;
   }
-  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_MFMA) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
+  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_SPLIT) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
   if (a->num_slices > MLORA_MAX_SLICES) { set_error("mlora_add_lora: %d slices exceed %d", a->num_slices, MLORA_MAX_SLICES); return MLORA_E_TOO_LARGE; }
   if (a->r > MLORA_MAX_RANK) { set_error("mlora_add_lora: rank %d exceeds %d", a->r, MLORA_MAX_RANK); return MLORA_E_TOO_LARGE; }
   if (a->num_slots > MLORA_MAX_SLOTS) { set_error("mlora_add_lora: %d slots exceed %d", a->num_slots, MLORA_MAX_SLOTS); return MLORA_E_TOO_LARGE; }
@@ -119,18 +155,24 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   int form = a->form;
   const bool vec = vector_ok(a);
   if (form == MLORA_FORM_AUTO) {
-    const int forced = env_int("MLORA_FORCE_FORM", 0);
-    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_MFMA && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
+    const int forced = knobs().force_form;
+    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_SPLIT && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
   }
   if (form == MLORA_FORM_AUTO) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
     // tiles for the long segments and 16-token tiles for the rest, as two launches.
+    const bool small_tiles = mfma_supported(a) && decode_supported(a);
+    const bool two_launches = mfma_supported(a) && sgmv_supported(a) && sgmv_workspace_ok(a);
     if (!vec) form = MLORA_FORM_TOKEN;
-    else if (!mfma_supported(a)) form = MLORA_FORM_BGMV;
-    else if (small_batch(a) || !sgmv_supported(a) || !sgmv_workspace_ok(a)) form = MLORA_FORM_MFMA;
-    else form = MLORA_FORM_SGMV;
+    else if (two_launches && !(small_tiles && small_batch(a))) form = MLORA_FORM_SGMV;
+    else if (small_tiles) form = MLORA_FORM_SPLIT;
+    else form = MLORA_FORM_BGMV;
   }
-  if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && vec && mfma_supported(a) && !(sgmv_supported(a) && sgmv_workspace_ok(a))) form = MLORA_FORM_MFMA;
+  // the split form where it pays (long K: the shrink of a tile is worth sharing) and shape and
+  // workspace allow it, else one workgroup per (tile, column range)
+  if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
+      (knobs().no_split || !split_supported(a) || (a->k < knobs().split_min_k && knobs().force_form != MLORA_FORM_SPLIT)))
+    form = MLORA_FORM_MFMA;
   switch (form) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
@@ -138,9 +180,18 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
       if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
       return launch_bgmv(a, /*include_long=*/true);
     case MLORA_FORM_SGMV:
+    case MLORA_FORM_SPLIT:
     case MLORA_FORM_MFMA: {
       if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
+      if (form == MLORA_FORM_SPLIT) {
+        if (!split_supported(a)) {
+          set_error("mlora_add_lora: the split form needs K %% 512 == 0, at most 8 K parts, no empty slice and a 256-byte aligned "
+                    "workspace of at least %d bytes whose exchange area holds every tile's partial sums", MLORA_WORKSPACE_HEAD_BYTES);
+          return MLORA_E_UNSUPPORTED;
+        }
+        return launch_split(a, /*include_long=*/true, trusted_workspace);
+      }
       if (!sgmv_supported(a)) { set_error("mlora_add_lora: SGMV form needs K %% 128 == 0"); return MLORA_E_UNSUPPORTED; }
       if (!sgmv_workspace_ok(a)) {
         set_error("mlora_add_lora: SGMV form needs a 16-byte aligned workspace of %zu bytes and no empty slice",
@@ -153,6 +204,8 @@ extern "C" int mlora_add_lora(const MloraAddArgs* a) {
   set_error("mlora_add_lora: unreachable form %d", form);
   return MLORA_E_INVALID;
 }
+
+}  // namespace
 
 // ---- the entry point that allocates nothing --------------------------------------------------
 // Scratch of mlora_add_lora_static: part of the library's device image, so every GPU the
@@ -193,9 +246,9 @@ extern "C" int mlora_add_lora_static(const MloraAddArgs* a) {
   if (a->num_tokens < 0 || a->num_slices < 0 || a->r < 0) { set_error("mlora_add_lora_static: negative size"); return MLORA_E_INVALID; }
   const unsigned long long one_copy = 4ull * static_cast<unsigned long long>(a->num_tokens) * static_cast<unsigned long long>(a->num_slices) *
                                       static_cast<unsigned long long>(a->r);
-  if (one_copy > MLORA_STATIC_SCRATCH_BYTES) {
-    set_error("mlora_add_lora_static: num_tokens x num_slices x r x 4 = %llu bytes exceed the static scratch of %u bytes (use mlora_add_lora with a workspace)",
-              one_copy, static_cast<unsigned>(MLORA_STATIC_SCRATCH_BYTES));
+  if (one_copy > MLORA_STATIC_SCRATCH_BYTES - MLORA_WORKSPACE_HEAD_BYTES) {
+    set_error("mlora_add_lora_static: num_tokens x num_slices x r x 4 = %llu bytes exceed the static scratch of %u bytes behind its head (use mlora_add_lora with a workspace)",
+              one_copy, static_cast<unsigned>(MLORA_STATIC_SCRATCH_BYTES - MLORA_WORKSPACE_HEAD_BYTES));
     return MLORA_E_TOO_LARGE;
   }
   void* ptr = static_scratch();
@@ -203,13 +256,23 @@ extern "C" int mlora_add_lora_static(const MloraAddArgs* a) {
   MloraAddArgs b = *a;
   b.workspace = ptr;
   b.workspace_bytes = MLORA_STATIC_SCRATCH_BYTES;
-  return mlora_add_lora(&b);
+  // The array starts out zeroed (it is part of the loaded image) and only this library's kernels
+  // ever write it, so its head is always either in the initial state or as a launch left it.
+  return add_lora_impl(&b, /*trusted_workspace=*/true);
 }
 
 extern "C" size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype) {
   if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
-  const size_t big = sgmv_workspace_bytes(num_tokens, num_slices, r, dtype), small = decode_workspace_bytes(r);
-  return big > small ? big : small;
+  return sgmv_workspace_bytes(num_tokens, num_slices, r, dtype);  // head + room for every K part of the intermediate
+}
+
+extern "C" int mlora_workspace_init(void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255)) { set_error("mlora_workspace_init: workspace must be 256-byte aligned"); return MLORA_E_INVALID; }
+  if (workspace_bytes < MLORA_WORKSPACE_HEAD_BYTES) {
+    set_error("mlora_workspace_init: %lld bytes are fewer than MLORA_WORKSPACE_HEAD_BYTES = %d", static_cast<long long>(workspace_bytes), MLORA_WORKSPACE_HEAD_BYTES);
+    return MLORA_E_INVALID;
+  }
+  return workspace_init(workspace, static_cast<hipStream_t>(stream));
 }
 
 extern "C" uint64_t mlora_stream_capture_id(void* stream) {
@@ -221,6 +284,20 @@ extern "C" uint64_t mlora_stream_capture_id(void* stream) {
   }
   return status == hipStreamCaptureStatusActive ? static_cast<uint64_t>(id) : 0;
 }
+
+extern "C" int mlora_trace_set(void* buf) {
+#ifdef MLORA_TRACE
+  decode_trace_set(buf);
+  split_trace_set(buf);
+  return 0;
+#else
+  (void)buf;
+  set_error("mlora_trace_set: this library was built without MLORA_TRACE (make trace builds the variant that records timelines)");
+  return MLORA_E_UNSUPPORTED;
+#endif
+}
+
+extern "C" void mlora_reload_knobs(void) { ++g_knob_generation; }
 
 extern "C" int mlora_abi_version(void) { return MLORA_ABI_VERSION; }
 

@@ -76,6 +76,45 @@ template <> __device__ __forceinline__ void pack8<_Float16>(const float (&in)[8]
   for (int i = 0; i < 8; ++i) p.hf[i] = static_cast<_Float16>(in[i]);
 }
 
+// ---- matrix-core products (fp32 accumulate) -------------------------------------------------
+// 16x16x32: operand lane l holds row (or column) l % 16, elements 8 * (l / 16) .. + 7 of the
+// contraction; the result lane holds rows 4 * (l / 16) .. + 3 of column l % 16.
+template <typename T> struct Mma;
+template <> struct Mma<__bf16> {
+  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.bf, b.bf, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<_Float16> {
+  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.hf, b.hf, c, 0, 0, 0);
+  }
+};
+
+// 16x16x16 variant (four operand elements per lane): for rank 16 the contraction of the
+// expand is exactly sixteen long, so no lane fetches B elements it would multiply by zero.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+template <typename T> struct Mma16;
+template <> struct Mma16<__bf16> {
+  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<_Float16> {
+  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h16x4, a), __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
+  }
+};
+
+// Zero the elements of an eight-element chunk that hold ranks at or above `eff`; `first` is the
+// rank of the chunk's element 0.
+__device__ __forceinline__ void mask_ranks(Pack8& p, int first, int eff) {
+  const int keep = eff - first;  // elements 0 .. keep - 1 stay
+#pragma unroll
+  for (int d = 0; d < 4; ++d) p.u[d] &= (2 * d < keep ? 0x0000ffffu : 0u) | (2 * d + 1 < keep ? 0xffff0000u : 0u);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
@@ -86,7 +125,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles
 // Small tiles are 32-word records (128-byte aligned), big tiles four words; see mlora.h.
 struct PlanLayout {
-  int sorted_off, counts_off, offsets_off, small_off, big_off, coop_off, cap_small, cap_big, total_words;
+  int sorted_off, counts_off, offsets_off, small_off, big_off, cap_small, cap_big, total_words;
 };
 
 __host__ __device__ inline int round_up4(int v) { return (v + 3) & ~3; }
@@ -103,11 +142,40 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   p.cap_small = ((T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs + 7) & ~7;
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
   p.cap_big = (T / MLORA_TILE_BIG + segs + 31) & ~31;  // groups of up to four tiles, eight groups abreast
-  // arrival counters of the workgroups that share one small tile's shrink (zero between launches)
-  p.coop_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
-  p.total_words = p.coop_off + MLORA_COOP_SPLITS * p.cap_small;
+  p.total_words = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
   return p;
 }
+
+// ---- workspace head (see MLORA_WORKSPACE_HEAD_BYTES in mlora.h) -------------------------------
+// uint32 words:  [0] signature | [1] waits that ran out (diagnostic) | ... ; at byte kWsTileOff one
+// {generation, arrivals} pair per small tile; at byte kWsXchgOff the exchange area of the split
+// form: 64-bit words {fp32 bits, tag}, valid when tag == generation of the tile + 1.
+constexpr uint32_t kWsMagic = 0x4d4c5733u;  // "MLW3"
+constexpr int kWsTimeoutsWord = 1;
+constexpr int kWsTileOff = 256;
+constexpr int kWsTiles = 1024;
+constexpr int kWsXchgOff = 16384;
+constexpr int kWsXchgBytes = 1 << 20;
+static_assert(kWsTileOff + 8 * kWsTiles <= kWsXchgOff, "tile state overlaps the exchange area");
+static_assert(kWsXchgOff + kWsXchgBytes == MLORA_WORKSPACE_HEAD_BYTES, "head size");
+
+// ---- in-kernel timeline (builds with -DMLORA_TRACE only) ---------------------------------------
+// MLORA_STAMP(i) makes thread 0 of a workgroup record the 100 MHz clock in slot i of the
+// workgroup's row of the buffer handed to mlora_trace_set (16 slots per workgroup, workgroups in
+// dispatch order).  Without MLORA_TRACE it expands to nothing.
+#ifdef MLORA_TRACE
+#define MLORA_TRACE_DECL static __device__ unsigned long long* trace_buf = nullptr;
+#define MLORA_STAMP(i)                                                                                       \
+  do {                                                                                                       \
+    if (threadIdx.x == 0 && trace_buf)                                                                       \
+      trace_buf[(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 16ull + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define MLORA_TRACE_DECL
+#define MLORA_STAMP(i) \
+  do {                 \
+  } while (0)
+#endif
 
 // ---- error reporting --------------------------------------------------------------------
 void set_error(const char* fmt, ...);

@@ -32,37 +32,11 @@ namespace mlora {
 
 namespace {
 
-constexpr int kMaxSplits = 64;
+constexpr int kMaxSplits = 32;
 constexpr int kNW = 8;          // wavefronts per workgroup
 constexpr int kSpansAhead = 2;  // output spans per wavefront whose loads are issued up front
 
-template <typename T> struct Mma;
-template <> struct Mma<__bf16> {
-  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.bf, b.bf, c, 0, 0, 0);
-  }
-};
-template <> struct Mma<_Float16> {
-  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.hf, b.hf, c, 0, 0, 0);
-  }
-};
-
-// 16x16x16 variant (four operand elements per lane): for rank 16 the contraction of the
-// expand is exactly sixteen long, so no lane fetches B elements it would multiply by zero.
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
-template <typename T> struct Mma16;
-template <> struct Mma16<__bf16> {
-  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma16<_Float16> {
-  static __device__ __forceinline__ f32x4 run(uint2 a, uint2 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h16x4, a), __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
-  }
-};
+MLORA_TRACE_DECL
 
 struct DecodeSplit {
   const void* a;
@@ -75,23 +49,11 @@ struct DecodeSplits {
 };
 
 // KSPW: k-steps (32 elements of K) each wavefront covers when that is known at compile time
-// (K = 32 * kNW * KSPW << kshift), 0 when it has to be worked out from K at run time.
+// (K = 32 * kNW * KSPW), 0 when it has to be worked out from K at run time.
 //
-// A compute unit fills its caches from cold memory far more slowly than the chip as a whole
-// can deliver, so 1 << kshift workgroups can share the shrink of a tile: each covers one part
-// of K, leaves its partial sums in `partials` and counts its arrival in `counters`.  Two ways
-// to go on from there:
-//   mode 1 — the last to arrive adds the parts up and does the expand of the column range; the
-//            others simply exit.  Nobody waits.
-//   mode 2 — every workgroup also owns one part of the slice's columns: it waits (bounded, by
-//            `spin_ticks` of the 100 MHz clock) until all parts have arrived, adds them up and
-//            does the expand of its own columns, so both A[slot] and B[slot] are spread over
-//            the compute units.  A workgroup whose wait runs out computes the missing parts
-//            itself: the wait is a shortcut, never a dependency.
-// The parts are always added in the same order, so the result does not depend on timing.  All
-// exchanged words are written and read with device-scope atomic accesses, which are performed
-// at the level of the memory system that all compute units share, so no cache has to be
-// flushed.  The counter is back at zero when the launch ends.
+// eff_rank (may be null): rank of the adapter resident in each slot.  16-rank blocks of A[slot] at
+// or above it are neither fetched nor multiplied, the intermediate is zero from that rank on, and
+// B[slot] elements from that rank on are replaced by zeros before they reach a multiplier.
 //
 // TR (KSPW a multiple of four): a compute unit's vector L1 handles a 128-bit load whose consecutive
 // lanes touch different rows (what the MFMA operand layout asks for) at about a quarter of the
@@ -104,8 +66,7 @@ template <typename T, int R, int KSPW, bool TR>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
-                                                            int kshift, int mode, int spin_ticks, int32_t* __restrict__ counters,
-                                                            float* __restrict__ partials, DecodeSplits splits) {
+                                                            const int32_t* __restrict__ eff_rank, DecodeSplits splits) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
@@ -116,7 +77,6 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
   __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
   __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
-  __shared__ int s_arrived;
   constexpr int kStageRow = 17;  // 16 chunks of 16 bytes + one of padding: operand reads hit every bank once
   constexpr int SB = RB < 2 ? RB : 2;  // 16-rank blocks of A staged together (rank 64 goes through in two passes)
   __shared__ __attribute__((aligned(16))) i32x4 s_stage[TR ? kNW * (1 + SB) * 16 * kStageRow : 1];
@@ -124,12 +84,12 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
+  MLORA_STAMP(0);  // first instruction
 
   // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first and
   // consecutive ids go to consecutive XCDs, so blockIdx.x is the XCD: the column ranges of one
   // tile share an XCD and its L2.
-  const int group = blockIdx.y >> kshift, kpart = blockIdx.y & ((1 << kshift) - 1);
-  const int split_id = mode == 2 ? blockIdx.y : group;  // mode 2: every part has its own column range
+  const int split_id = blockIdx.y;
   const int tile = blockIdx.z * 8 + blockIdx.x;
 
   // ---- round trip 1 ---------------------------------------------------------------------------
@@ -148,9 +108,19 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // instead of piece by piece behind a chain of branches.
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) &
-                     int(slot < num_slots) & (int(sp.n0 < sp.n1) | int(mode == 2)) & int(sp.a != nullptr) & int(sp.b != nullptr) &
+                     int(slot < num_slots) & int(sp.n0 < sp.n1) & int(sp.a != nullptr) & int(sp.b != nullptr) &
                      int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0);
   if (!usable) return;
+  MLORA_STAMP(1);  // tile record and plan header are here
+
+  // rank of the adapter in this slot (one more dependent fetch, only when the caller gave the vector)
+  int eff = R;
+  if (eff_rank) {
+    eff = eff_rank[slot];
+    eff = eff < 0 ? 0 : eff > R ? R : eff;
+    if (eff == 0) return;
+  }
+  const int rb_n = (eff + 15) >> 4;  // 16-rank blocks of A in use
 
   const bool live = lr < m;  // this lane's token exists
   const T* xrow = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + lg * 8;
@@ -165,9 +135,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   T* yrow = static_cast<T*>(yv_) + static_cast<int64_t>(row) * ys + sp.y_col + 16 * lg;
 
   // ---- round trip 2: issue every load ---------------------------------------------------------
-  const int nks = (K / 32) >> kshift;  // k-steps of this workgroup's part of K
-  const int ks0 = kpart * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
-  const int ks1 = KSPW > 0 ? ks0 + KSPW : kpart * nks + (wave + 1) * nks / kNW;
+  const int nks = K / 32;  // k-steps of the contraction
+  const int ks0 = KSPW > 0 ? wave * KSPW : wave * nks / kNW;
+  const int ks1 = KSPW > 0 ? ks0 + KSPW : (wave + 1) * nks / kNW;
   Pack8 xa[CH], aw[RB][CH];
   i32x4 xst[TR ? 4 * ROUNDS : 1], ast[TR ? RB : 1][TR ? 4 * ROUNDS : 1];
   if constexpr (TR) {
@@ -182,7 +152,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           const int rr = rb * 16 + 4 * lg + i;
-          ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          if (RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          else ast[rb][4 * r + i] = i32x4{0, 0, 0, 0};
         }
       }
     }
@@ -213,6 +184,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         int n = c0 + 32 * h + (lane >> 1);
         n = n < sp.n1 ? n : sp.n1 - 1;
         bo[h][0].raw = load128(B + static_cast<int64_t>(n) * R + (lane & 1) * 8);
+        if (eff < R) mask_ranks(bo[h][0], (lane & 1) * 8, eff);
       }
     } else {
 #pragma unroll
@@ -223,6 +195,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          if (eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
     }
@@ -247,6 +220,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
             // zero, and an unconditional load keeps the whole batch of loads in flight together
             const int kc = (lg + 4 * ks) & (R / 8 - 1);
             bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+            if (eff < R) mask_ranks(bop[s][j][ks], kc * 8, eff);
           }
         }
 #pragma unroll
@@ -256,6 +230,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     }
   }
 
+  MLORA_STAMP(2);  // every load is issued
   // ---- shrink: H[token, rank] partial over this wavefront's K range ----------------------------
   f32x4 acc[RB];
 #pragma unroll
@@ -324,130 +299,24 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // Sum the K-partials of the wavefronts.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
+  MLORA_STAMP(3);  // wavefront 0: x and A arrived, staged and multiplied
   __syncthreads();
-  if (kshift == 0) {
-    for (int e = tid; e < RB * 256; e += NT) {
-      const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-      float sum = 0.f;
+  MLORA_STAMP(4);  // every wavefront's partial is in LDS
+  for (int e = tid; e < RB * 256; e += NT) {
+    const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+    float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-      const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-      if (r < R) {
-        const float v = sum * scaling;
-        const T hi = from_f32<T>(v);
-        s_hi[tok * HSTRIDE + r] = hi;
-        s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
-      }
-    }
-  } else {
-    // This part's sums -> memory, then count the arrival (a workgroup only waits for its own
-    // stores to be acknowledged before it is counted).
-    constexpr int kArrive = 1, kDepart = 1 << 16;
-    const int P = 1 << kshift;
-    const int first = tile * gridDim.y + (group << kshift);  // first of the workgroups sharing this shrink
-    float* mine = partials + static_cast<int64_t>(first + kpart) * (16 * R);
-    for (int e = tid; e < RB * 256; e += NT) {
-      const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-      const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-      if (r < R) __hip_atomic_store(mine + tok * R + r, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    int32_t* ctr = counters + tile * MLORA_COOP_SPLITS + group;
-    if (tid == 0) {
-      int v = __hip_atomic_fetch_add(ctr, kArrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kArrive;
-      if (mode == 1) {
-        if (v == P) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      } else {
-        const long long t0 = wall_clock64();
-        while ((v & 0xffff) < P && wall_clock64() - t0 < spin_ticks) {
-          __builtin_amdgcn_s_sleep(2);
-          v = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (spin_ticks < 0) v = 0;  // diagnostic: never take the shortcut
-      }
-      s_arrived = (v & 0xffff) >= P;
-    }
-    __syncthreads();
-    if (s_arrived) {
-      const float* parts = partials + static_cast<int64_t>(first) * (16 * R);
-      for (int e = tid; e < 16 * R; e += NT) {
-        float sum = 0.f;
-        for (int kp = 0; kp < P; ++kp)
-          sum += __hip_atomic_load(parts + kp * (16 * R) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int tok = e / R, r = e % R;
-        const float v = sum * scaling;
-        const T hi = from_f32<T>(v);
-        s_hi[tok * HSTRIDE + r] = hi;
-        s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
-      }
-    } else if (mode == 1) {
-      return;  // someone else finishes this tile
-    } else {
-      // The other parts did not show up in time: compute every part here, with the same split
-      // of K over the wavefronts and the same order of additions as the workgroups that own them.
-      constexpr int EPT = (RB * 256 + NT - 1) / NT;
-      float total[EPT];
-#pragma unroll
-      for (int n = 0; n < EPT; ++n) total[n] = 0.f;
-      for (int kp = 0; kp < P; ++kp) {
-        const int b0 = kp * nks + (KSPW > 0 ? wave * KSPW : wave * nks / kNW);
-        const int b1 = KSPW > 0 ? b0 + KSPW : kp * nks + (wave + 1) * nks / kNW;
-        f32x4 part[RB];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) part[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int ks = b0; ks < b1; ++ks) {
-          Pack8 xv8, av8[RB];
-          xv8.raw = load128(xrow + ks * 32);
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb) av8[rb].raw = load128(arow[rb] + ks * 32);
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb) part[rb] = Mma<T>::run(xv8, av8[rb], part[rb]);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = part[rb];
-        __syncthreads();
-#pragma unroll
-        for (int n = 0; n < EPT; ++n) {
-          const int e = tid + n * NT;
-          if (e < RB * 256) {
-            const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-            float sum = 0.f;
-#pragma unroll
-            for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-            total[n] += sum;
-          }
-        }
-      }
-#pragma unroll
-      for (int n = 0; n < EPT; ++n) {
-        const int e = tid + n * NT;
-        if (e < RB * 256) {
-          const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-          const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-          if (r < R) {
-            const float v = total[n] * scaling;
-            const T hi = from_f32<T>(v);
-            s_hi[tok * HSTRIDE + r] = hi;
-            s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
-          }
-        }
-      }
-    }
-    if (mode == 2) {
-      __syncthreads();  // every thread is done with the exchanged parts
-      if (tid == 0) {
-        const int v = __hip_atomic_fetch_add(ctr, kDepart, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kDepart;
-        if (v == (P | (P << 16))) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      if (sp.n0 >= sp.n1) return;  // a part without columns of its own
+    for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+    const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+    if (r < R) {
+      const float v = r < eff ? sum * scaling : 0.f;  // ranks the adapter does not have contribute nothing
+      const T hi = from_f32<T>(v);
+      s_hi[tok * HSTRIDE + r] = hi;
+      s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
     }
   }
   __syncthreads();
+  MLORA_STAMP(5);  // the intermediate is in LDS
 
   // ---- expand ---------------------------------------------------------------------------------
   Pack8 hop[KSTEPS], hlo[KSTEPS];
@@ -551,6 +420,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       else finish_span(c0, bop[s], yreg[s]);
     }
   }
+  MLORA_STAMP(6);  // wavefront 0: its first spans are multiplied and their stores issued
   for (int c0 = sp.n0 + (wave + kSpansAhead * kNW) * 64; c0 < sp.n1; c0 += kNW * 64) {  // wide ranges
     Pack8 bo[4][KSTEPS], yy[2];
     if constexpr (TR) {
@@ -566,6 +436,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          if (eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
 #pragma unroll
@@ -574,12 +445,17 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       finish_span(c0, bo, yy);
     }
   }
+#ifdef MLORA_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  MLORA_STAMP(7);  // wavefront 0: its stores are acknowledged
+  __syncthreads();
+  MLORA_STAMP(8);  // every wavefront is done
+#endif
 }
 
 struct Launch {
   const MloraAddArgs* a;
-  int small_off, include_long, kshift, mode, spin_ticks, staged;
-  int32_t* counters;
+  int small_off, include_long, staged;
   dim3 grid;
   const DecodeSplits* splits;
 };
@@ -589,18 +465,17 @@ void launch_one(const Launch& l) {
   const MloraAddArgs* a = l.a;
   hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
-                     a->num_slots, a->scaling, l.kshift, l.mode, l.spin_ticks, l.counters, static_cast<float*>(a->workspace),
-                     *l.splits);
+                     a->num_slots, a->scaling, a->effective_rank, *l.splits);
 }
 
-// The steps-per-wavefront specialisations kept: 1, 2 and 4 (K or a part of K = 256, 512, 1024)
-// for every rank and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
+// The steps-per-wavefront specialisations kept: 1, 2 and 4 (K = 256, 512, 1024) for every rank
+// and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
   if (l.staged) {
     // staged operands, the k-steps of a wavefront four at a time (rank 64 in two passes of 32 ranks
     // through the same LDS block); how many k-steps fit is a matter of registers: every load of
-    // the workgroup's K part is issued before the first is used
+    // the workgroup's K range is issued before the first is used
     if (kspw == 4) return launch_one<T, R, 4, true>(l);
     if constexpr (R <= 32) {
       if (kspw == 8) return launch_one<T, R, 8, true>(l);
@@ -629,28 +504,32 @@ void launch_rank(const Launch& l, int r, int kspw) {
   }
 }
 
-// Largest power of two <= want that divides the k-steps into whole steps per wavefront and
-// whose partial sums (units x parts x 16 x r floats) fit the caller's workspace.
-int usable_parts(const MloraAddArgs* a, int want, long long units) {
-  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 15)) return 1;
-  const int nks = a->k / 32;
-  int parts = 1;
-  while (parts * 2 <= want) parts *= 2;
-  while (parts > 1) {
-    const size_t need = static_cast<size_t>(units) * parts * 16 * a->r * sizeof(float);
-    if (nks % (parts * kNW) == 0 && static_cast<size_t>(a->workspace_bytes) >= need) break;
-    parts /= 2;
+// Diagnostic knobs, read from the environment once per process.
+struct DecodeKnobs {
+  int generation = -1, staged, nt;
+  void read() {
+    generation = knob_generation();
+    staged = env_int("MLORA_DECODE_STAGED", 1);
+    nt = env_int("MLORA_DECODE_NT", 0);
   }
-  return parts;
-}
+};
 
 }  // namespace
 
-// Workspace that lets the small-tile form share a shrink between workgroups: room for 1024
-// partial tiles of 16 x r sums (sharing is only chosen for grids that fit).
-size_t decode_workspace_bytes(int r) { return static_cast<size_t>(1024) * 16 * r * sizeof(float); }
+// Nothing in the kernel limits the size of x or y.
+bool decode_supported(const MloraAddArgs*) { return true; }
+
+void decode_trace_set(void* buf) {
+#ifdef MLORA_TRACE
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(trace_buf), &buf, sizeof(buf));
+#else
+  (void)buf;
+#endif
+}
 
 int launch_decode(const MloraAddArgs* a, bool include_long) {
+  static DecodeKnobs knobs;
+  if (knobs.generation != knob_generation()) knobs.read();
   DecodeSplits splits;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
   int cap = lay.cap_small;
@@ -661,108 +540,53 @@ int launch_decode(const MloraAddArgs* a, bool include_long) {
   if (cap == 0) return 0;
   cap = (cap + 7) & ~7;
 
-  int live = 0;
-  for (int i = 0; i < a->num_slices; ++i) live += a->slices[i].n > 0;
-  if (live == 0) return 0;
-
   Launch l;
   l.a = a; l.small_off = lay.small_off; l.include_long = include_long ? 1 : 0; l.splits = &splits;
-  l.counters = a->plan + lay.coop_off;
-  l.spin_ticks = env_int("MLORA_DECODE_SPIN_TICKS", 20000);  // 200 us of the 100 MHz clock
-  l.kshift = 0;
-  l.mode = 0;
-  l.staged = env_int("MLORA_DECODE_STAGED", 1);
-  int total = 0;
+  l.staged = knobs.staged;
 
-  // Mode 2: the workgroups of a (tile, slice) each take one part of K and one part of the columns.
-  // The exchange costs a few trips through memory (about 2 us measured), which pays when K is
-  // long (6144 x 1536: 10.4 -> 7.7 us per launch at 32 tiles, 8192 x 2048: 12.9 -> 7.5; at 4096 x 1024
-  // the two are level since the staged loads reach sixteen k-steps per wavefront) and does not at
-  // K = 1024; at K = 2048 and 3072 it pays for wide outputs only (2048 -> 2 x 8192 columns:
-  // 11.1 -> 9.6 us, but 2048 -> 2048 4.7 -> 6.0, 3072 -> 3072 5.9 -> 6.8, and three slices of 3072
-  // columns 5.5 -> 8.6).
-  int mode = env_int("MLORA_DECODE_MODE", -1);
-  const int want = env_int("MLORA_DECODE_KPARTS", 0);
-  long long all_cols = 0;
-  for (int i = 0; i < a->num_slices; ++i) all_cols += a->slices[i].n;
-  if (mode == 2 || (mode < 0 && (a->k >= 4096 || (a->k >= 2048 && all_cols >= 8192)))) {
-    int parts = 1;
-    if (live == a->num_slices && live <= MLORA_COOP_SPLITS) parts = usable_parts(a, want > 0 ? want : 4, static_cast<long long>(cap) * live);
-    if (parts > 1 && (mode == 2 || static_cast<long long>(cap) * live * parts <= 1024)) {
-      int s = 0;
-      for (int i = 0; i < a->num_slices; ++i) {
-        const MloraSlice& sl = a->slices[i];
-        const int w = ((sl.n + parts - 1) / parts + 63) & ~63;  // columns per part, whole 64-column spans
-        for (int j = 0; j < parts; ++j) {
-          DecodeSplit& d = splits.split[s++];
-          d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
-          d.n0 = j * w < sl.n ? j * w : sl.n;
-          d.n1 = (j + 1) * w < sl.n ? (j + 1) * w : sl.n;
-        }
-      }
-      total = s;
-      l.mode = 2;
-      while ((1 << l.kshift) < parts) ++l.kshift;
-    } else if (mode == 2) {
-      mode = 0;
+  // Column range per workgroup.  Every range repeats the shrink of its tile, but a compute unit
+  // takes in only 30-60 bytes per cycle even from the L2, so a launch is fastest when its
+  // bytes are spread over 150-250 workgroups: ranges shrink down to 128 columns for narrow
+  // projections and stay at 1024 (two 64-column spans per wavefront, all loads still in
+  // registers) for wide ones.  Measured per launch at 32 tiles: o 6.2 us at 1024 columns,
+  // 5.1 at 512, 4.7 at 256; gate_up 8.2 / 8.9 / 11.1.
+  int nt = knobs.nt;
+  if (nt <= 0) {
+    long long cols = 0;
+    for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+    const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
+    const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
+    const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
+    nt = static_cast<int>(cols * tiles / 160);
+    if (nt > 1024) nt = 1024;
+    if (nt < 128) nt = 128;
+  }
+  if (nt < 64) nt = 64;
+  nt = (nt + 63) & ~63;
+  int total = 0;
+  for (;;) {
+    total = 0;
+    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
+    if (total <= kMaxSplits) break;
+    nt *= 2;
+  }
+  if (total == 0) return 0;
+  int s = 0;
+  for (int i = 0; i < a->num_slices; ++i) {
+    const MloraSlice& sl = a->slices[i];
+    for (int n0 = 0; n0 < sl.n; n0 += nt) {
+      DecodeSplit& d = splits.split[s++];
+      d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
+      d.n0 = n0; d.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
     }
   }
-  if (l.mode == 0) {
-    // Column range per workgroup.  Every range repeats the shrink of its tile, but a compute unit
-    // takes in only 30-60 bytes per cycle even from the L2, so a launch is fastest when its
-    // bytes are spread over 150-250 workgroups: ranges shrink down to 128 columns for narrow
-    // projections and stay at 1024 (two 64-column spans per wavefront, all loads still in
-    // registers) for wide ones.  Measured per launch at 32 tiles: o 6.2 us at 1024 columns,
-    // 5.1 at 512, 4.7 at 256; gate_up 8.2 / 8.9 / 11.1.
-    int nt = env_int("MLORA_DECODE_NT", 0);
-    if (nt <= 0) {
-      long long cols = 0;
-      for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
-      const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
-      const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
-      const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
-      nt = static_cast<int>(cols * tiles / 160);
-      if (nt > 1024) nt = 1024;
-      if (nt < 128) nt = 128;
-    }
-    if (nt < 64) nt = 64;
-    nt = (nt + 63) & ~63;
-    for (;;) {
-      total = 0;
-      for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
-      if (total <= kMaxSplits) break;
-      nt *= 2;
-    }
-    if (total == 0) return 0;
-    int s = 0;
-    for (int i = 0; i < a->num_slices; ++i) {
-      const MloraSlice& sl = a->slices[i];
-      for (int n0 = 0; n0 < sl.n; n0 += nt) {
-        DecodeSplit& d = splits.split[s++];
-        d.a = sl.a; d.b = sl.b; d.n = sl.n; d.y_col = sl.y_col;
-        d.n0 = n0; d.n1 = n0 + nt < sl.n ? n0 + nt : sl.n;
-      }
-    }
-    // Mode 1: workgroups sharing the shrink of a (tile, column range), the last one finishing it.
-    // Only worth its extra round trip through memory when a workgroup would otherwise pull a long
-    // K through a single compute unit while most of the chip idles.
-    if ((mode == 1 || mode < 0) && total <= MLORA_COOP_SPLITS) {
-      int parts = 1;
-      if (want > 0) parts = want;
-      else if (a->k >= 2048 && static_cast<long long>(cap) * total <= 128) parts = 4;
-      parts = usable_parts(a, parts, static_cast<long long>(cap) * total);
-      if (parts > 1) {
-        l.mode = 1;
-        while ((1 << l.kshift) < parts) ++l.kshift;
-      }
-    }
-  }
-  l.grid = dim3(8, static_cast<unsigned>(l.mode == 2 ? total : total << l.kshift), static_cast<unsigned>(cap / 8));
-  const int nks = (a->k / 32) >> l.kshift;
+  for (; s < kMaxSplits; ++s) splits.split[s] = DecodeSplit{nullptr, nullptr, 0, 0, 0, 0};
+  l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>(cap / 8));
+  const int nks = a->k / 32;
   const int kspw = (nks % kNW == 0) ? nks / kNW : 0;
   if (a->dtype == MLORA_DTYPE_BF16) launch_rank<__bf16>(l, a->r, kspw);
   else launch_rank<_Float16>(l, a->r, kspw);
-  return check_launch("mlora_add_lora(small tiles, mfma)");
+  return check_launch("mlora_add_lora(small tiles, one workgroup per column range)");
 }
 
 }  // namespace mlora

@@ -1,11 +1,16 @@
 // Internal launch entry points shared by the C-ABI front door.
 #pragma once
 
+#include <hip/hip_runtime.h>
+
 #include "mlora.h"
 
 namespace mlora {
 
 int env_int(const char* name, int fallback);
+// Diagnostic knobs are read from the environment once and kept; mlora_reload_knobs() advances
+// this number, and a holder whose copy is older reads its variables again.
+int knob_generation();
 
 // token.hip: one workgroup per token; needs only token_to_slot.
 int launch_token_add(const MloraAddArgs* a);
@@ -14,9 +19,17 @@ int launch_token_add(const MloraAddArgs* a);
 // whether the small tiles of segments at or above the threshold are walked too.
 int launch_bgmv(const MloraAddArgs* a, bool include_long);
 
-// decode.hip: the same small tiles with both products on the matrix cores.
+// decode.hip: the same small tiles with both products on the matrix cores, one workgroup per
+// (tile, column range).
+bool decode_supported(const MloraAddArgs* a);  // x and y below 2 GiB each
 int launch_decode(const MloraAddArgs* a, bool include_long);
-size_t decode_workspace_bytes(int r);
+
+// split.hip: the same small tiles, producers and consumers of the intermediate in one launch.
+// trusted_workspace: the head of the workspace is known to be in its initial or a left-behind
+// state without carrying the signature (the library's own zero-initialised array).
+bool split_supported(const MloraAddArgs* a);
+int launch_split(const MloraAddArgs* a, bool include_long, bool trusted_workspace);
+int workspace_init(void* workspace, hipStream_t stream);
 
 // sgmv.hip: 64-token MFMA tiles of the segments at or above the threshold, as a shrink launch
 // and an expand launch that meet in the caller's workspace.
@@ -24,5 +37,9 @@ bool sgmv_supported(const MloraAddArgs* a);
 bool sgmv_workspace_ok(const MloraAddArgs* a);
 size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype);
 int launch_sgmv(const MloraAddArgs* a);
+
+// in-kernel timeline of trace builds (no-ops otherwise)
+void decode_trace_set(void* buf);
+void split_trace_set(void* buf);
 
 }  // namespace mlora

@@ -202,8 +202,8 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
     if (p.compact_offsets) p.compact_offsets[i + 1] = 0;
   }
 
-  // Tile lists of the plan.  A small-tile record starts with its header and sixteen zeroed row
-  // entries; the scatter below overwrites the entries that exist.
+  // Tile lists of the plan.  A small-tile record starts with its header and zeroed row entries;
+  // the scatter below fills all sixteen (the tile's tokens, repeated cyclically past its count).
   i32x4* small = p.plan ? reinterpret_cast<i32x4*>(p.plan + lay.small_off) : nullptr;
   if (p.plan) {
     i32x4* big = reinterpret_cast<i32x4*>(p.plan + lay.big_off);
@@ -225,7 +225,6 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       int left = c - j * MLORA_TILE_BIG;
       big[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
     }
-    for (int i = tid; i < MLORA_COOP_SPLITS * lay.cap_small; i += kMetaThreads) p.plan[lay.coop_off + i] = 0;
   }
   __syncthreads();
 
@@ -260,7 +259,13 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
           plan_sorted[off[key] + r] = t;
           const int c = total[key];
           const int q = (c < MLORA_SEGMENT_THRESHOLD ? ts_short[key] : n_short + ts_long[key]) + r / MLORA_TILE_SMALL;
-          p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (r % MLORA_TILE_SMALL)] = t;
+          // the token's own entry, and every entry past the tile's count that repeats it: a tile of
+          // n < 16 tokens lists them cyclically, so that a kernel which fetches all sixteen rows
+          // touches no memory beyond the rows of the tile itself
+          const int left = c - (r / MLORA_TILE_SMALL) * MLORA_TILE_SMALL;
+          const int n = left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL;
+          for (int pos = r % MLORA_TILE_SMALL; pos < MLORA_TILE_SMALL; pos += n)
+            p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + pos] = t;
         }
         if (p.sorted_idx) p.sorted_idx[n_neg + off[key] + r] = t;
       } else if (p.sorted_idx) {

@@ -42,18 +42,6 @@ constexpr int kMaxSplits = 64;
 constexpr int kExpandWaves = 4;
 constexpr int kMaxKSplit = 4;  // most K parts the shrink ever uses (the workspace has room for them)
 
-template <typename T> struct Mma;
-template <> struct Mma<__bf16> {
-  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.bf, b.bf, c, 0, 0, 0);
-  }
-};
-template <> struct Mma<_Float16> {
-  static __device__ __forceinline__ f32x4 run(const Pack8& a, const Pack8& b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.hf, b.hf, c, 0, 0, 0);
-  }
-};
-
 struct ShrinkSlices {
   const void* a[MLORA_MAX_SLICES];
 };
@@ -509,6 +497,34 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   }
 }
 
+// The fp32 partials of the intermediate live behind the head of the workspace.
+float* partials_of(const MloraAddArgs* a) { return reinterpret_cast<float*>(static_cast<char*>(a->workspace) + MLORA_WORKSPACE_HEAD_BYTES); }
+size_t partials_room(const MloraAddArgs* a) {
+  return a->workspace_bytes > MLORA_WORKSPACE_HEAD_BYTES ? static_cast<size_t>(a->workspace_bytes) - MLORA_WORKSPACE_HEAD_BYTES : 0;
+}
+
+// Diagnostic knobs, read from the environment once and again after mlora_reload_knobs().
+struct SgmvKnobs {
+  int generation = -1, nt_hint, kr, ksplit, all_slices, xdb, group, wgs, nt, cpl;
+  void read() {
+    generation = knob_generation();
+    nt_hint = env_int("MLORA_SGMV_NT_HINT", 0);
+    kr = env_int("MLORA_SGMV_KR", 0);
+    ksplit = env_int("MLORA_SGMV_KSPLIT", 0);
+    all_slices = env_int("MLORA_SGMV_ALL_SLICES", 3);
+    xdb = env_int("MLORA_SGMV_XDB", 1);
+    group = env_int("MLORA_SGMV_GROUP", 0);
+    wgs = env_int("MLORA_SGMV_WGS", 2048);
+    nt = env_int("MLORA_SGMV_NT", 0);
+    cpl = env_int("MLORA_SGMV_CPL", 8);
+  }
+};
+const SgmvKnobs& sgmv_knobs() {
+  static SgmvKnobs k;
+  if (k.generation != knob_generation()) k.read();
+  return k;
+}
+
 struct ShrinkLaunch {
   const MloraAddArgs* a;
   PlanLayout lay;
@@ -523,7 +539,7 @@ void launch_shrink_one(const ShrinkLaunch& l) {
   const MloraAddArgs* a = l.a;
   dim3 grid(8, static_cast<unsigned>(l.all_slices ? l.ksplit : a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
   hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR, XW, DB>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
-                     a->plan, a->x, static_cast<float*>(a->workspace), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
+                     a->plan, a->x, partials_of(a), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
                      l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, l.sl);
 }
 
@@ -550,8 +566,8 @@ template <typename T, int R>
 void launch_expand_group(const MloraAddArgs* a, const PlanLayout& lay, int big_units, dim3 grid, int ksplit, int cpl, int group,
                          const ExpandSplits& sp) {
   hipStream_t st = static_cast<hipStream_t>(a->stream);
-  const float* h = static_cast<const float*>(a->workspace);
-  const int nt = env_int("MLORA_SGMV_NT_HINT", 0);
+  const float* h = partials_of(a);
+  const int nt = sgmv_knobs().nt_hint;
 #define MLORA_EXPAND(CPL_, TPF_, G_)                                                                                       \
   hipLaunchKernelGGL((sgmv_expand_kernel<T, R, CPL_, TPF_, G_>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, \
                      a->y_stride, lay.big_off, lay.small_off, big_units, lay.sorted_off, a->num_tokens, a->num_slots,      \
@@ -608,17 +624,17 @@ static size_t partial_bytes(int num_tokens, int num_slices, int r) {
 size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype) {
   (void)dtype;
   if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
-  return kMaxKSplit * partial_bytes(num_tokens, num_slices, r);
+  return MLORA_WORKSPACE_HEAD_BYTES + kMaxKSplit * partial_bytes(num_tokens, num_slices, r);
 }
 
 bool sgmv_supported(const MloraAddArgs* a) { return a->k % 128 == 0 && a->k >= 128; }
 
 // A workspace that holds at least one partial can be used (fewer K parts are taken then).
 bool sgmv_workspace_ok(const MloraAddArgs* a) {
-  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 15)) return false;
+  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 255)) return false;
   for (int i = 0; i < a->num_slices; ++i)
     if (a->slices[i].n <= 0) return false;  // every slice owns a workspace column block
-  return a->workspace_bytes > 0 && static_cast<size_t>(a->workspace_bytes) >= partial_bytes(a->num_tokens, a->num_slices, a->r);
+  return partials_room(a) >= partial_bytes(a->num_tokens, a->num_slices, a->r);
 }
 
 // Every segment of the batch: 64-token tiles of the long ones, one short tile each for the rest.
@@ -647,12 +663,12 @@ int launch_sgmv(const MloraAddArgs* a) {
   // workgroups per compute unit
   int xw = 512;
   while (xw > 128 && a->k % xw != 0) xw /= 2;
-  int kr = env_int("MLORA_SGMV_KR", 0);
+  int kr = sgmv_knobs().kr;
   if (kr != 128 && kr != 256 && kr != 512) kr = xw;
   if (kr > xw) kr = xw;
   if (kr == 128) xw = 128;  // 128-column slabs come with 128-column batches only
-  const int max_parts = static_cast<int>(static_cast<size_t>(a->workspace_bytes) / partial_bytes(a->num_tokens, a->num_slices, a->r));
-  int ksplit = env_int("MLORA_SGMV_KSPLIT", 0);
+  const int max_parts = static_cast<int>(partials_room(a) / partial_bytes(a->num_tokens, a->num_slices, a->r));
+  int ksplit = sgmv_knobs().ksplit;
   if (ksplit <= 0) {
     ksplit = 1;
     while (ksplit < kMaxKSplit && static_cast<long long>(est_tiles) * a->num_slices * ksplit < 512 && a->k % (xw * ksplit * 2) == 0) ksplit *= 2;
@@ -664,7 +680,7 @@ int launch_sgmv(const MloraAddArgs* a) {
   // its K part is a single batch (measured on the prefill batch: qkv 31.9 -> 29.6 us per call;
   // with two slices the shorter chain of separate workgroups wins, gate_up 76.6 vs 77.8)
   l.all_slices = 0;
-  if (a->num_slices >= env_int("MLORA_SGMV_ALL_SLICES", 3)) {
+  if (a->num_slices >= sgmv_knobs().all_slices) {
     const int parts = a->k / xw;
     if (parts <= kMaxKSplit && parts <= max_parts) {
       ksplit = parts;
@@ -674,7 +690,7 @@ int launch_sgmv(const MloraAddArgs* a) {
   l.ksplit = ksplit;
   l.krange = a->k / ksplit;
   // a K part of several batches: the form with two x buffers (256-column batches)
-  if (xw == 512 && l.krange > xw && env_int("MLORA_SGMV_XDB", 1)) { xw = 256; kr = 256; }
+  if (xw == 512 && l.krange > xw && sgmv_knobs().xdb) { xw = 256; kr = 256; }
   if (a->dtype == MLORA_DTYPE_BF16) launch_shrink_rank<__bf16>(l, kr, xw);
   else launch_shrink_rank<_Float16>(l, kr, xw);
   int rc = check_launch("mlora_add_lora(sgmv shrink)");
@@ -683,16 +699,16 @@ int launch_sgmv(const MloraAddArgs* a) {
   // expand: consecutive tiles per workgroup (they share their B rows when they share their
   // slot), then column ranges so that the grid has about 2048 workgroups
   ExpandSplits splits;
-  int group = env_int("MLORA_SGMV_GROUP", 0);
+  int group = sgmv_knobs().group;
   if (group != 1 && group != 2 && group != 4) group = (cols >= 4096 && est_tiles >= 64) ? 4 : 1;  // wide projections only: narrow ones need the workgroups
-  const int target = env_int("MLORA_SGMV_WGS", 2048);
-  int nt = env_int("MLORA_SGMV_NT", 0);
+  const int target = sgmv_knobs().wgs;
+  int nt = sgmv_knobs().nt;
   if (nt <= 0) {
     const long long want = static_cast<long long>(cols) * (est_tiles / group + 1) / (target > 0 ? target : 1);
     nt = want > 8192 ? 8192 : static_cast<int>(want);
   }
   const int nsplit = fill_splits(a, nt, splits.split);
-  const int cpl = env_int("MLORA_SGMV_CPL", 8) == 4 ? 4 : 8;
+  const int cpl = sgmv_knobs().cpl == 4 ? 4 : 8;
   const int big_units = l.big_cap / group;  // big_cap is a multiple of 32: a multiple of 8 again
   const int units = big_units + (l.tiles8 * 8 - l.big_cap);
   dim3 grid(8, static_cast<unsigned>(nsplit), static_cast<unsigned>(units / 8));

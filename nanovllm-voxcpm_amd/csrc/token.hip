@@ -280,6 +280,15 @@ extern "C" int mlora_install_slot(const MloraInstallArgs* a) {
     set_error("mlora_install_slot: bad sizes (slot=%d k=%d n=%d r=%d rank=%d)", a->slot, a->k, a->n, a->r, a->rank);
     return MLORA_E_INVALID;
   }
+  if (a->slot >= a->num_slots) {
+    set_error("mlora_install_slot: slot %d is outside the %d slots of the buffers", a->slot, a->num_slots);
+    return MLORA_E_INVALID;
+  }
+  if (a->rank > 0 && (a->a_src_stride < a->k || a->b_src_stride < a->rank)) {
+    set_error("mlora_install_slot: source row strides (%lld, %lld) are shorter than the rows they carry (%d, %d)",
+              static_cast<long long>(a->a_src_stride), static_cast<long long>(a->b_src_stride), a->k, a->rank);
+    return MLORA_E_INVALID;
+  }
   if (!valid_dtype(a->dtype) || !valid_dtype(a->src_dtype)) { set_error("mlora_install_slot: unknown dtype"); return MLORA_E_INVALID; }
   if (!a->a_dst || !a->b_dst || (a->rank > 0 && (!a->a_src || !a->b_src))) { set_error("mlora_install_slot: NULL pointer"); return MLORA_E_INVALID; }
   const int64_t total = static_cast<int64_t>(a->r) * a->k + static_cast<int64_t>(a->n) * a->r;

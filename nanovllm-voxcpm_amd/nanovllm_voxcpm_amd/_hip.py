@@ -22,8 +22,8 @@ MAX_SLOTS = 1024
 MAX_RANK = 256
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
-FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA = 0, 1, 2, 3, 4
-FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA}
+FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT = 0, 1, 2, 3, 4, 5
+FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA, "split": FORM_SPLIT}
 
 PLAN_HEADER_WORDS = 16
 (
@@ -43,6 +43,8 @@ PLAN_MAGIC_VALUE = 0x4D4C5031
 SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 16, 64
 SMALL_TILE_WORDS, SMALL_TILE_ROWS, BIG_TILE_WORDS = 32, 4, 4
 STATIC_SCRATCH_BYTES = 16 << 20
+WORKSPACE_HEAD_BYTES = 16384 + (1 << 20)
+WORKSPACE_TIMEOUTS_WORD = 1  # uint32 index in the workspace head: waits of the split form that ran out
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 
@@ -50,12 +52,15 @@ EXPORTS = (
     "mlora_add_lora",
     "mlora_add_lora_static",
     "mlora_add_workspace_bytes",
+    "mlora_workspace_init",
     "mlora_shrink",
     "mlora_expand",
     "mlora_plan_workspace_bytes",
     "mlora_meta_build",
     "mlora_install_slot",
     "mlora_stream_capture_id",
+    "mlora_reload_knobs",
+    "mlora_trace_set",
     "mlora_abi_version",
     "mlora_last_error",
     "mlora_build_info",
@@ -86,6 +91,7 @@ class MloraAddArgs(C.Structure):
         ("slices", MloraSlice * MAX_SLICES),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_int64),
+        ("effective_rank", C.c_void_p),
     ]
 
 
@@ -166,6 +172,7 @@ class MloraInstallArgs(C.Structure):
         ("dtype", C.c_int32),
         ("src_dtype", C.c_int32),
         ("scaling", C.c_float),
+        ("num_slots", C.c_int32),
     ]
 
 
@@ -212,8 +219,14 @@ def load() -> C.CDLL:
     lib.mlora_plan_workspace_bytes.restype = C.c_size_t
     lib.mlora_add_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
     lib.mlora_add_workspace_bytes.restype = C.c_size_t
+    lib.mlora_workspace_init.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
+    lib.mlora_workspace_init.restype = C.c_int
     lib.mlora_stream_capture_id.argtypes = [C.c_void_p]
     lib.mlora_stream_capture_id.restype = C.c_uint64
+    lib.mlora_trace_set.argtypes = [C.c_void_p]
+    lib.mlora_trace_set.restype = C.c_int
+    lib.mlora_reload_knobs.argtypes = []
+    lib.mlora_reload_knobs.restype = None
     lib.mlora_abi_version.argtypes = []
     lib.mlora_abi_version.restype = C.c_int
     lib.mlora_last_error.argtypes = []
@@ -280,8 +293,19 @@ def plan_workspace_words(num_tokens: int, max_slots: int) -> int:
 
 
 def add_workspace_bytes(num_tokens: int, num_slices: int, r: int, dtype: torch.dtype) -> int:
-    """Bytes of scratch that let the fused apply use the two-launch form for long segments."""
+    """Bytes of scratch that let the fused apply use every form it has for this shape."""
     return int(load().mlora_add_workspace_bytes(num_tokens, num_slices, r, dtype_code(dtype)))
+
+
+def workspace_init(workspace: torch.Tensor, stream: int | None = None) -> None:
+    """Clear the head of a freshly allocated workspace and write its signature (one kernel on
+    ``stream``, torch's current one when omitted)."""
+    lib = load()
+    _require_cuda(workspace, "workspace")
+    nbytes = workspace.numel() * workspace.element_size()
+    with _on(workspace.device):
+        _check(lib.mlora_workspace_init(workspace.data_ptr(), nbytes, _stream(workspace.device) if stream is None else stream),
+               "mlora_workspace_init")
 
 
 def add_lora(
@@ -297,11 +321,14 @@ def add_lora(
     workspace: torch.Tensor | None = None,
     stream: int | None = None,
     static_scratch: bool = False,
+    effective_rank: torch.Tensor | None = None,
 ) -> None:
     """y[:, col_i : col_i + n_i] += scaling * (x . A_i[slot]^T) . B_i[slot]^T for every slice.
     ``stream``: handle of the stream to launch on, torch's current one when omitted.
     ``static_scratch``: call the entry point that allocates nothing and keeps its scratch in the
-    library's own device image (``workspace`` is ignored then)."""
+    library's own device image (``workspace`` is ignored then).
+    ``effective_rank``: int32 [slots] on the device, rank of the adapter resident in each slot of
+    these buffers; rows / columns at or above it are then neither read nor multiplied."""
     lib = load()
     _require_cuda(x, "x")
     if len(a_slices) > MAX_SLICES:
@@ -331,6 +358,12 @@ def add_lora(
     if workspace is not None:
         args.workspace = workspace.data_ptr()
         args.workspace_bytes = workspace.numel() * workspace.element_size()
+    if effective_rank is not None:
+        if effective_rank.dtype != torch.int32 or not effective_rank.is_contiguous() or effective_rank.numel() < args.num_slots:
+            raise ValueError("effective_rank must be a contiguous int32 tensor with one entry per slot")
+        if effective_rank.device != x.device:
+            raise ValueError("effective_rank must live on the device of x")
+        args.effective_rank = effective_rank.data_ptr()
     with _on(x.device):
         if static_scratch:
             _check(lib.mlora_add_lora_static(C.byref(args)), "mlora_add_lora_static")
@@ -468,6 +501,7 @@ def install_slot(
     args.dtype = dtype_code(a_dst.dtype)
     args.src_dtype = dtype_code(a_src.dtype)
     args.scaling = scaling
+    args.num_slots = a_dst.size(0)
     with _on(a_dst.device):
         _check(lib.mlora_install_slot(C.byref(args)), "mlora_install_slot")
 
@@ -476,6 +510,17 @@ def stream_capture_id(device: torch.device, stream: int | None = None) -> int:
     """Identifier of the graph capture in progress on ``stream`` (torch's current stream on
     ``device`` when omitted), 0 when none."""
     return int(load().mlora_stream_capture_id(_stream(device) if stream is None else stream))
+
+
+def reload_knobs() -> None:
+    """Make the library read its MLORA_* environment variables again (it keeps them otherwise)."""
+    load().mlora_reload_knobs()
+
+
+def trace_set(buf: torch.Tensor | None) -> None:
+    """Hand the trace build of the library a zeroed uint64 [workgroups, 16] buffer to record
+    in-kernel timelines into (None switches recording off).  Raises with the regular build."""
+    _check(load().mlora_trace_set(buf.data_ptr() if buf is not None else None), "mlora_trace_set")
 
 
 def build_info() -> str:

@@ -179,7 +179,8 @@ class HipLoRABackend:
         if buf is None or buf.numel() < nbytes:
             if len(self._scratch) >= 8:
                 self._scratch.clear()
-            buf = self._scratch[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=x.device)
+            buf = self._scratch[key] = torch.empty(max(nbytes, 4 << 20), dtype=torch.uint8, device=x.device)
+            _hip.workspace_init(buf, stream)  # one kernel, once per buffer: head cleared, signature written
         return buf
 
     @staticmethod

@@ -36,3 +36,8 @@ def _clean_lora_state():
     yield
     reset_lora_context()
     set_backend_for_testing(None)
+    # environment changes of the test are undone by now: let the library drop what it read
+    from nanovllm_voxcpm_amd import _hip
+
+    if _hip.load_error() is None:
+        _hip.reload_knobs()

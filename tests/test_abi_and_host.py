@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     assert declared and set(declared) == set(_hip.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mlora_abi_version() == int(re.search(r"#define MLORA_ABI_VERSION (\d+)", HEADER.read_text()).group(1)) == 2
+    assert lib.mlora_abi_version() == int(re.search(r"#define MLORA_ABI_VERSION (\d+)", HEADER.read_text()).group(1)) == 3
     assert "gfx950" in _hip.build_info()
 
 
@@ -64,8 +64,10 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
     text = HEADER.read_text()
     for macro, value in (("MLORA_MAX_SLICES", 8), ("MLORA_MAX_SLOTS", _hip.MAX_SLOTS), ("MLORA_MAX_RANK", _hip.MAX_RANK),
                          ("MLORA_TILE_SMALL", 16), ("MLORA_SMALL_TILE_WORDS", _hip.SMALL_TILE_WORDS), ("MLORA_BIG_TILE_WORDS", _hip.BIG_TILE_WORDS), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
-                         ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS)):
+                         ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS), ("MLORA_FORM_SPLIT", _hip.FORM_SPLIT)):
         assert re.search(rf"#define {macro} {value}\b", text), macro
+    assert re.search(r"#define MLORA_WORKSPACE_HEAD_BYTES \(16384 \+ \(1 << 20\)\)", text) and _hip.WORKSPACE_HEAD_BYTES == 16384 + (1 << 20)
+    assert re.search(r"#define MLORA_STATIC_SCRATCH_BYTES \(16u << 20\)", text) and _hip.STATIC_SCRATCH_BYTES == 16 << 20
 
 
 def test_arguments_are_rejected_before_any_launch():
@@ -102,6 +104,20 @@ def test_arguments_are_rejected_before_any_launch():
     meta.max_slots, meta.num_tokens = 4, 3
     assert lib.mlora_meta_build(C.byref(meta)) == -1  # NULL token_to_slot with tokens
     assert lib.mlora_shrink(None) == -1 and lib.mlora_expand(None) == -1 and lib.mlora_install_slot(None) == -1
+    # slot install: a slot beyond the buffers and source rows shorter than what they carry are refused
+    inst = _hip.MloraInstallArgs()
+    inst.a_dst, inst.b_dst, inst.a_src, inst.b_src = 0x1000, 0x2000, 0x3000, 0x4000
+    inst.k, inst.n, inst.r, inst.rank, inst.num_slots, inst.slot = 64, 32, 16, 8, 4, 4
+    inst.a_src_stride, inst.b_src_stride, inst.dtype, inst.src_dtype = 64, 8, 2, 0
+    assert lib.mlora_install_slot(C.byref(inst)) == -1 and b"outside the 4 slots" in lib.mlora_last_error()
+    inst.slot, inst.a_src_stride = 3, 32
+    assert lib.mlora_install_slot(C.byref(inst)) == -1 and b"row strides" in lib.mlora_last_error()
+    inst.a_src_stride, inst.rank = 64, 17
+    assert lib.mlora_install_slot(C.byref(inst)) == -1 and b"bad sizes" in lib.mlora_last_error()
+    # workspace initialisation: alignment and the minimum size are checked before any launch
+    assert lib.mlora_workspace_init(0x1010, 1 << 22, None) == -1 and b"aligned" in lib.mlora_last_error()
+    assert lib.mlora_workspace_init(0x1000, 4096, None) == -1 and b"MLORA_WORKSPACE_HEAD_BYTES" in lib.mlora_last_error()
+    assert lib.mlora_add_workspace_bytes(256, 3, 16, 2) == _hip.WORKSPACE_HEAD_BYTES + 4 * 256 * 3 * 16 * 4
     assert lib.mlora_plan_workspace_bytes(256, 32) == 4 * _hip.plan_workspace_words(256, 32) > 0
     assert lib.mlora_plan_workspace_bytes(-1, 2) == 0
 

@@ -18,6 +18,27 @@ pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-2, 1e-3  # stated for bf16 outputs with fp32 accumulation
 
 
+def _knobs(monkeypatch, **env):
+    """Set (or, with None, unset) diagnostic MLORA_* variables and make the library read them."""
+    from nanovllm_voxcpm_amd import _hip
+
+    for key, value in env.items():
+        if value is None:
+            monkeypatch.delenv(key, raising=False)
+        else:
+            monkeypatch.setenv(key, str(value))
+    _hip.reload_knobs()
+
+
+def _waits_run_out(backend) -> int:
+    """Waits of the split form that ran out, summed over the backend's scratch buffers."""
+    from nanovllm_voxcpm_amd import _hip
+
+    torch.cuda.synchronize()
+    return sum(int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
+               for buf in backend._scratch.values())
+
+
 def _backend(form="auto"):
     from nanovllm_voxcpm_amd.lora import HipLoRABackend
 
@@ -110,7 +131,7 @@ def test_config1_fp32_matches_reference_torch_loop():
 # ---- config 2: decode, 256 tokens, 32 adapters of rank 16 -----------------------------------------
 
 
-@pytest.mark.parametrize("form", ["auto", "bgmv", "mfma", "sgmv", "token"])
+@pytest.mark.parametrize("form", ["auto", "bgmv", "mfma", "split", "sgmv", "token"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 def test_config2_decode_bf16(name, form):
     from nanovllm_voxcpm_amd import synthetic
@@ -124,23 +145,22 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
-@pytest.mark.parametrize("mode", [1, 2])
-@pytest.mark.parametrize("parts", [1, 2, 4, 8])
-@pytest.mark.parametrize("name,rank", [("down", 16), ("down", 64), ("qkv", 16), ("gate_up", 8)])
-def test_shrink_shared_between_workgroups(name, rank, parts, mode, monkeypatch):
-    """Small-tile form with the shrink of a tile split over several workgroups.  Mode 1: the last
-    one to arrive adds the parts up and does the expand.  Mode 2: every workgroup waits (bounded)
-    for the parts and expands its own columns; with the wait disabled from the host every
-    workgroup takes the path that computes all parts itself.  Checked: parity for every part
-    count, bit-identical results from one launch to the next and between the waiting and the
-    non-waiting path (the order of the sum is fixed, whatever the timing), slot -1 rows untouched,
-    and the arrival counters back at zero after every launch."""
-    from nanovllm_voxcpm_amd import synthetic
-    from nanovllm_voxcpm_amd.lora import _PLAN_ATTR
+@pytest.mark.parametrize("wide", [7, 8])
+@pytest.mark.parametrize("kpart", [512, 1024])
+@pytest.mark.parametrize("name,rank", [("down", 16), ("down", 64), ("qkv", 16), ("gate_up", 8), ("o", 32)])
+def test_split_form_producers_and_consumers(name, rank, kpart, wide, monkeypatch):
+    """Small-tile form with the two products in different workgroups of one launch: producers
+    publish the partial sums of their K part in the workspace, consumers pick them up (bounded
+    wait) and expand their column range; a consumer whose wait runs out computes the sums itself.
+    Checked: parity for both K-part widths and both access scopes, bit-identical results from one
+    launch to the next and between accepting published sums, never accepting them and not waiting
+    at all (the order of every sum is fixed, whatever the timing), slot -1 rows untouched, no wait
+    running out in the ordinary runs, every tile's arrival count back at zero after each launch,
+    and the same result from a workspace that was never initialised."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
 
-    print(f"shared shrink {name} r={rank} parts={parts} mode={mode}", flush=True)
-    monkeypatch.setenv("MLORA_DECODE_KPARTS", str(parts))
-    monkeypatch.setenv("MLORA_DECODE_MODE", str(mode))
+    print(f"split form {name} r={rank} kpart={kpart} wide={wide}", flush=True)
+    _knobs(monkeypatch, MLORA_SPLIT_KPART=kpart, MLORA_SPLIT_WIDE=wide, MLORA_SPLIT_W=128 if name == "qkv" else None)
     proj = _make(name, 12, rank, torch.bfloat16, seed=130 + rank)
     T = 90
     x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=131, device="cuda")
@@ -148,24 +168,37 @@ def test_shrink_shared_between_workgroups(name, rank, parts, mode, monkeypatch):
     slots = torch.randint(-1, 12, (T,), generator=g, dtype=torch.int32)
     slots[:20] = 3  # one segment above the threshold: two small tiles of the same slot
     slots = slots.cuda()
-    backend = _backend("mfma")
+    backend = _backend("split")
     meta = _metadata(slots)
-    runs = []
-    for spin in ("20000", "20000", "-1", "0"):
-        monkeypatch.setenv("MLORA_DECODE_SPIN_TICKS", spin)
+
+    def run():
         y = y0.clone()
         blocks = list(y.split(proj.widths, dim=-1))
         backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0,
                          y_packed=y if len(blocks) > 1 else None)
-        runs.append(y)
+        return y
+
+    runs = []
+    for spin in (20000, 20000, -1, 0):
+        _knobs(monkeypatch, MLORA_SPLIT_SPIN_TICKS=spin)
+        runs.append(run())
+        if spin > 0:
+            assert _waits_run_out(backend) == 0, "a consumer gave up waiting for its producers"
     exact, mag = _exact(proj, x, y0, slots)
-    _check(runs[0], y0, exact, mag, slots, f"shared/{name}/r{rank}/p{parts}/m{mode}")
+    _check(runs[0], y0, exact, mag, slots, f"split/{name}/r{rank}/k{kpart}/w{wide}")
     for other in runs[1:]:
         assert torch.equal(runs[0], other)
-    (plan,) = getattr(meta, _PLAN_ATTR).values()
-    words = plan.workspace.tolist()
-    cap_small = ((T + 15) // 16 + 12 + 7) & ~7
-    assert words[-8 * cap_small:] == [0] * (8 * cap_small)
+    (scratch,) = backend._scratch.values()
+    head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
+    state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} per tile
+    assert all(arrivals == 0 for _, arrivals in state)
+    assert any(generation > 0 for generation, _ in state)
+    # a workspace without the signature: same bits, nothing published, nobody waits
+    scratch[:4].zero_()
+    _knobs(monkeypatch, MLORA_SPLIT_SPIN_TICKS=20000)
+    assert torch.equal(run(), runs[0])
+    assert _waits_run_out(backend) == 0
+    assert head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist() == state
 
 
 def test_config2_matches_reference_torch_loop():
@@ -214,16 +247,16 @@ def test_ranks_and_dtypes_small(rank, dtype, form):
 @pytest.mark.parametrize("rank", [8, 16, 32, 64])
 def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
     """The small-tile kernel at the K values that select its specialisations (1024, 2048, 3072:
-    four, eight, twelve k-steps per wavefront with staged operands; 4096: K shared between
-    workgroups, or sixteen k-steps when it is not; 512 and 160: two k-steps / run-time split),
+    4096: four, eight, twelve, sixteen k-steps per wavefront with staged operands; 512 and 160: two
+    k-steps / run-time split),
     with ragged slice widths, narrow and wide column ranges,
     row-strided x and y views, rows without adapter and a segment longer than one tile."""
     from nanovllm_voxcpm_amd import synthetic
 
     print(f"small tiles r={rank} {dtype} staged={staged}", flush=True)
-    monkeypatch.setenv("MLORA_DECODE_STAGED", staged)
+    _knobs(monkeypatch, MLORA_DECODE_STAGED=staged)
     shapes = {"a": (1024, [72, 200, 8]), "b": (4096, [328]), "c": (512, [1096, 64]), "d": (160, [24]),
-              "e": (2048, [136, 64]), "f": (3072, [72]), "b0": (4096, [328])}  # 8, 12 (and, unshared, 16) k-steps per wavefront
+              "e": (2048, [136, 64]), "f": (3072, [72])}  # 8, 12 and (K = 4096) 16 k-steps per wavefront
     g = torch.Generator().manual_seed(40 + rank)
     T = 77
     slots = torch.randint(-1, 9, (T,), generator=g, dtype=torch.int32)
@@ -234,10 +267,7 @@ def test_small_tile_form_shapes(rank, dtype, staged, monkeypatch):
         xw, yw = synthetic.make_activations(T, proj.k + 16, sum(proj.widths) + 24, dtype, seed=951, device="cuda")
         x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 8 : 8 + sum(proj.widths)]
         y = yw.clone()[:, 8 : 8 + sum(proj.widths)]
-        if name == "b0":
-            monkeypatch.setenv("MLORA_DECODE_MODE", "0")  # all of K = 4096 in one workgroup
         got = _apply("mfma", proj, x, y, slots, scaling=1.25)
-        monkeypatch.delenv("MLORA_DECODE_MODE", raising=False)
         exact, mag = _exact(proj, x, y0, slots, scaling=1.25)
         _check(got, y0, exact, mag, slots, f"small/{name}/r{rank}/{dtype}/staged{staged}")
         assert torch.equal(y._base[:, :8], yw[:, :8]) and torch.equal(y._base[:, 8 + sum(proj.widths):], yw[:, 8 + sum(proj.widths):])
@@ -301,6 +331,7 @@ def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
     print(f"long form r={rank} {dtype} {knobs}", flush=True)
     for key, value in knobs.items():
         monkeypatch.setenv(key, value)
+    _knobs(monkeypatch)
     # K = 640 and 768 take 128- and 256-column x batches, 1536 and 2048 several batches per K part
     shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520]), "s": (640, [64, 72]), "t": (768, [264]), "u": (1536, [136]), "v": (2048, [64])}
     lengths = [130, 1, 64, 15, 16, 65, 3, 128, 17, 7]
@@ -685,9 +716,7 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     small_off = (offsets_off + r4(L + 2) + 31) & ~31
     cap_small = ((T + 15) // 16 + min(L, T) + 7) & ~7
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
-    coop_off = big_off + 4 * ((T // 64 + min(L, T) + 31) & ~31)
-    assert len(ws) == coop_off + 8 * cap_small
-    assert ws[coop_off:] == [0] * (8 * cap_small)  # arrival counters rest at zero
+    assert len(ws) == big_off + 4 * ((T // 64 + min(L, T) + 31) & ~31)
     assert ws[sorted_off : sorted_off + len(s)] == s
     dense = [0] * (L + 1)
     for slot, n in zip(a, c):
@@ -697,7 +726,8 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     for q, (slot, start, count) in enumerate(short + long_small):
         rec = ws[small_off + 32 * q : small_off + 32 * (q + 1)]
         assert rec[:4] == [slot, count, start, 0]
-        assert rec[4 : 4 + count] == s[start : start + count] and rec[4 + count :] == [0] * (28 - count)
+        own = s[start : start + count]
+        assert rec[4:20] == [own[j % count] for j in range(16)] and rec[20:] == [0] * 12  # cyclic repeats past the count
     assert [tuple(ws[big_off + 4 * i : big_off + 4 * i + 3]) for i in range(len(long_big))] == long_big
 
 
@@ -777,9 +807,9 @@ def test_graph_capture_replays_follow_new_slots_inputs_and_weights():
 
 @pytest.mark.parametrize("name,tokens,rank", [("down", 256, 16), ("gate_up", 1500, 64), ("down", 1500, 32)])
 def test_graph_replays_of_the_shared_and_the_two_launch_forms(name, tokens, rank):
-    """Backend call captured once (K = 4096 at decode size: workgroups exchanging partial sums
-    through the scratch and the plan's counters; 1500 tokens: the two-launch form with its scratch
-    allocated inside the capture) and replayed with new activations, base outputs and slot ids in
+    """Backend call captured once (K = 4096 at decode size: producer and consumer workgroups
+    exchanging partial sums through the scratch; 1500 tokens: the two-launch form; in both the
+    scratch is allocated and initialised inside the capture) and replayed with new activations, base outputs and slot ids in
     the same buffers; every replay is checked against the fp64 evaluation and against an eager
     call on the same inputs, with eager work and synchronisations between the replays."""
     from nanovllm_voxcpm_amd import synthetic
