@@ -177,6 +177,8 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
     case MLORA_FORM_BGMV:
+      if (a->effective_rank && a->form == MLORA_FORM_AUTO) return launch_token_add(a);  // the vector-ALU tiles read whole rank-r rows
+      if (a->effective_rank) { set_error("mlora_add_lora: the BGMV form does not take effective_rank"); return MLORA_E_UNSUPPORTED; }
       if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
       return launch_bgmv(a, /*include_long=*/true);
     case MLORA_FORM_SGMV:

@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
                                                                              float* __restrict__ hws, int64_t xs, int big_off,
                                                                              int small_off, int big_cap, int sorted_off, int T_, int K,
                                                                              int num_slots, int num_slices, int ksplit, int krange,
-                                                                             int all_slices, ShrinkSlices sl) {
+                                                                             int all_slices, const int32_t* __restrict__ eff_rank, ShrinkSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -126,6 +126,16 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
   if (!tr.ok) return;
   const int slot = tr.slot, start = tr.start, m = tr.m;
+  // rank of the adapter in this slot: 16-rank blocks of A[slot] at or above it are neither copied
+  // to LDS nor multiplied, and their partial sums are not written (the expand does not read them)
+  int eff = R;
+  if (eff_rank) {
+    eff = eff_rank[slot];
+    eff = eff < 0 ? 0 : eff > R ? R : eff;
+    if (eff == 0) return;
+  }
+  const int rb_n = (eff + 15) >> 4;
+  const int rows_used = rb_n * 16 < R ? rb_n * 16 : R;
 
   const int k0 = kpart * krange;
   const int nbatch = krange / XW;
@@ -142,14 +152,14 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = i * NT + tid;
-      if (TOTAL % NT == 0 || c < TOTAL) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
+      if ((TOTAL % NT == 0 || c < TOTAL) && c / CPR < rows_used) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
     }
   };
   auto store_slab = [&]() {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = i * NT + tid;
-      if (TOTAL % NT == 0 || c < TOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
+      if ((TOTAL % NT == 0 || c < TOTAL) && c / CPR < rows_used) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
     }
   };
   auto request_x = [&](Pack8(&buf)[XK], int kc) {
@@ -179,6 +189,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
         for (int i = 0; i < KS; ++i) {
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
+            if (RB > 1 && rb >= rb_n) continue;
             const int rr = rb * 16 + lr;
             Pack8 aw;
             aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + i * 32 + lg * 8]);
@@ -209,7 +220,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const int r0 = rb * 16 + 4 * lg;
-        if (r0 < R) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
+        if (r0 < R && rb < rb_n) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
       }
     }
   }
@@ -258,7 +269,8 @@ template <typename T, int R, int CPL, int TPF, int G>
 __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                                                              void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
                                                                              int big_units, int sorted_off, int T_, int num_slots,
-                                                                             int num_slices, int ksplit, float scaling, int nt, ExpandSplits splits) {
+                                                                             int num_slices, int ksplit, float scaling, int nt,
+                                                                             const int32_t* __restrict__ eff_rank, ExpandSplits splits) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int NB = TB / TPF;           // y batches per tile
   constexpr int STEPS = G * NB;          // (tile, batch) steps of a span
@@ -271,7 +283,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
 
   __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
   __shared__ __attribute__((aligned(16))) int s_row[G * MLORA_TILE_BIG];
-  __shared__ int s_slot[G], s_m[G];
+  __shared__ int s_slot[G], s_m[G], s_eff[G];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
@@ -300,6 +312,18 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
     start[g] = is_big ? big[g][1] : small[2];
     m[g] = is_big ? big[g][2] : small[1];
     if (!have || m[g] <= 0 || slot[g] < 0 || slot[g] >= num_slots) m[g] = 0;
+  }
+  // rank of the adapter in each tile's slot (a second, dependent fetch, only with the vector
+  // given): ranks at or above it are left out of the intermediate, of the B rows and of the MFMAs
+  int eff[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    eff[g] = R;
+    if (eff_rank && m[g] > 0) {
+      const int e = eff_rank[slot[g]];
+      eff[g] = e < 0 ? 0 : e > R ? R : e;
+      if (eff[g] == 0) m[g] = 0;  // nothing resident: the tile is skipped
+    }
     any |= m[g];
   }
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
@@ -310,7 +334,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   // never written)
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; }
+    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
     if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
   }
   __syncthreads();
@@ -341,27 +365,50 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   };
   Pack8 bop[CPL][KSTEPS];
   int b_slot = -1, b_c0 = -1;  // what bop holds
-  auto load_b = [&](int c0, int sg) {
+  int b_ks = KSTEPS;  // k-steps of the slot bop holds
+  auto load_b = [&](int c0, int sg, int eg) {
     // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
     // their H operand is zero; columns past the range repeat the last one and are never stored)
     const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
+    if (eg >= R) {
 #pragma unroll
-    for (int j = 0; j < CPL; ++j) {
-      int n = c0 + CPL * lr + j;
-      n = n < sp.n1 ? n : sp.n1 - 1;
+      for (int j = 0; j < CPL; ++j) {
+        int n = c0 + CPL * lr + j;
+        n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = (lg + 4 * ks) & (R / 8 - 1);
-        bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = (lg + 4 * ks) & (R / 8 - 1);
+          bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        }
+      }
+    } else {
+      // an adapter of lower rank: only its own chunks of eight ranks are fetched, the rest of the
+      // operand is zero, and what the boundary chunk holds beyond the rank is masked out
+      const int eg8 = (eg + 7) >> 3;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        int n = c0 + CPL * lr + j;
+        n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = lg + 4 * ks;
+          if (kc < eg8) {
+            bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+            if (eg & 7) mask_ranks(bop[j][ks], kc * 8, eg);
+          } else {
+            bop[j][ks].raw = i32x4{0, 0, 0, 0};
+          }
+        }
       }
     }
     b_slot = sg;
     b_c0 = c0;
+    b_ks = (eg + 31) >> 5;
   };
   auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
     const int g = st / NB, tp = (st % NB) * TPF;
     const int mg = s_m[g], sg = s_slot[g];
-    if (sg != b_slot || c0 != b_c0) load_b(c0, sg);
+    if (sg != b_slot || c0 != b_c0) load_b(c0, sg, s_eff[g]);
     const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
     const int c = c0 + CPL * lr;
     const bool col_ok = c < sp.n1;
@@ -387,6 +434,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
         out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
+          if (KSTEPS > 1 && ks >= b_ks) continue;
           out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
           out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
         }
@@ -409,7 +457,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   int c0 = sp.n0 + wave * SPAN, st = first_step;
   const bool has_work = c0 < sp.n1;
   if (has_work) {
-    load_b(c0, s_slot[st / NB]);
+    load_b(c0, s_slot[st / NB], s_eff[st / NB]);
     issue_y(ya, c0, st);
   }
 
@@ -429,11 +477,17 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
         int tok = c / CPR;
         tok = tok < m[g] ? tok : m[g] - 1;
         const float* q = src + tok * hrow + (c % CPR) * 8;
+        const bool used = (c % CPR) * 8 < ((eff[g] + 15) & ~15);  // the shrink wrote this chunk
 #pragma unroll
         for (int kp = 0; kp < kMaxKSplit; ++kp) {
           if (kp < ksplit) {
-            t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
-            t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+            if (used) {
+              t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
+              t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+            } else {
+              t[h][kp][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+              t[h][kp][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
           }
         }
       }
@@ -454,8 +508,8 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
         const float live = tok < m[g] ? scaling : 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          v[i] = s0[i] * live;
-          v[4 + i] = s1[i] * live;
+          v[i] = ch * 8 + i < eff[g] ? s0[i] * live : 0.f;  // ranks the adapter does not have contribute nothing
+          v[4 + i] = ch * 8 + 4 + i < eff[g] ? s1[i] * live : 0.f;
         }
         pack8<T>(v, hi);
         unpack8<T>(hi, back);
@@ -540,7 +594,7 @@ void launch_shrink_one(const ShrinkLaunch& l) {
   dim3 grid(8, static_cast<unsigned>(l.all_slices ? l.ksplit : a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
   hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR, XW, DB>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, partials_of(a), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
-                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, l.sl);
+                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, a->effective_rank, l.sl);
 }
 
 // (slab width, x batch width): 128/128 and 256/256 with two x buffers, 256/512 and 512/512 with one
@@ -571,7 +625,7 @@ void launch_expand_group(const MloraAddArgs* a, const PlanLayout& lay, int big_u
 #define MLORA_EXPAND(CPL_, TPF_, G_)                                                                                       \
   hipLaunchKernelGGL((sgmv_expand_kernel<T, R, CPL_, TPF_, G_>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, \
                      a->y_stride, lay.big_off, lay.small_off, big_units, lay.sorted_off, a->num_tokens, a->num_slots,      \
-                     a->num_slices, ksplit, a->scaling, nt, sp)
+                     a->num_slices, ksplit, a->scaling, nt, a->effective_rank, sp)
   if (cpl == 4) {
     if (group == 4) MLORA_EXPAND(4, 4, 4); else if (group == 2) MLORA_EXPAND(4, 4, 2); else MLORA_EXPAND(4, 4, 1);
   } else {

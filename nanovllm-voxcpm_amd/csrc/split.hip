@@ -519,19 +519,30 @@ int workspace_init(void* workspace, hipStream_t stream) {
   return check_launch("mlora_workspace_init");
 }
 
+// Columns of a K part: 1024 (eight wavefronts) when K is long, 512 (four) otherwise, so that a
+// producer pulls 24-48 KB and a consumer adds up at most eight parts; the other width when the
+// preferred one does not divide K or its partial sums do not fit the exchange area.  0: none fits.
+static int pick_kpart(const MloraAddArgs* a, int wanted) {
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+  const int preferred = (a->k % 1024 == 0 && a->k >= 2048) ? 1024 : 512;
+  const int order[3] = {wanted, preferred, preferred == 512 ? 1024 : 512};
+  for (int kp : order) {
+    if (kp != 512 && kp != 1024) continue;
+    if (a->k % kp != 0 || a->k / kp > 8) continue;
+    if (static_cast<int64_t>(lay.cap_small) * a->num_slices * (a->k / kp) * 16 * a->r * 8 <= kWsXchgBytes) return kp;
+  }
+  return 0;
+}
+
 // Whether the split form can take this call at all (shape, workspace, partial sums that fit the
 // exchange area).
 bool split_supported(const MloraAddArgs* a) {
   if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 255) || a->workspace_bytes < MLORA_WORKSPACE_HEAD_BYTES) return false;
   if (a->k % 512 != 0 || a->k < 512) return false;
-  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  if (lay.cap_small > kWsTiles) return false;
+  if (plan_layout(a->num_tokens, a->num_slots).cap_small > kWsTiles) return false;
   for (int i = 0; i < a->num_slices; ++i)
     if (a->slices[i].n <= 0) return false;
-  const int kp = (a->k % 1024 == 0 && a->k >= 2048) ? 1024 : 512;
-  const int64_t parts = a->k / kp;
-  if (parts > 8) return false;
-  return static_cast<int64_t>(lay.cap_small) * a->num_slices * parts * 16 * a->r * 8 <= kWsXchgBytes;
+  return pick_kpart(a, 0) != 0;
 }
 
 int launch_split(const MloraAddArgs* a, bool include_long, bool trusted_workspace) {
@@ -550,12 +561,7 @@ int launch_split(const MloraAddArgs* a, bool include_long, bool trusted_workspac
   l.a = a; l.small_off = lay.small_off; l.include_long = include_long ? 1 : 0;
   l.S = a->num_slices;
   l.spin_ticks = knobs.spin_ticks; l.wide = knobs.wide; l.trusted = trusted_workspace ? 1 : 0;
-  // K parts: 1024 columns (eight wavefronts) when K is long, 512 (four) otherwise, so that a
-  // producer pulls 24-48 KB and a consumer adds up at most eight parts
-  int kp = (a->k % 1024 == 0 && a->k >= 2048) ? 1024 : 512;
-  if ((knobs.kpart == 512 || knobs.kpart == 1024) && a->k % knobs.kpart == 0 && a->k / knobs.kpart <= 8 &&
-      static_cast<int64_t>(lay.cap_small) * a->num_slices * (a->k / knobs.kpart) * 16 * a->r * 8 <= kWsXchgBytes)
-    kp = knobs.kpart;
+  const int kp = pick_kpart(a, knobs.kpart);  // split_supported() was true: some width fits
   l.P = a->k / kp;
   const int nwp = kp / 128;
 

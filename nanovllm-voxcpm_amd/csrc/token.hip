@@ -20,6 +20,7 @@ struct TokenAddParams {
   const int32_t* tts;
   int T, K, r, num_slots, nsplit;
   float scaling;
+  const int32_t* eff_rank;  // per slot, or null
   MloraSlice slices[MLORA_MAX_SLICES];
 };
 
@@ -38,7 +39,14 @@ __global__ __launch_bounds__(kTokThreads) void token_add_kernel(TokenAddParams p
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const T* x = static_cast<const T*>(p.x) + static_cast<int64_t>(t) * p.xs;
   const T* A = static_cast<const T*>(sl.a) + static_cast<int64_t>(s) * p.r * p.K;
-  for (int j = wave; j < p.r; j += kTokWaves) {
+  // rows of A and columns of B at or above the rank of the adapter in this slot are not read
+  int eff = p.r;
+  if (p.eff_rank) {
+    eff = p.eff_rank[s];
+    eff = eff < 0 ? 0 : eff > p.r ? p.r : eff;
+    if (eff == 0) return;
+  }
+  for (int j = wave; j < eff; j += kTokWaves) {
     const T* a = A + static_cast<int64_t>(j) * p.K;
     float acc = 0.f;
     for (int k = lane; k < p.K; k += kWave) acc += to_f32(x[k]) * to_f32(a[k]);
@@ -51,7 +59,7 @@ __global__ __launch_bounds__(kTokThreads) void token_add_kernel(TokenAddParams p
   for (int n = n0 + tid; n < n1; n += kTokThreads) {
     const T* b = B + static_cast<int64_t>(n) * p.r;
     float acc = 0.f;
-    for (int j = 0; j < p.r; ++j) acc += h[j] * to_f32(b[j]);
+    for (int j = 0; j < eff; ++j) acc += h[j] * to_f32(b[j]);
     y[n] = from_f32<T>(to_f32(y[n]) + acc);
   }
 }
@@ -167,6 +175,7 @@ int launch_token_add(const MloraAddArgs* a) {
   TokenAddParams p;
   p.x = a->x; p.y = a->y; p.xs = a->x_stride; p.ys = a->y_stride; p.tts = a->token_to_slot;
   p.T = a->num_tokens; p.K = a->k; p.r = a->r; p.num_slots = a->num_slots; p.scaling = a->scaling;
+  p.eff_rank = a->effective_rank;
   int n_max = 0;
   for (int i = 0; i < a->num_slices; ++i) { p.slices[i] = a->slices[i]; n_max = a->slices[i].n > n_max ? a->slices[i].n : n_max; }
   p.nsplit = column_splits(n_max);

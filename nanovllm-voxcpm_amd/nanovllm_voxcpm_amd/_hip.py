@@ -330,9 +330,21 @@ def add_lora(
     ``effective_rank``: int32 [slots] on the device, rank of the adapter resident in each slot of
     these buffers; rows / columns at or above it are then neither read nor multiplied."""
     lib = load()
-    _require_cuda(x, "x")
     if len(a_slices) > MAX_SLICES:
         raise ValueError(f"at most {MAX_SLICES} slices per call, got {len(a_slices)}")
+    for name, t in (("y", y), ("token_to_slot", token_to_slot), *((f"lora_a[{i}]", a) for i, a in enumerate(a_slices)),
+                    *((f"lora_b[{i}]", b) for i, b in enumerate(b_slices))):
+        if t.device != x.device:
+            raise ValueError(f"{name} lives on {t.device}, x on {x.device}")
+        if name != "token_to_slot" and t.dtype != x.dtype:
+            raise ValueError(f"{name} has element type {t.dtype}, x has {x.dtype}")
+    if token_to_slot.dtype != torch.int32 or not token_to_slot.is_contiguous():
+        raise ValueError("token_to_slot must be a contiguous int32 tensor")
+    if token_to_slot.numel() < x.size(0):
+        raise ValueError(f"token_to_slot has {token_to_slot.numel()} entries for {x.size(0)} rows of x")
+    if y.size(0) < x.size(0):
+        raise ValueError(f"y has {y.size(0)} rows for {x.size(0)} rows of x")
+    _require_cuda(x, "x")
     args = MloraAddArgs()
     args.stream = _stream(x.device) if stream is None else stream
     args.x = x.data_ptr()
@@ -375,6 +387,15 @@ def shrink(
     x: torch.Tensor, a_slices: list[torch.Tensor], out: torch.Tensor, token_to_slot: torch.Tensor, scaling: float
 ) -> None:
     lib = load()
+    if token_to_slot.dtype != torch.int32 or not token_to_slot.is_contiguous() or token_to_slot.numel() < x.size(0):
+        raise ValueError(f"token_to_slot must be a contiguous int32 tensor with an entry for each of the {x.size(0)} rows of x")
+    for name, t in (("out", out), ("token_to_slot", token_to_slot), *((f"lora_a[{i}]", a) for i, a in enumerate(a_slices))):
+        if t.device != x.device:
+            raise ValueError(f"{name} lives on {t.device}, x on {x.device}")
+    if any(a.dtype != x.dtype for a in a_slices):
+        raise ValueError("lora_a slices must have the element type of x")
+    if out.size(-2) < x.size(0):
+        raise ValueError(f"out has {out.size(-2)} rows for {x.size(0)} rows of x")
     _require_cuda(x, "x")
     args = MloraShrinkArgs()
     args.stream = _stream(x.device)
@@ -405,6 +426,16 @@ def expand(
     add_inputs: bool,
 ) -> None:
     lib = load()
+    rows = h.size(1)
+    if token_to_slot.dtype != torch.int32 or not token_to_slot.is_contiguous() or token_to_slot.numel() < rows:
+        raise ValueError(f"token_to_slot must be a contiguous int32 tensor with an entry for each of the {rows} rows")
+    for name, t in (("y", y), ("token_to_slot", token_to_slot), *((f"lora_b[{i}]", b) for i, b in enumerate(b_slices))):
+        if t.device != h.device:
+            raise ValueError(f"{name} lives on {t.device}, the inputs on {h.device}")
+    if any(b.dtype != y.dtype for b in b_slices):
+        raise ValueError("lora_b slices must have the element type of y")
+    if y.size(0) < rows:
+        raise ValueError(f"y has {y.size(0)} rows for {rows} rows of the inputs")
     _require_cuda(h, "inputs")
     args = MloraExpandArgs()
     args.stream = _stream(h.device)
@@ -484,6 +515,20 @@ def install_slot(
 ) -> None:
     """Rewrite one slot of A [slots, r, K] and B [slots, n, r] from an adapter payload."""
     lib = load()
+    if not 0 <= slot < a_dst.size(0) or b_dst.size(0) != a_dst.size(0):
+        raise IndexError(f"slot {slot} is outside the {a_dst.size(0)} slots of the LoRA buffers")
+    if a_src.ndim != 2 or b_src.ndim != 2:
+        raise ValueError(f"adapter payload must be 2D, got lora_a {tuple(a_src.shape)} and lora_b {tuple(b_src.shape)}")
+    if a_src.size(1) != a_dst.size(2):
+        raise ValueError(f"Expected lora_a input dim {a_dst.size(2)}, got {a_src.size(1)}")
+    if b_src.size(0) != b_dst.size(1):
+        raise ValueError(f"Expected lora_b output dim {b_dst.size(1)}, got {b_src.size(0)}")
+    if not 0 <= rank <= a_dst.size(1) or rank > a_src.size(0) or rank > b_src.size(1):
+        raise ValueError(f"rank {rank} does not fit the payload {tuple(a_src.shape)} / {tuple(b_src.shape)} and the buffers' rank {a_dst.size(1)}")
+    if a_src.stride(1) != 1 or b_src.stride(1) != 1:
+        raise ValueError("adapter payload rows must be contiguous")
+    if a_src.device != a_dst.device or b_src.device != a_dst.device or b_dst.device != a_dst.device:
+        raise ValueError("adapter payload and LoRA buffers must live on one device")
     _require_cuda(a_dst, "lora_A")
     args = MloraInstallArgs()
     args.stream = _stream(a_dst.device)

@@ -22,7 +22,7 @@ import torch
 
 from nanovllm_voxcpm_amd import _hip
 from nanovllm_voxcpm_amd.lora_ops.segment_meta import as_slot_vector
-from nanovllm_voxcpm_amd.utils.context import LORA_DOMAINS, LoRAContext, set_lora_context
+from nanovllm_voxcpm_amd.utils.context import LORA_DOMAINS, LoRAContext, get_lora_context, invalidate_lora_context, set_lora_context
 
 
 def make_graph_domain_buffers(
@@ -58,6 +58,13 @@ def copy_lora_domain_to_graph_vars(domain_vars: dict[str, torch.Tensor], context
         dense_offsets=domain_vars["slot_start_offsets"],
         padded_token_to_slot=tts_buf,
     )
+    # Installed contexts that view these buffers were just rewritten in place (by a kernel, which
+    # no tensor version counter sees): what they derived from the old contents is dropped.
+    for domain in LORA_DOMAINS:
+        installed = get_lora_context(domain)
+        view = installed.token_to_slot
+        if view is not None and view.is_cuda and view.numel() and view.data_ptr() == tts_buf.data_ptr():
+            invalidate_lora_context(installed)
 
 
 def set_graph_lora_contexts(graph_vars: dict, contexts: dict[str, LoRAContext]) -> None:

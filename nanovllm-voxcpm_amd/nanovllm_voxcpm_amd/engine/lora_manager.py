@@ -10,20 +10,44 @@ re-exported here under the reference's import path.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-
 import torch
 
 from nanovllm_voxcpm_amd import _hip
 from nanovllm_voxcpm_amd.utils.context import LoRAContext
 
 
-@dataclass
 class LoRABatchPlan:
-    """What the scheduler knows on the host: which slot every token of the batch uses."""
+    """What the scheduler knows on the host: which slot every token of the batch uses.
 
-    adapter_to_slot: dict[int, int]
-    token_to_slot: list[int]
+    Takes the six fields of the reference's dataclass (lora_manager.py:67-75) in its order; the
+    four segment arrays may be left out and are then derived from ``token_to_slot`` on demand
+    (the device path never reads them: the GPU sorts the tokens itself)."""
+
+    __slots__ = ("adapter_to_slot", "token_to_slot", "_sorted", "_active", "_counts", "_offsets")
+
+    def __init__(
+        self,
+        adapter_to_slot: dict[int, int],
+        token_to_slot: list[int],
+        token_indices_sorted_by_slot: list[int] | None = None,
+        active_slot_ids: list[int] | None = None,
+        num_tokens_per_slot: list[int] | None = None,
+        slot_start_offsets: list[int] | None = None,
+    ) -> None:
+        self.adapter_to_slot = adapter_to_slot
+        self.token_to_slot = token_to_slot
+        self._sorted = token_indices_sorted_by_slot
+        self._active = active_slot_ids
+        self._counts = num_tokens_per_slot
+        self._offsets = slot_start_offsets
+
+    def __repr__(self) -> str:
+        return f"LoRABatchPlan(adapter_to_slot={self.adapter_to_slot!r}, token_to_slot={self.token_to_slot!r})"
+
+    def __eq__(self, other) -> bool:
+        if not isinstance(other, LoRABatchPlan):
+            return NotImplemented
+        return self.adapter_to_slot == other.adapter_to_slot and list(self.token_to_slot) == list(other.token_to_slot)
 
     @property
     def num_lora_tokens(self) -> int:
@@ -31,25 +55,31 @@ class LoRABatchPlan:
 
     @property
     def active_slot_ids(self) -> list[int]:
-        return sorted({s for s in self.token_to_slot if s >= 0})
+        if self._active is None:
+            self._active = sorted({s for s in self.token_to_slot if s >= 0})
+        return self._active
 
-    # The remaining host-side views of the reference's plan (lora_manager.py:67-91) are derived
-    # on demand; the device path never reads them (the GPU sorts the tokens itself).
     @property
     def num_tokens_per_slot(self) -> list[int]:
-        return [sum(1 for s in self.token_to_slot if s == slot) for slot in self.active_slot_ids]
+        if self._counts is None:
+            self._counts = [sum(1 for s in self.token_to_slot if s == slot) for slot in self.active_slot_ids]
+        return self._counts
 
     @property
     def slot_start_offsets(self) -> list[int]:
-        offsets = [0]
-        for count in self.num_tokens_per_slot:
-            offsets.append(offsets[-1] + count)
-        return offsets
+        if self._offsets is None:
+            offsets = [0]
+            for count in self.num_tokens_per_slot:
+                offsets.append(offsets[-1] + count)
+            self._offsets = offsets
+        return self._offsets
 
     @property
     def token_indices_sorted_by_slot(self) -> list[int]:
-        keyed = [(s, t) for t, s in enumerate(self.token_to_slot) if s >= 0]
-        return [t for _, t in sorted(keyed)]
+        if self._sorted is None:
+            keyed = [(s, t) for t, s in enumerate(self.token_to_slot) if s >= 0]
+            self._sorted = [t for _, t in sorted(keyed)]
+        return self._sorted
 
 
 def build_lora_batch_plan_from_token_to_slot(

@@ -143,6 +143,8 @@ class _LoRALayerBase(nn.Module):
                 no_lora_flag=context.no_lora_flag,
                 num_active_loras=context.num_active_loras,
             )
+            # the context's own table of segment plans travels with the view (frozen dataclass)
+            object.__setattr__(meta, "_mlora_context_plans", context._segment_plans)
             context._cached_metadata = meta
         return meta  # type: ignore[return-value]
 
@@ -162,6 +164,8 @@ class _LoRALayerBase(nn.Module):
         b_slices = [self._b_of(p) for p in range(len(block_of_target))]
         call = dict(indices=token_to_slot, metadata=self._runtime_metadata(), scaling=1.0)
         backend = get_backend()
+        if self._wants_rank_masking() and getattr(backend, "takes_effective_rank", False):
+            call["effective_rank"] = self.effective_lora_rank
         if len(block_sizes) == 1:
             out_flat = backend.add_lora([out_flat], x_flat, a_slices, b_slices, **call)[0]
         else:
@@ -177,6 +181,17 @@ class _LoRALayerBase(nn.Module):
         if x.ndim == 2:
             return out_flat
         return out_flat.reshape(*x.shape[:-1], out_flat.size(-1))
+
+    def _wants_rank_masking(self) -> bool:
+        """Whether the backend should be told the per-slot ranks: only buffers of more than one
+        16-rank block can skip anything, and only when some resident adapter is below the padded
+        rank — or while a graph is captured, whose launches must serve adapters installed later.
+        Decided from the host mirror only."""
+        if self.max_lora_rank <= 16:
+            return False
+        if _is_cuda_graph_capture():
+            return True
+        return any(0 < rank < self.max_lora_rank for rank in self._effective_lora_rank_values)
 
     def prime_lora_cache(self) -> None:
         if not self.supports_lora:
@@ -238,6 +253,8 @@ class _LoRALayerBase(nn.Module):
         """Make slot ``slot_id`` hold this adapter.  Multi-target layers take ``lora_a`` as
         [targets, >=rank, in] and ``lora_b`` as a list ordered like ``lora_targets``."""
         self._validate_effective_rank(effective_rank)
+        if not 0 <= slot_id < self.max_loras:
+            raise IndexError(f"slot_id={slot_id} is outside the {self.max_loras} slots of this layer")
         if self._target_keys():
             given = min(len(lora_a), len(lora_b))
             for position in range(self._num_targets()):
@@ -257,6 +274,8 @@ class _LoRALayerBase(nn.Module):
     def clear_slot_lora(self, slot_id: int) -> None:
         if not self.supports_lora:
             return
+        if not 0 <= slot_id < self.max_loras:
+            raise IndexError(f"slot_id={slot_id} is outside the {self.max_loras} slots of this layer")
         for position in range(self._num_targets()):
             self._zero_slot(slot_id, position)
         self._record_slot(slot_id, 0, 0.0)

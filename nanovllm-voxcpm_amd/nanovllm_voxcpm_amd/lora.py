@@ -94,10 +94,13 @@ class _UnavailableBackend:
 
 _VECTOR_RANKS = (8, 16, 32, 64)
 _PLAN_ATTR = "_mlora_segment_plans"
+_CONTEXT_PLANS_ATTR = "_mlora_context_plans"  # plan table of the LoRAContext a metadata object was made from
 
 
 class HipLoRABackend:
     """``LoRABackend`` whose arithmetic runs in the hand-written gfx950 kernels."""
+
+    takes_effective_rank = True  # add_lora accepts the per-slot rank vector of the calling layer
 
     def __init__(self, form: str | None = None) -> None:
         name = form if form is not None else os.environ.get("MLORA_FORM", "auto")
@@ -131,30 +134,44 @@ class HipLoRABackend:
     @staticmethod
     def _plan_for(metadata: LoRAMetadata, tts: torch.Tensor, max_slots: int, capture: int | None = None) -> SegmentPlan:
         """One metadata launch per batch: every LoRA layer of a step shares the metadata
-        object, so the plan is cached on it.
+        object, so the plan is kept on it.
 
-        A cached plan is reused only for the same slot vector (address, length, in-place
-        version) and inside the same stream capture it was built in: a plan built eagerly
-        during warm-up must not satisfy a later graph capture, or the captured graph would
-        contain no metadata launch and replay stale segments.
+        Two holders, neither of which can go stale silently:
+
+        * a metadata object made from a ``LoRAContext`` carries the context's own plan table
+          (``_mlora_context_plans``).  The plan is then a derived array of the context, like the
+          sorted indices and counts the reference keeps there: it lives until the context is
+          installed again, and whoever refreshes the context's buffers in place
+          (``graph_meta.copy_lora_domain_to_graph_vars``) drops it;
+        * any other metadata object gets a table keyed by the slot vector's address, length and
+          in-place version.  Inference tensors have no version counter, so an in-place rewrite
+          could not be noticed: for them nothing is kept and every call builds its plan.
+
+        Either way a plan is reused only inside the stream capture it was built in: a plan built
+        eagerly during warm-up must not satisfy a later graph capture, or the captured graph
+        would contain no metadata launch and replay stale segments.
         """
         own = metadata.token_to_slot
         if own is None or own.data_ptr() != tts.data_ptr():
             return build_segment_plan(tts, max_slots)  # converted / foreign vector: do not cache
-        try:
-            version = own._version
-        except RuntimeError:  # inference tensors carry no version counter
-            version = None
         if capture is None:
             capture = _hip.stream_capture_id(tts.device)
-        key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, capture)
-        cache = getattr(metadata, _PLAN_ATTR, None)
-        if cache is None:
-            cache = {}
+        cache = getattr(metadata, _CONTEXT_PLANS_ATTR, None)
+        if cache is not None:
+            key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, capture)
+        else:
             try:
-                object.__setattr__(metadata, _PLAN_ATTR, cache)
-            except (AttributeError, TypeError):
-                return build_segment_plan(tts, max_slots)  # slotted metadata type
+                version = own._version
+            except RuntimeError:  # inference tensors carry no version counter
+                return build_segment_plan(tts, max_slots)
+            key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, capture)
+            cache = getattr(metadata, _PLAN_ATTR, None)
+            if cache is None:
+                cache = {}
+                try:
+                    object.__setattr__(metadata, _PLAN_ATTR, cache)
+                except (AttributeError, TypeError):
+                    return build_segment_plan(tts, max_slots)  # slotted metadata type
         plan = cache.get(key)
         if plan is None:
             if len(cache) >= 4:
@@ -210,9 +227,15 @@ class HipLoRABackend:
         metadata: LoRAMetadata | None,
         scaling: float,
         y_packed: torch.Tensor | None = None,
+        effective_rank: torch.Tensor | None = None,
     ) -> list[torch.Tensor]:
         """y_i[t] += scaling * (x[t] . A_i[slot_t]^T) . B_i[slot_t]^T for every slice i and every
         token with a slot; rows with slot -1 keep their bits.
+
+        ``effective_rank`` (beyond the reference's protocol, optional): int32 [slots] on the
+        device, the rank of the adapter resident in each slot of these buffers
+        (``layer.effective_lora_rank``).  Rows of A and columns of B at or above it are then
+        neither read nor multiplied.
 
         With ``y_packed`` the slices must be its column blocks in order (``split`` views) and
         are updated in place; a single slice is updated in place; several slices without
@@ -254,9 +277,13 @@ class HipLoRABackend:
             return outputs
 
         source = metadata.token_to_slot if metadata.token_to_slot is not None else indices
+        if source.numel() < x.size(0):
+            raise ValueError(f"LoRA slot vector has {source.numel()} entries for {x.size(0)} rows of x")
         tts = as_slot_vector(source[: x.size(0)])
         if not tts.is_cuda:
             raise RuntimeError("LoRA slot ids must live on the GPU; the HIP LoRA path has no host fallback")
+        if target.size(0) < x.size(0):
+            raise ValueError(f"y has {target.size(0)} rows for {x.size(0)} rows of x")
 
         x2 = x if x.stride(-1) == 1 else x.contiguous()
         staged = None
@@ -284,7 +311,8 @@ class HipLoRABackend:
                         capture = _hip.stream_capture_id(x2.device, stream)
                     plan = self._plan_for(metadata, tts, a_list[0].size(0), capture).workspace
                     scratch = self._scratch_for(x2, len(chunk), a_list[0].size(-2), stream, capture)
-                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch, stream)
+                _hip.add_lora(target, x2, a_list, b_list, c_list, tts, plan, float(scaling), form, scratch, stream,
+                              effective_rank=effective_rank)
         if staged is not None:
             staged.copy_(target)
         return outputs

@@ -214,6 +214,12 @@ def install_lora_payload(model: torch.nn.Module, slot_id: int, payload: LoRAMode
             raise ValueError(f"Unknown LoRA target module '{name}'")
         if name not in modules:
             raise ValueError(f"Module '{name}' does not support LoRA slots")
+    # every module's payload is checked against the module before anything is written: a payload
+    # for another hidden size, rank budget or TP shard must not leave a half-installed slot
+    for name, m in payload.modules.items():
+        modules[name].validate_slot_lora_payload(m.lora_a, m.lora_b, m.effective_rank, m.scaling)
+        if not 0 <= slot_id < modules[name].max_loras:
+            raise IndexError(f"slot_id={slot_id} is outside the {modules[name].max_loras} slots of '{name}'")
     previous = loaded.get(slot_id) if loaded is not None and slot_id in loaded else list(modules)
     for name in previous:
         if name not in payload.modules and name in modules:

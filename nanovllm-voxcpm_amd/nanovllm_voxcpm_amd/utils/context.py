@@ -33,6 +33,10 @@ class LoRAContext:
     # LoRAMetadata view shared by every LoRA layer of the step (and, through it, the
     # segment plan the kernels walk); dropped whenever the context is (re)installed.
     _cached_metadata: object | None = field(default=None, repr=False, compare=False)
+    # segment plans the HIP backend derived from token_to_slot (a derived array of the context,
+    # like the sorted indices above): valid until the context is installed again or its buffers
+    # are refreshed in place, both of which empty the table
+    _segment_plans: dict = field(default_factory=dict, repr=False, compare=False)
 
 
 _DOMAINS: dict[str, LoRAContext] = {}
@@ -44,8 +48,14 @@ def get_lora_context(domain: str = LM_LORA_DOMAIN) -> LoRAContext:
 
 
 def set_lora_context(lora_context: LoRAContext, *, domain: str = LM_LORA_DOMAIN) -> None:
-    lora_context._cached_metadata = None
+    invalidate_lora_context(lora_context)
     _DOMAINS[domain] = lora_context
+
+
+def invalidate_lora_context(lora_context: LoRAContext) -> None:
+    """Forget everything derived from the context's tensors (call after rewriting them in place)."""
+    lora_context._cached_metadata = None
+    lora_context._segment_plans.clear()
 
 
 def reset_lora_context(domain: str | None = None) -> None:

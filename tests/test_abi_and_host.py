@@ -334,3 +334,85 @@ def test_repo_has_no_product_import_of_the_oracle():
         text = path.read_text()
         assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), path
     assert "oracle" not in sys.modules or True
+
+
+def test_batch_plan_takes_the_six_reference_fields():
+    """reference nanovllm_voxcpm/engine/lora_manager.py:67-75, 380: positional construction"""
+    from nanovllm_voxcpm_amd.engine.lora_manager import LoRABatchPlan, build_lora_batch_plan_from_token_to_slot
+
+    empty = LoRABatchPlan({}, [-1, -1], [], [], [], [0])
+    assert (empty.token_indices_sorted_by_slot, empty.active_slot_ids, empty.num_tokens_per_slot, empty.slot_start_offsets) == ([], [], [], [0])
+    derived = build_lora_batch_plan_from_token_to_slot({7: 0}, [0, 0, -1, 0])
+    assert derived == LoRABatchPlan({7: 0}, [0, 0, -1, 0], [0, 1, 3], [0], [3], [0, 3])
+    assert (derived.token_indices_sorted_by_slot, derived.active_slot_ids, derived.num_tokens_per_slot, derived.slot_start_offsets) == ([0, 1, 3], [0], [3], [0, 3])
+
+
+def test_boundary_rejects_mismatched_tensors_before_any_launch():
+    """The ctypes boundary hands raw pointers to the kernels, so what torch's own indexing and
+    copy_ would have caught is checked here: element types, devices, lengths, slot range and
+    payload shapes (all on host tensors: nothing is launched)."""
+    from nanovllm_voxcpm_amd import _hip
+
+    x = torch.zeros(4, 8, dtype=torch.bfloat16)
+    y = torch.zeros(4, 16, dtype=torch.bfloat16)
+    a, b = torch.zeros(2, 8, 8, dtype=torch.bfloat16), torch.zeros(2, 16, 8, dtype=torch.bfloat16)
+    slots = torch.zeros(4, dtype=torch.int32)
+    with pytest.raises(ValueError, match="element type"):
+        _hip.add_lora(y.float(), x, [a], [b], [0], slots, None, 1.0)
+    with pytest.raises(ValueError, match="element type"):
+        _hip.add_lora(y, x, [a.half()], [b], [0], slots, None, 1.0)
+    with pytest.raises(ValueError, match="3 entries for 4 rows"):
+        _hip.add_lora(y, x, [a], [b], [0], slots[:3], None, 1.0)
+    with pytest.raises(ValueError, match="int32"):
+        _hip.add_lora(y, x, [a], [b], [0], slots.long(), None, 1.0)
+    with pytest.raises(ValueError, match="y has 2 rows"):
+        _hip.add_lora(y[:2], x, [a], [b], [0], slots, None, 1.0)
+    with pytest.raises(RuntimeError, match="no host fallback"):  # everything consistent: only the GPU is missing
+        _hip.add_lora(y, x, [a], [b], [0], slots, None, 1.0)
+    out = torch.zeros(1, 4, 8, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="token_to_slot"):
+        _hip.shrink(x, [a], out, slots[:2], 1.0)
+    with pytest.raises(ValueError, match="token_to_slot"):
+        _hip.expand(out, [b], y, slots[:1], 0, True)
+    with pytest.raises(ValueError, match="element type of y"):
+        _hip.expand(out, [b.float()], y, slots, 0, True)
+    # slot install
+    a_src, b_src = torch.zeros(8, 8), torch.zeros(16, 8)
+    with pytest.raises(IndexError, match="outside the 2 slots"):
+        _hip.install_slot(a, b, 2, a_src, b_src, 8, 1.0)
+    with pytest.raises(ValueError, match="input dim 8"):
+        _hip.install_slot(a, b, 0, torch.zeros(8, 4), b_src, 8, 1.0)
+    with pytest.raises(ValueError, match="output dim 16"):
+        _hip.install_slot(a, b, 0, a_src, torch.zeros(12, 8), 8, 1.0)
+    with pytest.raises(ValueError, match="rank 9"):
+        _hip.install_slot(a, b, 0, a_src, b_src, 9, 1.0)
+    with pytest.raises(ValueError, match="rank 6"):
+        _hip.install_slot(a, b, 0, a_src[:4], b_src, 6, 1.0)
+
+
+def test_layers_refuse_a_slot_outside_their_buffers_before_writing():
+    from nanovllm_voxcpm_amd.layers.lora import LoRALinear
+
+    layer = LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=4)
+    before = layer.lora_A.detach().clone()
+    with pytest.raises(IndexError, match="outside the 2 slots"):
+        layer.set_slot_lora(2, torch.ones(4, 8), torch.ones(4, 4), effective_rank=4, scaling=1.0)
+    with pytest.raises(IndexError, match="outside the 2 slots"):
+        layer.clear_slot_lora(-1)
+    assert torch.equal(layer.lora_A.detach(), before) and layer._effective_lora_rank_values == [0, 0]
+
+
+def test_rank_masking_is_requested_only_when_it_can_pay():
+    """The layer hands its per-slot rank vector to the backend only for buffers of more than one
+    16-rank block that hold an adapter below the padded rank."""
+    from nanovllm_voxcpm_amd.layers.lora import LoRALinear
+
+    narrow = LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=16)
+    narrow.set_slot_lora(0, torch.ones(8, 8), torch.ones(4, 8), effective_rank=8, scaling=1.0)
+    assert narrow._wants_rank_masking() is False
+    wide = LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=64)
+    assert wide._wants_rank_masking() is False  # nothing resident
+    wide.set_slot_lora(0, torch.ones(64, 8), torch.ones(4, 64), effective_rank=64, scaling=1.0)
+    assert wide._wants_rank_masking() is False  # only full-rank adapters
+    wide.set_slot_lora(1, torch.ones(8, 8), torch.ones(4, 8), effective_rank=8, scaling=1.0)
+    assert wide._wants_rank_masking() is True

@@ -165,6 +165,34 @@ def test_shrink_expand_oracle_match_reference_test_formulas():
         assert torch.equal(got[:, :2], out0[:, :2])
 
 
+EXPAND_ORDER_CASES = [
+    # (inputs h [1, 1, r], B [1, 1, r], y before, add_inputs, expected y) — all bf16 except h where noted.
+    # Product 2^-8 - 2^-18 is rounded to B's type first (-> 2^-8), then added to y = 1 + 2^-7 in
+    # that type: an exact tie that goes to the even neighbour 1 + 2^-6.  Adding in fp32 and
+    # rounding once would stay at 1 + 2^-7.
+    dict(h=[1.0, -(2.0 ** -9)], h_dtype=torch.bfloat16, b=[2.0 ** -8, 2.0 ** -9], y=1.0 + 2.0 ** -7, add=True, want=1.0 + 2.0 ** -6),
+    dict(h=[1.0, -(2.0 ** -9)], h_dtype=torch.bfloat16, b=[2.0 ** -8, 2.0 ** -9], y=1.0 + 2.0 ** -7, add=False, want=2.0 ** -8),
+    # fp32 intermediate with bf16 weights: the intermediate is cast to the weights' type before the
+    # product (1 + 2^-8 + 2^-9 -> 1 + 2^-7), so the difference is 2^-7, not 1.5 * 2^-8.
+    dict(h=[1.0 + 2.0 ** -8 + 2.0 ** -9, -1.0], h_dtype=torch.float32, b=[1.0, 1.0], y=0.0, add=False, want=2.0 ** -7),
+    dict(h=[1.0 + 2.0 ** -8 + 2.0 ** -9, -1.0], h_dtype=torch.float32, b=[1.0, 1.0], y=4.0, add=True, want=4.0),  # 4 + 2^-7 rounds back to 4
+]
+
+
+@pytest.mark.parametrize("case", EXPAND_ORDER_CASES, ids=lambda c: f"{c['h_dtype']}-add{c['add']}")
+def test_lora_expand_rounds_in_the_reference_order(case):
+    """Hand-picked 16-bit values on which the reference's order of roundings
+    (nanovllm_voxcpm/lora_ops/triton_ops/kernel_utils.py:219-228: cast the intermediate to the
+    weights' type, accumulate in fp32, round the product to the weights' type, add to y in that
+    type) gives a different bf16 result than any other order."""
+    h = torch.tensor(case["h"], dtype=case["h_dtype"]).view(1, 1, -1)
+    b = torch.tensor(case["b"], dtype=torch.bfloat16).view(1, 1, -1)
+    y = torch.tensor([[case["y"]]], dtype=torch.bfloat16)
+    assert h.double().flatten().tolist() == case["h"] and b.double().flatten().tolist() == case["b"]  # exactly representable
+    got = oracle.lora_expand(h, [b], y, torch.zeros(1, dtype=torch.int32), add_inputs=case["add"])
+    assert got.dtype == torch.bfloat16 and got.item() == case["want"]
+
+
 # ---- segment metadata -----------------------------------------------------------------------
 
 
