@@ -56,15 +56,20 @@ WORKLOADS = {
 }
 
 
-def algorithmic_bytes(k: int, widths: list[int], t_lora: int, used_slots: int, rank: int, num_tokens: int) -> int:
+def algorithmic_bytes(k: int, widths: list[int], t_lora: int, used_slots: int, rank: int, num_tokens: int,
+                      rank_sum: int | None = None) -> int:
     """bf16 bytes one fused call has to move: x rows, the A and B slices of the slots in use,
-    y read and written once, plus the int32 slot ids; the rank-r intermediate counts as zero."""
+    y read and written once, plus the int32 slot ids; the rank-r intermediate counts as zero.
+    ``rank_sum``: sum of the true ranks of the slots in use when adapters of lower rank sit in
+    rank-``rank`` buffers and the kernels are told so (rows beyond a slot's rank are not moved)."""
     s, n = len(widths), sum(widths)
-    return 2 * (t_lora * k + used_slots * s * rank * k + used_slots * rank * n + 2 * t_lora * n) + 4 * num_tokens
+    ranks = used_slots * rank if rank_sum is None else rank_sum
+    return 2 * (t_lora * k + ranks * s * k + ranks * n + 2 * t_lora * n) + 4 * num_tokens
 
 
-def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int) -> int:
-    return 2 * t_lora * rank * (len(widths) * k + sum(widths))
+def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int, token_rank_sum: int | None = None) -> int:
+    """``token_rank_sum``: sum over the tokens of their slot's true rank, when it is below ``rank``."""
+    return 2 * (t_lora * rank if token_rank_sum is None else token_rank_sum) * (len(widths) * k + sum(widths))
 
 
 def build_workload(name: str, device: str, rank: int | None = None):
@@ -98,11 +103,13 @@ def build_workload(name: str, device: str, rank: int | None = None):
             entry[proj_name] = (proj, x, y)
         distinct.append(entry)
     layers = [distinct[i % len(distinct)] for i in range(NUM_LAYERS)]
-    return layers, slots.to(device)
+    eff = torch.tensor(ranks, dtype=torch.int32, device=device) if ranks is not None else None
+    return layers, slots.to(device), eff
 
 
-def make_step(layers, slots, form: str, only: str | None = None):
-    """Returns step(): metadata build + every fused apply of one step, via the backend."""
+def make_step(layers, slots, form: str, only: str | None = None, eff=None):
+    """Returns step(): metadata build + every fused apply of one step, via the backend.  ``eff``:
+    per-slot true ranks, handed to the backend as the LoRA linears do for padded buffers."""
     from nanovllm_voxcpm_amd.lora import HipLoRABackend, LoRAMetadata
 
     backend = HipLoRABackend(form)
@@ -122,7 +129,7 @@ def make_step(layers, slots, form: str, only: str | None = None):
         # the first call builds the segment plan on the device, the others reuse it
         meta = LoRAMetadata(slots, None, None, None, None, False, 0)
         for blocks, x, a, b, packed in calls:
-            backend.add_lora(blocks, x, a, b, indices=slots, metadata=meta, scaling=1.0, y_packed=packed)
+            backend.add_lora(blocks, x, a, b, indices=slots, metadata=meta, scaling=1.0, y_packed=packed, effective_rank=eff)
 
     step.backend = backend
     return step, len(calls)
@@ -250,7 +257,7 @@ def run_timeline(args) -> None:
     from nanovllm_voxcpm_amd import _hip
 
     device = "cuda:0"
-    layers, slots = build_workload("decode", device, args.rank or None)
+    layers, slots, _ = build_workload("decode", device, args.rank or None)
     step, launches = make_step(layers, slots, args.form, args.timeline)
     for _ in range(3):
         step()
@@ -280,7 +287,7 @@ def run_timeline(args) -> None:
     print(json.dumps(out))
 
 
-def run_backbone(args) -> None:
+def measure_backbone(steps: int, warmup: int) -> dict:
     """BASELINE configs[4]: decode-step latency of a synthetic 24-layer decoder (hidden 1024, 16 query /
     2 KV heads of 64, SwiGLU 4096, RMSNorm; 64 streams with context lengths U[128, 2048]; 32 rank-32
     adapters on all linears) with the LoRA kernels against the same step with LoRA disabled."""
@@ -307,31 +314,227 @@ def run_backbone(args) -> None:
             for _ in range(2):
                 out = model(x, caches, positions)
             torch.cuda.synchronize()
-            eager = time_region(lambda: model(x, caches, positions), 5)
+            eager = time_region(lambda: model(x, caches, positions), 3)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 out = model(x, caches, positions)
-            for _ in range(args.warmup):
+            for _ in range(warmup):
                 graph.replay()
-            ms = time_region(graph.replay, args.steps)
+            ms = time_region(graph.replay, steps)
         reset_lora_context()
         return ms, eager, out.float().clone()
 
     off_ms, off_eager, y_off = timed(False)
     on_ms, on_eager, y_on = timed(True)
-    print(json.dumps({
-        "metric": "decode-step latency of the synthetic backbone, LoRA kernels on vs LoRA disabled (us), 1 GPU",
-        "value": round(on_ms * 1e3, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(on_ms, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": WORKLOADS["backbone"]["text"], "streams": streams, "adapters": adapters, "rank": rank,
-                   "launch": "graph replay"},
-        "us_per_step_lora_off": round(off_ms * 1e3, 2),
-        "us_lora_cost": round((on_ms - off_ms) * 1e3, 2),
+    return {
+        "workload": WORKLOADS["backbone"]["text"], "streams": streams, "adapters": adapters, "rank": rank, "launch": "graph replay",
+        "steps": steps, "us_per_step": round(on_ms * 1e3, 2), "us_per_step_lora_off": round(off_ms * 1e3, 2),
+        "us_lora_cost": round((on_ms - off_ms) * 1e3, 2), "us_lora_cost_per_call": round((on_ms - off_ms) * 1e3 / (4 * NUM_LAYERS), 3),
         "lora_overhead_pct": round(100 * (on_ms - off_ms) / off_ms, 2),
         "us_per_step_eager": {"lora_on": round(on_eager * 1e3, 1), "lora_off": round(off_eager * 1e3, 1)},
         "lora_changes_output": bool((y_on - y_off).abs().max().item() > 0),
+    }
+
+
+def run_backbone(args) -> None:
+    r = measure_backbone(args.steps, args.warmup)
+    print(json.dumps({
+        "metric": "decode-step latency of the synthetic backbone, LoRA kernels on vs LoRA disabled (us), 1 GPU",
+        "value": r["us_per_step"], "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["us_per_step"] / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {k: r[k] for k in ("workload", "streams", "adapters", "rank", "launch")},
+        **{k: r[k] for k in ("us_per_step_lora_off", "us_lora_cost", "us_lora_cost_per_call", "lora_overhead_pct", "us_per_step_eager",
+                             "lora_changes_output")},
     }))
+
+
+KERNELS = {
+    "decode": "decode_kernel<bf16,16> (qkv, o, gate_up) + split_kernel<bf16,16> (down)",
+    "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
+    "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
+}
+
+
+def kernel_sources_sha256() -> str:
+    """Hash of the kernel sources: measured counter figures are quoted only for the sources they
+    were measured on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = ROOT / "nanovllm-voxcpm_amd" / "csrc"
+    for path in sorted(list(csrc.glob("*.hip")) + list(csrc.glob("*.h")) + [ROOT / "include" / "mlora.h"]):
+        h.update(path.name.encode())
+        h.update(path.read_bytes())
+    return h.hexdigest()
+
+
+def recorded_traffic(workload: str):
+    """HBM bytes per average launch of ``workload`` from the rocprofv3 counter runs summarised in
+    profiles/roofline.json, or None when that file was measured on other kernel sources."""
+    try:
+        rec = json.loads((ROOT / "profiles" / "roofline.json").read_text())
+    except (OSError, ValueError):
+        return None
+    if rec.get("kernel_sources_sha256") != kernel_sources_sha256():
+        return None
+    return rec.get("traffic_bytes_per_launch", {}).get(workload)
+
+
+def measure_workload(name: str, device: str, form: str, steps: int, warmup: int, *, only=None, rank=0, hot_layers=0, eager=False,
+                     per_projection=True, rank_vector=True) -> tuple[dict, tuple]:
+    """Time one workload: its step replayed as a captured graph (or eagerly), per-projection steps,
+    bytes, flops and the roofline object.  Returns (result, (layers, slots, rank, step))."""
+    import torch
+
+    spec = WORKLOADS[name]
+    rank = rank or spec["rank"]
+    layers, slots, eff = build_workload(name, device, rank)
+    if not rank_vector:
+        eff = None
+    if hot_layers > 0:
+        layers = [layers[i % hot_layers] for i in range(NUM_LAYERS)]
+    step, launches = make_step(layers, slots, form, only, eff)
+
+    num_tokens = slots.numel()
+    used_ids = torch.unique(slots[slots >= 0])
+    used = int(used_ids.numel())
+    t_lora = int((slots >= 0).sum())
+    rank_sum = token_rank_sum = None
+    if eff is not None:  # adapters of lower rank in rank-`rank` buffers, and the kernels are told
+        rank_sum = int(eff[used_ids.long()].sum())
+        token_rank_sum = int(eff[slots[slots >= 0].long()].sum())
+    names = [only] if only else list(ORDER)
+    shapes = {n: layers[0][n][0] for n in names}
+    per_proj = {n: algorithmic_bytes(p.k, p.widths, t_lora, used, rank, num_tokens, rank_sum) for n, p in shapes.items()}
+    per_proj_flops = {n: algorithmic_flops(p.k, p.widths, t_lora, rank, token_rank_sum) for n, p in shapes.items()}
+    step_bytes = NUM_LAYERS * sum(per_proj.values())
+    step_flops = NUM_LAYERS * sum(per_proj_flops.values())
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    eager_ms = time_region(step, max(3, min(steps, 20)))
+    if eager:
+        runner = step
+    else:
+        graph = capture(step)
+        runner = graph.replay
+    for _ in range(warmup):
+        runner()
+    ms = time_region(runner, steps)
+
+    # per-projection time: the same step restricted to one projection (24 launches)
+    per_proj_us = {}
+    if per_projection and not only and not eager:
+        for n in ORDER:
+            sub, cnt = make_step(layers, slots, form, n, eff)
+            g = capture(sub)
+            for _ in range(2):
+                g.replay()
+            per_proj_us[n] = round(time_region(g.replay, max(3, steps // 4)) * 1e3 / cnt, 3)
+
+    value = step_bytes / (ms * 1e-3) / 1e9
+    calls = launches
+    launch_bytes = step_bytes / calls
+    call_us = ms * 1e3 / calls
+    default_shape = form == "auto" and not only and not hot_layers and rank == spec["rank"]
+    result = {
+        "value": round(value, 2),
+        "ms_per_step": round(ms, 5),
+        "config": {
+            "workload": spec["text"] if rank == spec["rank"] else spec["text"] + f" -- run at rank {rank} instead",
+            "tokens": num_tokens, "tokens_with_adapter": t_lora, "adapters": spec["slots"], "adapters_in_batch": used,
+            "rank": rank, "layers": NUM_LAYERS, "projections": names, "form": form,
+            "launch": "eager" if eager else "graph replay",
+            "distinct_layer_buffers": hot_layers or spec["distinct_layers"],
+        },
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "us_per_step": round(ms * 1e3, 2),
+        "us_per_step_eager": round(eager_ms * 1e3, 2),
+        "algorithmic_bytes_per_step": step_bytes,
+        "algorithmic_flops_per_step": step_flops,
+        "tflops": round(step_flops / (ms * 1e-3) / 1e12, 2),
+        "pct_of_mfma_bf16_peak": round(100 * step_flops / (ms * 1e-3) / 1e12 / MFMA_BF16_TFLOPS, 3),
+        "calls_per_step": calls,
+        "us_per_call_by_projection": per_proj_us,
+        "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
+        "roofline": {
+            "kernel": "bgmv_kernel<bf16>" if form == "bgmv" else KERNELS[name],
+            "bound": "hbm",
+            # algorithmic bytes of an average call / time of an average call inside the replayed
+            # step (HIP events around the replays on the stream the kernels run on)
+            "achieved": round(value, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(value / HBM_PEAK_GBS, 4),
+            # HBM bytes per average call from the rocprofv3 counter runs (profiles/roofline.json),
+            # quoted only when the kernel sources are the ones those runs measured
+            "traffic": recorded_traffic(name) if default_shape else None,
+            "bytes_per_call": round(launch_bytes),
+            "us_per_call": round(call_us, 3),
+        },
+    }
+    if eff is not None:
+        result["config"]["true_rank_sum_of_adapters_in_batch"] = rank_sum
+        result["config"]["mean_true_rank_per_token"] = round(token_rank_sum / max(t_lora, 1), 2)
+    return result, (layers, slots, rank, step)
+
+
+def measure_floor(device: str, step_bytes: int, calls: int) -> dict:
+    """What bounds a step of `calls` dependent launches on this machine, measured in this run:
+    a replayed graph of as many kernels that do nothing (one wavefront each, then the grid of a
+    decode launch), the same number of real launches on a plan without any token to serve (every
+    workgroup fetches its tile record and leaves), and plain streams over a buffer of half a
+    step's bytes (read-modify-write as y is touched, and read-only)."""
+    import torch
+
+    from nanovllm_voxcpm_amd import _hip, synthetic
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend, LoRAMetadata
+
+    def graph_of(fn):
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        for _ in range(3):
+            g.replay()
+        return time_region(g.replay, 20) * 1e3
+
+    tiny = graph_of(lambda: [_hip.probe_launch(0, grid=(1, 1, 1), threads=64) for _ in range(calls)]) / calls
+    grid = graph_of(lambda: [_hip.probe_launch(0, grid=(8, 6, 6), threads=512) for _ in range(calls)]) / calls
+
+    # the real launches of a decode step on a batch in which no token has an adapter slot
+    backend = HipLoRABackend()
+    none = torch.full((256,), -1, dtype=torch.int32, device=device)
+    work = []
+    for j, name in enumerate(ORDER):
+        proj = synthetic.make_projection(name, 32, 16, torch.bfloat16, seed=90 + j, device=device)
+        x, y = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=95 + j, device=device)
+        blocks = list(y.split(proj.widths, dim=-1))
+        work.append((blocks, x, proj.a, proj.b, y if len(blocks) > 1 else None))
+
+    def empty_plan_step():
+        meta = LoRAMetadata(none, None, None, None, None, False, 0)
+        for i in range(calls):
+            blocks, x, a, b, packed = work[i % len(work)]
+            backend.add_lora(blocks, x, a, b, indices=none, metadata=meta, scaling=1.0, y_packed=packed)
+
+    empty_plan = graph_of(empty_plan_step) / calls
+
+    half = (step_bytes // 2 + 255) & ~255
+    buf = torch.zeros(half // 2, dtype=torch.bfloat16, device=device)
+    out = {"launches": calls, "us_per_empty_launch_one_wavefront": round(tiny, 3), "us_per_empty_launch_decode_grid": round(grid, 3),
+           "us_per_real_launch_on_a_plan_without_tokens": round(empty_plan, 3)}
+    for kind, key, factor in ((1, "stream_read_modify_write_gbs", 2), (2, "stream_read_only_gbs", 1)):
+        for _ in range(2):
+            _hip.probe_launch(kind, buf)
+        ms = time_region(lambda: _hip.probe_launch(kind, buf), 10)
+        out[key] = round(factor * half / (ms * 1e-3) / 1e9, 1)
+    # the step if every launch cost what a launch without tokens costs and its bytes moved at the
+    # rate of the read-modify-write stream, with no overlap between the two
+    out["us_per_step_floor_launches_plus_stream"] = round(calls * empty_plan + step_bytes / (out["stream_read_modify_write_gbs"] * 1e3), 1)
+    return out
 
 
 def main() -> None:
@@ -340,15 +543,21 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode", choices=sorted(WORKLOADS))
-    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | sgmv | token")
+    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | split | sgmv | token")
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip what the default run adds after the headline: the prefill, mixed and backbone steps and the floor")
+    ap.add_argument("--floor", action="store_true", help="print only the floor measurements (launch costs and stream rates)")
     ap.add_argument("--hot-layers", type=int, default=0,
                     help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
                          "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
     ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
                     help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
+    ap.add_argument("--no-rank-vector", action="store_true",
+                    help="diagnostic (mixed workload): do not tell the kernels the adapters' true ranks; the zero "
+                         "padding of the rank-64 buffers is then read and multiplied like any other data")
     ap.add_argument("--timeline", default=None, choices=ORDER,
                     help="diagnostic: in-kernel timeline of one projection's launch on the decode workload "
                          "(needs the trace build of the library)")
@@ -368,30 +577,15 @@ def main() -> None:
         sys.exit("bench.py: no ROCm GPU visible")
     device = "cuda:0"
     torch.cuda.set_device(0)
-    spec = WORKLOADS[args.workload]
-    rank = spec["rank"]
     if args.timeline:
         run_timeline(args)
         return
     if args.workload == "backbone":
         run_backbone(args)
         return
-    if args.rank and args.workload in ("decode", "prefill"):
-        rank = args.rank
-    layers, slots = build_workload(args.workload, device, rank)
-    if args.hot_layers > 0:
-        layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
-    step, launches = make_step(layers, slots, args.form, args.only)
-
-    num_tokens = slots.numel()
-    used = int(torch.unique(slots[slots >= 0]).numel())
-    t_lora = int((slots >= 0).sum())
-    names = [args.only] if args.only else list(ORDER)
-    shapes = {n: layers[0][n][0] for n in names}
-    per_proj = {n: algorithmic_bytes(p.k, p.widths, t_lora, used, rank, num_tokens) for n, p in shapes.items()}
-    per_proj_flops = {n: algorithmic_flops(p.k, p.widths, t_lora, rank) for n, p in shapes.items()}
-    step_bytes = NUM_LAYERS * sum(per_proj.values())
-    step_flops = NUM_LAYERS * sum(per_proj_flops.values())
+    if args.floor:
+        print(json.dumps({"floor": measure_floor(device, 918650880, 4 * NUM_LAYERS)}))
+        return
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device)
@@ -403,83 +597,26 @@ def main() -> None:
     heavy = args.workload != "decode"
     steps = args.steps if not heavy else max(3, min(args.steps, 30))
     warmup = args.warmup if not heavy else max(1, min(args.warmup, 3))
-    for _ in range(2):
-        step()
-    torch.cuda.synchronize()
-    eager_ms = time_region(step, max(3, min(steps, 50)))
-    if args.eager:
-        runner = step
-    else:
-        graph = capture(step)
-        runner = graph.replay
-    for _ in range(warmup):
-        runner()
-    ms = time_region(runner, steps)
-
-    # per-projection time: the same step restricted to one projection (24 launches)
-    per_proj_us = {}
-    if not args.only and not args.eager:
-        for n in ORDER:
-            sub, cnt = make_step(layers, slots, args.form, n)
-            g = capture(sub)
-            for _ in range(2):
-                g.replay()
-            per_proj_us[n] = round(time_region(g.replay, max(3, steps // 4)) * 1e3 / cnt, 3)
-
-    value = step_bytes / (ms * 1e-3) / 1e9
-    launch_bytes = step_bytes / launches
-    launch_us = ms * 1e3 / launches
-    achieved = launch_bytes / (launch_us * 1e-6) / 1e9
-    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers and rank == spec["rank"]
-    kernel = {"decode": "decode_kernel<bf16,16>", "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
-              "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>"}[args.workload]
-    if args.form == "bgmv":
-        kernel = "bgmv_kernel<bf16>"
+    rank = args.rank if args.workload in ("decode", "prefill") else 0
+    res, (layers, slots, rank, step) = measure_workload(args.workload, device, args.form, steps, warmup, only=args.only, rank=rank,
+                                                        hot_layers=args.hot_layers, eager=args.eager, rank_vector=not args.no_rank_vector)
     out = {
         "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
-        "value": round(value, 2),
+        "value": res["value"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,
-        "ms_per_step": round(ms, 5),
+        "ms_per_step": res["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {
-            "workload": spec["text"] if rank == spec["rank"] else spec["text"] + f" -- run at rank {rank} instead",
-            "tokens": num_tokens, "tokens_with_adapter": t_lora, "adapters": spec["slots"], "adapters_in_batch": used,
-            "rank": rank, "layers": NUM_LAYERS, "projections": names, "form": args.form,
-            "launch": "eager" if args.eager else "graph replay",
-            "distinct_layer_buffers": args.hot_layers or spec["distinct_layers"],
-        },
-        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-        "us_per_step": round(ms * 1e3, 2),
-        "us_per_step_eager": round(eager_ms * 1e3, 2),
-        "algorithmic_bytes_per_step": step_bytes,
-        "algorithmic_flops_per_step": step_flops,
-        "tflops": round(step_flops / (ms * 1e-3) / 1e12, 2),
-        "pct_of_mfma_bf16_peak": round(100 * step_flops / (ms * 1e-3) / 1e12 / MFMA_BF16_TFLOPS, 3),
-        "launches_per_step": launches + 1,
-        "us_per_launch_by_projection": per_proj_us,
-        "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
-        "roofline": {
-            "kernel": kernel,
-            "bound": "hbm",
-            "achieved": round(achieved, 2),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per average launch from the two rocprofv3 --pmc runs of the default workload
-            # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 256 MiB copy in the same runs);
-            # only quoted for the configuration those runs covered
-            "traffic": 9824051 if default_run else None,
-            "bytes_per_launch": round(launch_bytes),
-            "us_per_launch": round(launch_us, 3),
-        },
     }
+    out.update({k: v for k, v in res.items() if k not in ("value", "ms_per_step")})
+    out["launches_per_step"] = res["calls_per_step"] * (2 if args.workload != "decode" else 1) + 1
+
     # waits of the split form that ran out during everything above (0 in a healthy run: a consumer
     # workgroup that gives up computes its intermediate itself, which is correct but slow)
     from nanovllm_voxcpm_amd import _hip
@@ -488,8 +625,24 @@ def main() -> None:
     out["split_waits_run_out"] = sum(
         int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
         for buf in step.backend._scratch.values())
+
+    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers and not args.eager and not args.rank
+    if default_run and not args.no_extras:
+        # After the headline (outside its timed region): what one launch costs here and what a
+        # stream reaches here, and the other configurations of the benchmark, a few replays each.
+        out["floor"] = measure_floor(device, res["algorithmic_bytes_per_step"], res["calls_per_step"])
+        extra = {}
+        for name in ("prefill", "mixed"):
+            r, _ = measure_workload(name, device, "auto", 5, 2, per_projection=True)
+            extra[name] = {k: r[k] for k in ("config", "us_per_step", "value", "pct_of_hbm_peak", "tflops", "pct_of_mfma_bf16_peak",
+                                             "algorithmic_bytes_per_step", "us_per_call_by_projection", "roofline")}
+            extra[name]["unit"] = "GB/s"
+            torch.cuda.empty_cache()
+        extra["backbone"] = measure_backbone(10, 3)
+        torch.cuda.empty_cache()
+        out["extra"] = extra
     if not args.no_cpu_baseline and args.workload == "decode":
-        out["cpu_baseline"] = cpu_baseline(layers, slots, rank)
+        out["cpu_baseline"] = cpu_baseline(layers, slots, rank, budget_s=10.0)
     print(json.dumps(out))
 
 

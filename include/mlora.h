@@ -273,6 +273,14 @@ uint64_t mlora_stream_capture_id(void* stream);
  * this makes the next call read them again.  No counterpart in the reference. */
 void mlora_reload_knobs(void);
 
+/* Launches of known cost (measurement aid, no counterpart in the reference): kind 0 enqueues a
+ * kernel that does nothing with the given grid and workgroup size (what a launch costs by itself);
+ * kind 1 a read-modify-write stream over `bytes` of 16-bit elements at `buf` (every element read,
+ * incremented, written back once: the access pattern of y); kind 2 a read-only stream over them.
+ * bench.py quotes them beside the real kernels. */
+int mlora_probe_launch(void* stream, int32_t kind, void* buf, int64_t bytes, int32_t grid_x, int32_t grid_y, int32_t grid_z,
+                       int32_t threads);
+
 /* In-kernel timelines (diagnostic, no counterpart in the reference).  The library variant built
  * with `make trace` (libmlora_gfx950_trace.so) records, per workgroup of the small-tile kernels,
  * up to 16 readings of the 100 MHz clock at fixed points of the kernel into `buf` (uint64

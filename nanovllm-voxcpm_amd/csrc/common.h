@@ -115,6 +115,38 @@ __device__ __forceinline__ void mask_ranks(Pack8& p, int first, int eff) {
   for (int d = 0; d < 4; ++d) p.u[d] &= (2 * d < keep ? 0x0000ffffu : 0u) | (2 * d + 1 < keep ? 0xffff0000u : 0u);
 }
 
+// Rank of the adapter in a slot without a dependent fetch.  The slot of a tile is only known once
+// its record has arrived, and a fetch that waits for it costs a whole trip to memory in a kernel
+// that lives for a handful of trips.  The per-slot rank vector is small, so every lane requests
+// entries lane, lane + 64, ... of it together with the record (their addresses depend on nothing),
+// and the slot's entry is picked out of the registers afterwards.  Vectors beyond 256 slots fall
+// back to the dependent fetch.
+struct RankPrefetch {
+  int v[4];
+};
+__device__ __forceinline__ RankPrefetch rank_prefetch(const int32_t* __restrict__ eff_rank, int num_slots, int lane) {
+  RankPrefetch p;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    p.v[j] = (eff_rank && 64 * j < num_slots) ? eff_rank[i < num_slots ? i : num_slots - 1] : 0;
+  }
+  return p;
+}
+__device__ __forceinline__ int rank_pick(const RankPrefetch& p, const int32_t* __restrict__ eff_rank, int num_slots, int slot, int R) {
+  if (!eff_rank) return R;
+  int e;
+  if (num_slots <= 256) {
+    const int s = __builtin_amdgcn_readfirstlane(slot);  // the same in every lane
+    const int j = s >> 6;
+    const int word = j == 0 ? p.v[0] : j == 1 ? p.v[1] : j == 2 ? p.v[2] : p.v[3];
+    e = __builtin_amdgcn_readlane(word, s & 63);
+  } else {
+    e = eff_rank[slot];
+  }
+  return e < 0 ? 0 : e > R ? R : e;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -101,6 +101,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
   const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
   const DecodeSplit sp = splits.split[split_id];
+  const RankPrefetch ranks = rank_prefetch(eff_rank, num_slots, lane);
   const int slot = rec0[0], m = rec0[1];
   const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
   // One exit test, evaluated without short-circuit, that consumes everything fetched above
@@ -113,13 +114,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   if (!usable) return;
   MLORA_STAMP(1);  // tile record and plan header are here
 
-  // rank of the adapter in this slot (one more dependent fetch, only when the caller gave the vector)
-  int eff = R;
-  if (eff_rank) {
-    eff = eff_rank[slot];
-    eff = eff < 0 ? 0 : eff > R ? R : eff;
-    if (eff == 0) return;
-  }
+  // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
+  const int eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
+  if (eff == 0) return;
   const int rb_n = (eff + 15) >> 4;  // 16-rank blocks of A in use
 
   const bool live = lr < m;  // this lane's token exists

@@ -96,12 +96,14 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
 // after the previous one has been consumed; the launcher gives such parts the DB form).
 constexpr int kShrinkWaves = 4;
 
-template <typename T, int R, int KR, int XW, bool DB>
-__global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
-                                                                             float* __restrict__ hws, int64_t xs, int big_off,
-                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
-                                                                             int num_slots, int num_slices, int ksplit, int krange,
-                                                                             int all_slices, const int32_t* __restrict__ eff_rank, ShrinkSlices sl) {
+// Body of the shrink for one tile.  MASKED: the adapter in the tile's slot has fewer ranks than
+// the buffers (eff < R): 16-rank blocks of A[slot] at or above its rank are neither copied to LDS
+// nor multiplied, and their partial sums are not written (the expand does not read them).  The
+// unmasked instance is the code without any of those tests.
+template <typename T, int R, int KR, int XW, bool DB, bool MASKED>
+__device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                            float* __restrict__ hws, int64_t xs, int sorted_off, int T_, int K, int num_slices, int krange,
+                                            int all_slices, const ShrinkSlices& sl, int slice0, int kpart, int slot, int start, int m, int eff) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -113,29 +115,11 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   constexpr int SPB = XW / KR;           // slabs per x batch
   static_assert(XW % KR == 0 && XK <= 16, "batch shape");
 
-  __shared__ __attribute__((aligned(16))) T s_a[R * ASTRIDE];
-
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
-  // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
-  // registers (its K part is a single batch then), instead of one workgroup per slice
-  const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
   const int nsl = all_slices ? num_slices : 1;
-  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
-
-  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
-  if (!tr.ok) return;
-  const int slot = tr.slot, start = tr.start, m = tr.m;
-  // rank of the adapter in this slot: 16-rank blocks of A[slot] at or above it are neither copied
-  // to LDS nor multiplied, and their partial sums are not written (the expand does not read them)
-  int eff = R;
-  if (eff_rank) {
-    eff = eff_rank[slot];
-    eff = eff < 0 ? 0 : eff > R ? R : eff;
-    if (eff == 0) return;
-  }
-  const int rb_n = (eff + 15) >> 4;
-  const int rows_used = rb_n * 16 < R ? rb_n * 16 : R;
+  const int rb_n = MASKED ? (eff + 15) >> 4 : RB;          // 16-rank blocks of A[slot] in use
+  const int rows_used = MASKED ? (rb_n * 16 < R ? rb_n * 16 : R) : R;
 
   const int k0 = kpart * krange;
   const int nbatch = krange / XW;
@@ -152,14 +136,20 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = i * NT + tid;
-      if ((TOTAL % NT == 0 || c < TOTAL) && c / CPR < rows_used) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
+      if constexpr (MASKED) {
+        if (i * (NT / CPR) >= rows_used) continue;  // these rows lie beyond the adapter's rank (the same for every thread)
+      }
+      if (TOTAL % NT == 0 || c < TOTAL) v[i] = load128(Aslab + static_cast<int64_t>(c / CPR) * K + (c % CPR) * 8);
     }
   };
   auto store_slab = [&]() {
 #pragma unroll
     for (int i = 0; i < CHUNKS; ++i) {
       const int c = i * NT + tid;
-      if ((TOTAL % NT == 0 || c < TOTAL) && c / CPR < rows_used) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
+      if constexpr (MASKED) {
+        if (i * (NT / CPR) >= rows_used) continue;
+      }
+      if (TOTAL % NT == 0 || c < TOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / CPR) * ASTRIDE + (c % CPR) * 8]) = v[i];
     }
   };
   auto request_x = [&](Pack8(&buf)[XK], int kc) {
@@ -189,7 +179,9 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
         for (int i = 0; i < KS; ++i) {
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
-            if (RB > 1 && rb >= rb_n) continue;
+            if constexpr (MASKED) {
+              if (rb >= rb_n) continue;
+            }
             const int rr = rb * 16 + lr;
             Pack8 aw;
             aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + i * 32 + lg * 8]);
@@ -220,10 +212,40 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const int r0 = rb * 16 + 4 * lg;
-        if (r0 < R && rb < rb_n) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
+        if (r0 < R && (!MASKED || rb < rb_n)) *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
       }
     }
   }
+}
+
+
+template <typename T, int R, int KR, int XW, bool DB>
+__global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
+                                                                             float* __restrict__ hws, int64_t xs, int big_off,
+                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
+                                                                             int num_slots, int num_slices, int ksplit, int krange,
+                                                                             int all_slices, const int32_t* __restrict__ eff_rank, ShrinkSlices sl) {
+  constexpr int ASTRIDE = KR + 8;  // padded LDS row: 16 rows x 16 bytes cover all banks once
+  __shared__ __attribute__((aligned(16))) T s_a[R * ASTRIDE];
+  // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
+  // registers (its K part is a single batch then), instead of one workgroup per slice
+  const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
+  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
+  if (!tr.ok) return;
+  // rank of the adapter in this slot (a second, dependent fetch, only with the vector given)
+  int eff = R;
+  if (R > 16 && eff_rank) {
+    eff = eff_rank[tr.slot];
+    eff = eff < 0 ? 0 : eff > R ? R : eff;
+    if (eff == 0) return;
+  }
+  if (R > 16 && ((eff + 15) >> 4) < (R + 15) / 16)
+    shrink_body<T, R, KR, XW, DB, true>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart,
+                                        tr.slot, tr.start, tr.m, eff);
+  else
+    shrink_body<T, R, KR, XW, DB, false>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart,
+                                         tr.slot, tr.start, tr.m, eff);
 }
 
 // ---- expand -------------------------------------------------------------------------------------
@@ -265,12 +287,16 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
   else *reinterpret_cast<Raw*>(p) = r;
 }
 
-template <typename T, int R, int CPL, int TPF, int G>
-__global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
-                                                                             void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
-                                                                             int big_units, int sorted_off, int T_, int num_slots,
-                                                                             int num_slices, int ksplit, float scaling, int nt,
-                                                                             const int32_t* __restrict__ eff_rank, ExpandSplits splits) {
+// Body of the expand for the tiles of one workgroup.  MASKED: some tile's slot holds an adapter of
+// fewer ranks than the buffers: chunks of the intermediate the shrink did not write are not read,
+// ranks at or above the adapter's are zero in the intermediate, B columns from that rank on are
+// neither fetched nor multiplied.  The unmasked instance is the code without any of those tests.
+template <typename T, int R, int CPL, int TPF, int G, bool MASKED>
+__device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict__ s_row, int* __restrict__ s_slot, int* __restrict__ s_m,
+                                            int* __restrict__ s_eff, const int32_t* __restrict__ plan, const float* __restrict__ hws,
+                                            void* __restrict__ yv_, int64_t ys, int sorted_off, int T_, int num_slices, int ksplit,
+                                            float scaling, int nt, const ExpandSplit& sp, const int (&slot)[G], const int (&start)[G],
+                                            const int (&m)[G], const int (&eff)[G]) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int NB = TB / TPF;           // y batches per tile
   constexpr int STEPS = G * NB;          // (tile, batch) steps of a span
@@ -281,6 +307,239 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   constexpr int SPAN = 16 * CPL;         // columns of one span
   constexpr int HC = (MLORA_TILE_BIG * CPR + NT - 1) / NT;  // H chunks per thread and tile
 
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int lr = lane & 15, lg = lane >> 4;
+
+  // token rows -> LDS (entries past the end of a tile repeat its last token: a valid row to read,
+  // never written)
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
+    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
+  }
+  __syncthreads();
+
+  // A wavefront's work is a sequence of items: for each of its spans of 16 * CPL columns, the
+  // (tile, y batch) steps that hold tokens.  The y rows of the item after the current one are
+  // always in flight, and those of the first item (and its B rows) go out before the H tiles
+  // are staged, so that the stream of y never waits for anything but itself.
+  T* const ybase = static_cast<T*>(yv_) + sp.y_col;
+  auto next_step = [&](int st) {
+    for (++st; st < STEPS; ++st)
+      if (s_m[st / NB] > (st % NB) * TPF * 16) break;
+    return st;
+  };
+  const int first_step = next_step(-1);  // exists: some tile holds tokens
+  auto column = [&](int c0) {  // first of this lane's CPL columns, clamped into the range
+    const int c = c0 + CPL * lr;
+    return c < sp.n1 ? c : sp.n1 - 8;
+  };
+  auto issue_y = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+    const int g = st / NB, tp = (st % NB) * TPF, cl = column(c0);
+#pragma unroll
+    for (int u = 0; u < TPF; ++u) {
+      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + (tp + u) * 16 + 4 * lg]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) buf[u][i] = load_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + cl, nt);
+    }
+  };
+  Pack8 bop[CPL][KSTEPS];
+  int b_slot = -1, b_c0 = -1;  // what bop holds
+  int b_ks = KSTEPS;  // k-steps of the slot bop holds
+  auto load_b = [&](int c0, int sg, int eg) {
+    // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
+    // their H operand is zero; columns past the range repeat the last one and are never stored)
+    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
+    if (!MASKED || eg >= R) {
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        int n = c0 + CPL * lr + j;
+        n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = (lg + 4 * ks) & (R / 8 - 1);
+          bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+        }
+      }
+    } else if constexpr (MASKED) {
+      // an adapter of lower rank: only its own chunks of eight ranks are fetched, the rest of the
+      // operand is zero, and what the boundary chunk holds beyond the rank is masked out
+      const int eg8 = (eg + 7) >> 3;
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        int n = c0 + CPL * lr + j;
+        n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int kc = lg + 4 * ks;
+          if (kc < eg8) {
+            bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+            if (eg & 7) mask_ranks(bop[j][ks], kc * 8, eg);
+          } else {
+            bop[j][ks].raw = i32x4{0, 0, 0, 0};
+          }
+        }
+      }
+    }
+    b_slot = sg;
+    b_c0 = c0;
+    if constexpr (MASKED) b_ks = (eg + 31) >> 5;
+  };
+  auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+    const int g = st / NB, tp = (st % NB) * TPF;
+    const int mg = s_m[g], sg = s_slot[g];
+    if (sg != b_slot || c0 != b_c0) load_b(c0, sg, s_eff[g]);
+    const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
+    const int c = c0 + CPL * lr;
+    const bool col_ok = c < sp.n1;
+#pragma unroll
+    for (int u = 0; u < TPF; ++u) {
+      const int tb = tp + u;
+      if (tb * 16 >= mg) continue;
+      Pack8 hop[KSTEPS], hlo[KSTEPS];
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kc = lg + 4 * ks;
+        if (kc * 8 < R) {
+          hop[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + kc * 8]);
+          hlo[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
+        } else {
+          hop[ks].raw = i32x4{0, 0, 0, 0};
+          hlo[ks].raw = i32x4{0, 0, 0, 0};
+        }
+      }
+      f32x4 out[CPL];
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          if constexpr (MASKED && KSTEPS > 1) {
+            if (ks >= b_ks) continue;
+          }
+          out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
+          out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
+        }
+      }
+      // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
+      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + tb * 16 + 4 * lg]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (col_ok && tb * 16 + 4 * lg + i < mg) {
+          YVec<T, CPL> r;
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(buf[u][i].e[j]) + out[j][i]);
+          store_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + c, r, nt);
+        }
+      }
+    }
+  };
+
+  YVec<T, CPL> ya[TPF][4], yb[TPF][4];
+  int c0 = sp.n0 + wave * SPAN, st = first_step;
+  const bool has_work = c0 < sp.n1;
+  if (has_work) {
+    load_b(c0, s_slot[st / NB], s_eff[st / NB]);
+    issue_y(ya, c0, st);
+  }
+
+  // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
+  // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
+  {
+    const int64_t hrow = static_cast<int64_t>(num_slices) * R;
+    const int64_t part = static_cast<int64_t>(T_) * hrow;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (m[g] == 0) continue;
+      const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
+      f32x4 t[HC][kMaxKSplit][2];
+#pragma unroll
+      for (int h = 0; h < HC; ++h) {
+        const int c = h * NT + tid;
+        int tok = c / CPR;
+        tok = tok < m[g] ? tok : m[g] - 1;
+        const float* q = src + tok * hrow + (c % CPR) * 8;
+        const bool used = !MASKED || (c % CPR) * 8 < ((eff[g] + 15) & ~15);  // the shrink wrote this chunk
+#pragma unroll
+        for (int kp = 0; kp < kMaxKSplit; ++kp) {
+          if (kp < ksplit) {
+            if (used) {
+              t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
+              t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+            } else {
+              t[h][kp][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+              t[h][kp][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int h = 0; h < HC; ++h) {
+        const int c = h * NT + tid, tok = c / CPR, ch = c % CPR;
+        if ((MLORA_TILE_BIG * CPR) % NT != 0 && c >= MLORA_TILE_BIG * CPR) continue;
+        f32x4 s0 = t[h][0][0], s1 = t[h][0][1];
+#pragma unroll
+        for (int kp = 1; kp < kMaxKSplit; ++kp) {
+          if (kp < ksplit) {
+            s0[0] += t[h][kp][0][0]; s0[1] += t[h][kp][0][1]; s0[2] += t[h][kp][0][2]; s0[3] += t[h][kp][0][3];
+            s1[0] += t[h][kp][1][0]; s1[1] += t[h][kp][1][1]; s1[2] += t[h][kp][1][2]; s1[3] += t[h][kp][1][3];
+          }
+        }
+        Pack8 hi, lo;
+        float v[8], back[8], rem[8];
+        const float live = tok < m[g] ? scaling : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = (!MASKED || ch * 8 + i < eff[g]) ? s0[i] * live : 0.f;  // ranks the adapter does not have contribute nothing
+          v[4 + i] = (!MASKED || ch * 8 + 4 + i < eff[g]) ? s1[i] * live : 0.f;
+        }
+        pack8<T>(v, hi);
+        unpack8<T>(hi, back);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
+        pack8<T>(rem, lo);
+        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
+        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
+      }
+    }
+  }
+  __syncthreads();
+  if (!has_work) return;
+
+  // two y buffers, used in turn
+  auto advance = [&](int& nc0, int& nst) {  // item after (c0, st); false when there is none
+    nst = next_step(st);
+    nc0 = c0;
+    if (nst >= STEPS) {
+      nst = first_step;
+      nc0 = c0 + kExpandWaves * SPAN;
+    }
+    return nc0 < sp.n1;
+  };
+  for (;;) {
+    int nc0, nst;
+    bool more = advance(nc0, nst);
+    if (more) issue_y(yb, nc0, nst);
+    process(ya, c0, st);
+    if (!more) break;
+    c0 = nc0;
+    st = nst;
+    more = advance(nc0, nst);
+    if (more) issue_y(ya, nc0, nst);
+    process(yb, c0, st);
+    if (!more) break;
+    c0 = nc0;
+    st = nst;
+  }
+}
+
+template <typename T, int R, int CPL, int TPF, int G>
+__global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
+                                                                             void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
+                                                                             int big_units, int sorted_off, int T_, int num_slots,
+                                                                             int num_slices, int ksplit, float scaling, int nt,
+                                                                             const int32_t* __restrict__ eff_rank, ExpandSplits splits) {
+  constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
   __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
   __shared__ __attribute__((aligned(16))) int s_row[G * MLORA_TILE_BIG];
   __shared__ int s_slot[G], s_m[G], s_eff[G];
@@ -330,225 +589,15 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
   if (!usable) return;
 
-  // token rows -> LDS (entries past the end of a tile repeat its last token: a valid row to read,
-  // never written)
+  bool masked = false;
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
-    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
-  }
-  __syncthreads();
-
-  // A wavefront's work is a sequence of items: for each of its spans of 16 * CPL columns, the
-  // (tile, y batch) steps that hold tokens.  The y rows of the item after the current one are
-  // always in flight, and those of the first item (and its B rows) go out before the H tiles
-  // are staged, so that the stream of y never waits for anything but itself.
-  T* const ybase = static_cast<T*>(yv_) + sp.y_col;
-  auto next_step = [&](int st) {
-    for (++st; st < STEPS; ++st)
-      if (s_m[st / NB] > (st % NB) * TPF * 16) break;
-    return st;
-  };
-  const int first_step = next_step(-1);  // exists: some tile holds tokens
-  auto column = [&](int c0) {  // first of this lane's CPL columns, clamped into the range
-    const int c = c0 + CPL * lr;
-    return c < sp.n1 ? c : sp.n1 - 8;
-  };
-  auto issue_y = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
-    const int g = st / NB, tp = (st % NB) * TPF, cl = column(c0);
-#pragma unroll
-    for (int u = 0; u < TPF; ++u) {
-      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + (tp + u) * 16 + 4 * lg]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) buf[u][i] = load_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + cl, nt);
-    }
-  };
-  Pack8 bop[CPL][KSTEPS];
-  int b_slot = -1, b_c0 = -1;  // what bop holds
-  int b_ks = KSTEPS;  // k-steps of the slot bop holds
-  auto load_b = [&](int c0, int sg, int eg) {
-    // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
-    // their H operand is zero; columns past the range repeat the last one and are never stored)
-    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(sg) * sp.n * R;
-    if (eg >= R) {
-#pragma unroll
-      for (int j = 0; j < CPL; ++j) {
-        int n = c0 + CPL * lr + j;
-        n = n < sp.n1 ? n : sp.n1 - 1;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int kc = (lg + 4 * ks) & (R / 8 - 1);
-          bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-        }
-      }
-    } else {
-      // an adapter of lower rank: only its own chunks of eight ranks are fetched, the rest of the
-      // operand is zero, and what the boundary chunk holds beyond the rank is masked out
-      const int eg8 = (eg + 7) >> 3;
-#pragma unroll
-      for (int j = 0; j < CPL; ++j) {
-        int n = c0 + CPL * lr + j;
-        n = n < sp.n1 ? n : sp.n1 - 1;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int kc = lg + 4 * ks;
-          if (kc < eg8) {
-            bop[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-            if (eg & 7) mask_ranks(bop[j][ks], kc * 8, eg);
-          } else {
-            bop[j][ks].raw = i32x4{0, 0, 0, 0};
-          }
-        }
-      }
-    }
-    b_slot = sg;
-    b_c0 = c0;
-    b_ks = (eg + 31) >> 5;
-  };
-  auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
-    const int g = st / NB, tp = (st % NB) * TPF;
-    const int mg = s_m[g], sg = s_slot[g];
-    if (sg != b_slot || c0 != b_c0) load_b(c0, sg, s_eff[g]);
-    const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
-    const int c = c0 + CPL * lr;
-    const bool col_ok = c < sp.n1;
-#pragma unroll
-    for (int u = 0; u < TPF; ++u) {
-      const int tb = tp + u;
-      if (tb * 16 >= mg) continue;
-      Pack8 hop[KSTEPS], hlo[KSTEPS];
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int kc = lg + 4 * ks;
-        if (kc * 8 < R) {
-          hop[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + kc * 8]);
-          hlo[ks].raw = *reinterpret_cast<const i32x4*>(&hg[(tb * 16 + lr) * HSTRIDE + R + kc * 8]);
-        } else {
-          hop[ks].raw = i32x4{0, 0, 0, 0};
-          hlo[ks].raw = i32x4{0, 0, 0, 0};
-        }
-      }
-      f32x4 out[CPL];
-#pragma unroll
-      for (int j = 0; j < CPL; ++j) {
-        out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          if (KSTEPS > 1 && ks >= b_ks) continue;
-          out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
-          out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
-        }
-      }
-      // lane holds out[token 16*tb + 4*lg + i][column c0 + CPL*lr + j]
-      const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + tb * 16 + 4 * lg]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (col_ok && tb * 16 + 4 * lg + i < mg) {
-          YVec<T, CPL> r;
-#pragma unroll
-          for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(buf[u][i].e[j]) + out[j][i]);
-          store_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + c, r, nt);
-        }
-      }
-    }
-  };
-
-  YVec<T, CPL> ya[TPF][4], yb[TPF][4];
-  int c0 = sp.n0 + wave * SPAN, st = first_step;
-  const bool has_work = c0 < sp.n1;
-  if (has_work) {
-    load_b(c0, s_slot[st / NB], s_eff[st / NB]);
-    issue_y(ya, c0, st);
-  }
-
-  // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
-  // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
-  {
-    const int64_t hrow = static_cast<int64_t>(num_slices) * R;
-    const int64_t part = static_cast<int64_t>(T_) * hrow;
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      if (m[g] == 0) continue;
-      const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
-      f32x4 t[HC][kMaxKSplit][2];
-#pragma unroll
-      for (int h = 0; h < HC; ++h) {
-        const int c = h * NT + tid;
-        int tok = c / CPR;
-        tok = tok < m[g] ? tok : m[g] - 1;
-        const float* q = src + tok * hrow + (c % CPR) * 8;
-        const bool used = (c % CPR) * 8 < ((eff[g] + 15) & ~15);  // the shrink wrote this chunk
-#pragma unroll
-        for (int kp = 0; kp < kMaxKSplit; ++kp) {
-          if (kp < ksplit) {
-            if (used) {
-              t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
-              t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
-            } else {
-              t[h][kp][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-              t[h][kp][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int h = 0; h < HC; ++h) {
-        const int c = h * NT + tid, tok = c / CPR, ch = c % CPR;
-        if ((MLORA_TILE_BIG * CPR) % NT != 0 && c >= MLORA_TILE_BIG * CPR) continue;
-        f32x4 s0 = t[h][0][0], s1 = t[h][0][1];
-#pragma unroll
-        for (int kp = 1; kp < kMaxKSplit; ++kp) {
-          if (kp < ksplit) {
-            s0[0] += t[h][kp][0][0]; s0[1] += t[h][kp][0][1]; s0[2] += t[h][kp][0][2]; s0[3] += t[h][kp][0][3];
-            s1[0] += t[h][kp][1][0]; s1[1] += t[h][kp][1][1]; s1[2] += t[h][kp][1][2]; s1[3] += t[h][kp][1][3];
-          }
-        }
-        Pack8 hi, lo;
-        float v[8], back[8], rem[8];
-        const float live = tok < m[g] ? scaling : 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          v[i] = ch * 8 + i < eff[g] ? s0[i] * live : 0.f;  // ranks the adapter does not have contribute nothing
-          v[4 + i] = ch * 8 + 4 + i < eff[g] ? s1[i] * live : 0.f;
-        }
-        pack8<T>(v, hi);
-        unpack8<T>(hi, back);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
-        pack8<T>(rem, lo);
-        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
-        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
-      }
-    }
-  }
-  __syncthreads();
-  if (!has_work) return;
-
-  // two y buffers, used in turn
-  auto advance = [&](int& nc0, int& nst) {  // item after (c0, st); false when there is none
-    nst = next_step(st);
-    nc0 = c0;
-    if (nst >= STEPS) {
-      nst = first_step;
-      nc0 = c0 + kExpandWaves * SPAN;
-    }
-    return nc0 < sp.n1;
-  };
-  for (;;) {
-    int nc0, nst;
-    bool more = advance(nc0, nst);
-    if (more) issue_y(yb, nc0, nst);
-    process(ya, c0, st);
-    if (!more) break;
-    c0 = nc0;
-    st = nst;
-    more = advance(nc0, nst);
-    if (more) issue_y(ya, nc0, nst);
-    process(yb, c0, st);
-    if (!more) break;
-    c0 = nc0;
-    st = nst;
-  }
+  for (int g = 0; g < G; ++g) masked |= m[g] > 0 && eff[g] < R;
+  if (masked)
+    expand_body<T, R, CPL, TPF, G, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
+                                         sp, slot, start, m, eff);
+  else
+    expand_body<T, R, CPL, TPF, G, false>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
+                                          sp, slot, start, m, eff);
 }
 
 // The fp32 partials of the intermediate live behind the head of the workspace.

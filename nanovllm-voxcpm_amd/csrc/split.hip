@@ -109,6 +109,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
   const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
   const uint32_t signature = ws[0];
+  const RankPrefetch ranks = rank_prefetch(eff_rank, num_slots, lane);
   uint32_t* const tstate = ws + kWsTileOff / 4 + 2 * tile;  // {generation, arrivals}; tile < kWsTiles (host)
   const uint32_t tag = tstate[0] + 1u;
   const int slot = rec0[0], m = rec0[1];
@@ -121,13 +122,9 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   MLORA_STAMP(1);  // tile record, plan header and tile generation are here
   const bool xok = trusted | (signature == kWsMagic);  // the exchange area can be used
 
-  // rank of the adapter in this slot (one more dependent fetch, only when the caller gave the vector)
-  int eff = R;
-  if (eff_rank) {
-    eff = eff_rank[slot];
-    eff = eff < 0 ? 0 : eff > R ? R : eff;
-    if (eff == 0) return;  // nothing resident: the same for every workgroup of the tile
-  }
+  // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
+  const int eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
+  if (eff == 0) return;  // nothing resident: the same for every workgroup of the tile
   const int rb_n = (eff + 15) >> 4;  // 16-rank blocks of A in use
 
   const bool producer = role < S * P;

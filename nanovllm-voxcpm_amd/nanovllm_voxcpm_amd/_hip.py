@@ -61,6 +61,7 @@ EXPORTS = (
     "mlora_stream_capture_id",
     "mlora_reload_knobs",
     "mlora_trace_set",
+    "mlora_probe_launch",
     "mlora_abi_version",
     "mlora_last_error",
     "mlora_build_info",
@@ -223,6 +224,8 @@ def load() -> C.CDLL:
     lib.mlora_workspace_init.restype = C.c_int
     lib.mlora_stream_capture_id.argtypes = [C.c_void_p]
     lib.mlora_stream_capture_id.restype = C.c_uint64
+    lib.mlora_probe_launch.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.mlora_probe_launch.restype = C.c_int
     lib.mlora_trace_set.argtypes = [C.c_void_p]
     lib.mlora_trace_set.restype = C.c_int
     lib.mlora_reload_knobs.argtypes = []
@@ -560,6 +563,17 @@ def stream_capture_id(device: torch.device, stream: int | None = None) -> int:
 def reload_knobs() -> None:
     """Make the library read its MLORA_* environment variables again (it keeps them otherwise)."""
     load().mlora_reload_knobs()
+
+
+def probe_launch(kind: int, buf: torch.Tensor | None = None, grid: tuple[int, int, int] = (1, 1, 1), threads: int = 64,
+                 device: torch.device | None = None) -> None:
+    """Enqueue a launch of known cost on torch's current stream: kind 0 an empty kernel of the given
+    shape, kind 1 a read-modify-write stream over ``buf``, kind 2 a read-only stream over it."""
+    dev = buf.device if buf is not None else (device or torch.device("cuda", torch.cuda.current_device()))
+    nbytes = buf.numel() * buf.element_size() if buf is not None else 0
+    with _on(dev):
+        _check(load().mlora_probe_launch(_stream(dev), kind, buf.data_ptr() if buf is not None else None, nbytes, *grid, threads),
+               "mlora_probe_launch")
 
 
 def trace_set(buf: torch.Tensor | None) -> None:

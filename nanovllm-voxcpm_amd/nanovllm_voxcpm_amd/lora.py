@@ -108,6 +108,8 @@ class HipLoRABackend:
             raise ValueError(f"unknown LoRA kernel form {name!r}; expected one of {sorted(_hip.FORMS)}")
         self.form = name
         self._scratch: dict = {}
+        self._spares: dict = {}          # device -> initialised buffer kept for the next graph capture
+        self._graph_scratch: list = []   # buffers captured graphs refer to
 
     # -- capability ---------------------------------------------------------------------
     def availability(self) -> LoRAAvailability:
@@ -179,13 +181,22 @@ class HipLoRABackend:
             plan = cache[key] = build_segment_plan(tts, max_slots)
         return plan
 
+    def _new_scratch(self, device: torch.device, nbytes: int, stream: int | None) -> torch.Tensor:
+        buf = torch.empty(max(nbytes, 4 << 20), dtype=torch.uint8, device=device)
+        _hip.workspace_init(buf, stream)  # one kernel, once per buffer: head cleared, signature written
+        return buf
+
     def _scratch_for(self, x: torch.Tensor, num_slices: int, rank: int, stream: int | None = None,
                      capture: int | None = None) -> torch.Tensor:
         """Device scratch for the rank-r intermediate (between the two launches of the
-        long-segment form, or between workgroups sharing one shrink).  One buffer per
-        (device, stream), grown on demand: calls on one stream are ordered, so they can share
-        it; a buffer first created while a graph is being captured belongs to that graph's
-        memory pool and is not kept for later eager calls."""
+        long-segment form, or between producer and consumer workgroups of the split form).  One
+        buffer per (device, stream), grown on demand: calls on one stream are ordered, so they can
+        share it.  A graph being captured gets a buffer of its own (its replays may run beside
+        eager calls of any stream): preferably one that was allocated and initialised outside the
+        capture — every eager call keeps such a spare ready — so that the graph holds no
+        initialisation launch; the graph refers to it for as long as it lives, so it is never
+        freed.  Without a spare the buffer comes from the graph's own pool and its initialisation
+        is recorded with it."""
         nbytes = _hip.add_workspace_bytes(x.size(0), num_slices, rank, x.dtype)
         if stream is None:
             stream = _hip.current_stream_handle(x.device)
@@ -193,11 +204,25 @@ class HipLoRABackend:
             capture = _hip.stream_capture_id(x.device, stream)
         key = (x.device, stream, capture)
         buf = self._scratch.get(key)
-        if buf is None or buf.numel() < nbytes:
-            if len(self._scratch) >= 8:
-                self._scratch.clear()
-            buf = self._scratch[key] = torch.empty(max(nbytes, 4 << 20), dtype=torch.uint8, device=x.device)
-            _hip.workspace_init(buf, stream)  # one kernel, once per buffer: head cleared, signature written
+        if buf is not None and buf.numel() >= nbytes:
+            if not capture and x.device not in self._spares:  # a capture took the spare: make the next one
+                self._spares[x.device] = self._new_scratch(x.device, buf.numel(), stream)
+            return buf
+        if capture:
+            spare = self._spares.pop(x.device, None)
+            if spare is not None and spare.numel() >= nbytes:
+                self._graph_scratch.append(spare)
+                self._scratch[key] = spare
+                return spare
+            if spare is not None:
+                self._spares[x.device] = spare
+        if len(self._scratch) >= 8:
+            self._scratch.clear()
+        buf = self._scratch[key] = self._new_scratch(x.device, nbytes, stream)
+        if not capture:
+            spare = self._spares.get(x.device)
+            if spare is None or spare.numel() < buf.numel():
+                self._spares[x.device] = self._new_scratch(x.device, buf.numel(), stream)
         return buf
 
     @staticmethod

@@ -173,3 +173,108 @@ def test_checkpoint_to_resident_slot_to_forward(tmp_path):
         install_lora_payload(model, 0, load_voxcpm_lora_checkpoint(str(_write(tmp_path / "second" / "demo_lora", {"zzz.o_proj.lora_A": rnd(r, 8), "zzz.o_proj.lora_B": rnd(8, r)}, {"lora_config": {"alpha": 2.0}}))))
     with pytest.raises(ValueError, match="does not support LoRA slots"):
         install_lora_payload(model, 0, load_voxcpm_lora_checkpoint(str(_write(tmp_path / "second" / "demo_lora" / "demo_lora", {"blk.plain.lora_A": rnd(r, 8), "blk.plain.lora_B": rnd(8, r)}, {"lora_config": {"alpha": 2.0}}))))
+
+
+def test_mismatched_payload_is_refused_before_anything_is_written(tmp_path):
+    """A checkpoint made for another hidden size: every module's payload is validated against the
+    module before the first write, so the slot keeps its previous adapter."""
+    from nanovllm_voxcpm_amd.lora_checkpoint import install_lora_payload, load_voxcpm_lora_checkpoint
+
+    g = torch.Generator().manual_seed(5)
+    rnd = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    model = nn.ModuleDict({"blk": _Block()})
+    good = {"blk.o_proj.lora_A": rnd(2, 8), "blk.o_proj.lora_B": rnd(8, 2)}
+    install_lora_payload(model, 0, load_voxcpm_lora_checkpoint(str(_write(tmp_path, good))))
+    before = (model["blk"].o_proj.lora_A.detach().clone(), model["blk"].qkv_proj.lora_A.detach().clone())
+    bad = {"blk.q_proj.lora_A": rnd(2, 8), "blk.q_proj.lora_B": rnd(8, 2),
+           "blk.o_proj.lora_A": rnd(2, 16), "blk.o_proj.lora_B": rnd(8, 2)}  # o_proj for a model twice as wide
+    (tmp_path / "bad").mkdir()
+    with pytest.raises(ValueError, match="input dim 8"):
+        install_lora_payload(model, 0, load_voxcpm_lora_checkpoint(str(_write(tmp_path / "bad", bad))))
+    assert torch.equal(model["blk"].o_proj.lora_A.detach(), before[0]) and torch.equal(model["blk"].qkv_proj.lora_A.detach(), before[1])
+    with pytest.raises(IndexError, match="outside the 2 slots"):
+        install_lora_payload(model, 2, load_voxcpm_lora_checkpoint(str(tmp_path / "demo_lora")))
+
+
+class _WideBlock(nn.Module):
+    def __init__(self, hidden=256, heads=4, kv_heads=2, head_dim=64, inter=512, max_loras=3, rank=16):
+        super().__init__()
+        from nanovllm_voxcpm_amd.layers.lora import LoRAMergedColumnParallelLinear, LoRAQKVParallelLinear, LoRARowParallelLinear
+
+        kw = dict(max_loras=max_loras, max_lora_rank=rank)
+        self.qkv_proj = LoRAQKVParallelLinear(hidden, head_dim, heads, kv_heads, **kw)
+        self.o_proj = LoRARowParallelLinear(heads * head_dim, hidden, **kw)
+        self.gate_up_proj = LoRAMergedColumnParallelLinear(hidden, [inter, inter], **kw)
+        self.down_proj = LoRARowParallelLinear(inter, hidden, **kw)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_checkpoint_to_resident_slot_to_forward_on_the_gpu(tmp_path, dtype):
+    """The device leg of adapter admission: checkpoint directory -> payload packed into one pinned
+    host buffer -> one copy to the device -> one install launch per target -> forward of every
+    LoRA linear through the HIP kernels, against x W^T + (alpha / r) (x A^T) B^T in fp64; then a
+    second adapter of lower rank replaces the first in the same slot (reference:
+    nanovllm_voxcpm/models/voxcpm/lora_loader.py:27-42, 134-163, engine/model_runner.py:389-420,
+    fixture shape of tests/unit/test_voxcpm_lora_checkpoint_loader.py:9-69)."""
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend, get_backend
+    from nanovllm_voxcpm_amd.lora_checkpoint import install_lora_payload, load_voxcpm_lora_checkpoint
+    from nanovllm_voxcpm_amd.utils.context import LoRAContext, reset_lora_context, set_lora_context
+
+    print(f"checkpoint -> slot -> forward {dtype}", flush=True)
+    assert isinstance(get_backend(), HipLoRABackend)
+    g = torch.Generator().manual_seed(7)
+    rnd = lambda *s: torch.randn(*s, generator=g) * 0.05  # noqa: E731
+    hidden, q, kv, inter = 256, 256, 128, 512
+    model = nn.ModuleDict({"blk": _WideBlock()}).to(device="cuda", dtype=dtype)
+    mods = {n: getattr(model["blk"], n) for n in ("qkv_proj", "o_proj", "gate_up_proj", "down_proj")}
+    with torch.no_grad():
+        for m in mods.values():
+            m.weight.copy_((torch.randn(m.weight.shape, generator=g) * 0.05).to(dtype))
+
+    def adapter(r):
+        return {
+            "blk.q_proj.lora_A": rnd(r, hidden), "blk.q_proj.lora_B": rnd(q, r),
+            "blk.k_proj.lora_A": rnd(r, hidden), "blk.k_proj.lora_B": rnd(kv, r),
+            "blk.v_proj.lora_A": rnd(r, hidden), "blk.v_proj.lora_B": rnd(kv, r),
+            "blk.o_proj.lora_A": rnd(r, q), "blk.o_proj.lora_B": rnd(hidden, r),
+            "blk.gate_proj.lora_A": rnd(r, hidden), "blk.gate_proj.lora_B": rnd(inter, r),
+            "blk.up_proj.lora_A": rnd(r, hidden), "blk.up_proj.lora_B": rnd(inter, r),
+            "blk.down_proj.lora_A": rnd(r, inter), "blk.down_proj.lora_B": rnd(hidden, r),
+        }
+
+    T_ = 40
+    slots = torch.randint(-1, 3, (T_,), generator=g, dtype=torch.int32)
+    slots[:6] = 2
+    x_by_k = {hidden: torch.randn(T_, hidden, generator=g).to(dtype).cuda(), inter: torch.randn(T_, inter, generator=g).to(dtype).cuda()}
+    targets = {"qkv_proj": ["q", "k", "v"], "o_proj": ["o"], "gate_up_proj": ["gate", "up"], "down_proj": ["down"]}
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3)
+    loaded: dict = {}
+    for step, (r, alpha) in enumerate(((16, 32.0), (8, 4.0))):
+        tensors = adapter(r)
+        (tmp_path / f"a{step}").mkdir()
+        payload = load_voxcpm_lora_checkpoint(str(_write(tmp_path / f"a{step}", tensors, {"lora_config": {"r": r, "alpha": alpha}})))
+        assert payload.packed.is_pinned()  # one pinned buffer: a slot load is one host-to-device copy
+        install_lora_payload(model, 2, payload, loaded=loaded)
+        set_lora_context(LoRAContext(token_to_slot=slots.cuda(), no_lora_flag=False))
+        try:
+            for name, m in mods.items():
+                x = x_by_k[m.weight.size(1)]
+                with torch.no_grad():
+                    got = m(x)
+                    base = torch.nn.functional.linear(x, m.weight)  # the layer's own base product, rounded to its dtype
+                want = base.double().cpu()
+                rows = torch.nonzero(slots == 2).flatten()
+                col = 0
+                for t in targets[name]:
+                    a = tensors[f"blk.{t}_proj.lora_A"].to(dtype).double()
+                    b = (tensors[f"blk.{t}_proj.lora_B"] * (alpha / r)).to(dtype).double()  # alpha / r folded into B at install time
+                    want[rows, col : col + b.size(0)] += x.double().cpu()[rows] @ a.T @ b.T
+                    col += b.size(0)
+                assert torch.allclose(got.double().cpu(), want, **tol), f"{name} step {step}"
+                assert m._effective_lora_rank_values[2] == r and m.effective_lora_rank.tolist()[2] == r
+                # the slot holds exactly the adapter: rows / columns beyond its rank are zero
+                a_buf = m.lora_A.detach()
+                assert torch.count_nonzero(a_buf[..., 2, r:, :]) == 0
+        finally:
+            reset_lora_context()
