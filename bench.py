@@ -349,7 +349,7 @@ def run_backbone(args) -> None:
 
 
 KERNELS = {
-    "decode": "decode_kernel<bf16,16> (qkv, o, gate_up) + split_kernel<bf16,16> (down)",
+    "decode": "decode_kernel<bf16,16>",
     "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
     "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
 }

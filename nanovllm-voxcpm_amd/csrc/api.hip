@@ -84,7 +84,12 @@ struct ApiKnobs {
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
     force_form = env_int("MLORA_FORCE_FORM", 0);
     no_split = env_int("MLORA_NO_SPLIT", 0);
-    split_min_k = env_int("MLORA_SPLIT_MIN_K", 2048);
+    // Measured on the decode batch (32 tiles): at K = 4096 one workgroup per (tile, column range)
+    // takes 6.9 us per call, the split form 8.0 (what producers publish reaches the consumers 1.6 us
+    // later, two trips through the memory system; that is more than spreading the shrink saves), at
+    // K = 1024 4.2-7.4 against 6.9-11.5.  From K = 8192 on a workgroup's K range no longer fits its
+    // registers in one batch of loads, and the split form takes over.
+    split_min_k = env_int("MLORA_SPLIT_MIN_K", 8192);
   }
 };
 const ApiKnobs& knobs() {
@@ -168,8 +173,8 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     else if (small_tiles) form = MLORA_FORM_SPLIT;
     else form = MLORA_FORM_BGMV;
   }
-  // the split form where it pays (long K: the shrink of a tile is worth sharing) and shape and
-  // workspace allow it, else one workgroup per (tile, column range)
+  // the split form where it pays (very long K) and shape and workspace allow it, else one
+  // workgroup per (tile, column range)
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
       (knobs().no_split || !split_supported(a) || (a->k < knobs().split_min_k && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;

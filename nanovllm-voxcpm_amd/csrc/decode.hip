@@ -62,7 +62,7 @@ struct DecodeSplits {
 // row-contiguously (sixteen lanes per 256 bytes of a row) and turned into operand layout through
 // a private LDS block per wavefront, and the expand runs with the tokens as MFMA rows, so that
 // sixteen consecutive lanes cover 128 contiguous bytes of one y row.
-template <typename T, int R, int KSPW, bool TR>
+template <typename T, int R, int KSPW, bool TR, bool MASKED>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
   const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
   const DecodeSplit sp = splits.split[split_id];
-  const RankPrefetch ranks = rank_prefetch(eff_rank, num_slots, lane);
+  const RankPrefetch ranks = rank_prefetch(MASKED ? eff_rank : nullptr, num_slots, lane);
   const int slot = rec0[0], m = rec0[1];
   const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
   // One exit test, evaluated without short-circuit, that consumes everything fetched above
@@ -115,9 +115,11 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   MLORA_STAMP(1);  // tile record and plan header are here
 
   // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
-  const int eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
-  if (eff == 0) return;
-  const int rb_n = (eff + 15) >> 4;  // 16-rank blocks of A in use
+  // (MASKED = false is the instance for callers that gave no rank vector: eff is the constant R
+  // there and every test on it below folds away)
+  const int eff = MASKED ? rank_pick(ranks, eff_rank, num_slots, slot, R) : R;
+  if (MASKED && eff == 0) return;
+  const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
 
   const bool live = lr < m;  // this lane's token exists
   const T* xrow = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + lg * 8;
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           const int rr = rb * 16 + 4 * lg + i;
-          if (RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          if (!MASKED || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
           else ast[rb][4 * r + i] = i32x4{0, 0, 0, 0};
         }
       }
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         int n = c0 + 32 * h + (lane >> 1);
         n = n < sp.n1 ? n : sp.n1 - 1;
         bo[h][0].raw = load128(B + static_cast<int64_t>(n) * R + (lane & 1) * 8);
-        if (eff < R) mask_ranks(bo[h][0], (lane & 1) * 8, eff);
+        if (MASKED && eff < R) mask_ranks(bo[h][0], (lane & 1) * 8, eff);
       }
     } else {
 #pragma unroll
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-          if (eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
+          if (MASKED && eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
     }
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
             // zero, and an unconditional load keeps the whole batch of loads in flight together
             const int kc = (lg + 4 * ks) & (R / 8 - 1);
             bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-            if (eff < R) mask_ranks(bop[s][j][ks], kc * 8, eff);
+            if (MASKED && eff < R) mask_ranks(bop[s][j][ks], kc * 8, eff);
           }
         }
 #pragma unroll
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
     const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
     if (r < R) {
-      const float v = r < eff ? sum * scaling : 0.f;  // ranks the adapter does not have contribute nothing
+      const float v = (!MASKED || r < eff) ? sum * scaling : 0.f;  // ranks the adapter does not have contribute nothing
       const T hi = from_f32<T>(v);
       s_hi[tok * HSTRIDE + r] = hi;
       s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-          if (eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
+          if (MASKED && eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
 #pragma unroll
@@ -457,12 +459,19 @@ struct Launch {
   const DecodeSplits* splits;
 };
 
-template <typename T, int R, int KSPW, bool TR = false>
-void launch_one(const Launch& l) {
+template <typename T, int R, int KSPW, bool TR, bool MASKED>
+void launch_masked(const Launch& l) {
   const MloraAddArgs* a = l.a;
-  hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+  hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR, MASKED>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
                      a->num_slots, a->scaling, a->effective_rank, *l.splits);
+}
+
+// With a rank vector the instance that reads it; without, the one that has no such code at all.
+template <typename T, int R, int KSPW, bool TR = false>
+void launch_one(const Launch& l) {
+  if (l.a->effective_rank) launch_masked<T, R, KSPW, TR, true>(l);
+  else launch_masked<T, R, KSPW, TR, false>(l);
 }
 
 // The steps-per-wavefront specialisations kept: 1, 2 and 4 (K = 256, 512, 1024) for every rank

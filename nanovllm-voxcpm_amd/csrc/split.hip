@@ -76,11 +76,11 @@ __device__ __forceinline__ void xstore32(uint32_t* p, uint32_t v, int wide) {
 }
 
 // NWP: wavefronts of a producer that take part in the shrink; a K part is NWP * 128 columns.
-template <typename T, int R, int NWP>
+template <typename T, int R, int NWP, bool MASKED>
 __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv, void* __restrict__ yv_,
                                                     int64_t xs, int64_t ys, uint32_t* __restrict__ ws, int small_off, int T_, int K,
                                                     int num_slots, float scaling, int include_long, int S, int P, int W, int spin_ticks,
-                                                    int wide, int trusted, const int32_t* __restrict__ eff_rank, SplitSlices sl) {
+                                                    int wide, int trusted, int sym, const int32_t* __restrict__ eff_rank, SplitSlices sl) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
   const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
   const uint32_t signature = ws[0];
-  const RankPrefetch ranks = rank_prefetch(eff_rank, num_slots, lane);
+  const RankPrefetch ranks = rank_prefetch(MASKED ? eff_rank : nullptr, num_slots, lane);
   uint32_t* const tstate = ws + kWsTileOff / 4 + 2 * tile;  // {generation, arrivals}; tile < kWsTiles (host)
   const uint32_t tag = tstate[0] + 1u;
   const int slot = rec0[0], m = rec0[1];
@@ -123,16 +123,29 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   const bool xok = trusted | (signature == kWsMagic);  // the exchange area can be used
 
   // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
-  const int eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
-  if (eff == 0) return;  // nothing resident: the same for every workgroup of the tile
-  const int rb_n = (eff + 15) >> 4;  // 16-rank blocks of A in use
+  // (MASKED = false is the instance for callers that gave no rank vector: eff is the constant R
+  // there and every test on it below folds away)
+  const int eff = MASKED ? rank_pick(ranks, eff_rank, num_slots, slot, R) : R;
+  if (MASKED && eff == 0) return;  // nothing resident: the same for every workgroup of the tile
+  const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
 
+  // Roles.  Asymmetric launch: S * P producers (slice, K part), then the consumers (slice, column
+  // range of W columns).  Symmetric launch (sym, chosen for long K): S * P workgroups, each
+  // producer of its K part and consumer of the part-th column range of its slice, so that the
+  // shrink's operands AND the expand's are spread over all of them.
   const bool producer = role < S * P;
+  const bool consumer = sym || !producer;
   int slice, part = 0, n0 = 0, n1 = 0;
   if (producer) {
     slice = role / P;
     part = role - slice * P;
-    if (!xok) return;  // nobody would read what this workgroup publishes
+    if (sym) {
+      const int ws_cols = ((sl.n[slice] + P - 1) / P + 63) & ~63;  // columns per part, whole 64-column spans
+      n0 = part * ws_cols < sl.n[slice] ? part * ws_cols : sl.n[slice];
+      n1 = n0 + ws_cols < sl.n[slice] ? n0 + ws_cols : sl.n[slice];
+    } else if (!xok) {
+      return;  // nobody would read what this workgroup publishes
+    }
   } else {
     const int c = role - S * P;
     slice = 0;
@@ -218,26 +231,8 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
     }
   };
 
-  // ================================ producer ====================================================
-  if (producer) {
-    float tot[WPT];
-    shrink_part(part, tot);
-    MLORA_STAMP(2);  // producer: its K part is multiplied and summed over the wavefronts
-    u64* mine = xchg + part * WORDS;
-#pragma unroll
-    for (int j = 0; j < WPT; ++j) {
-      const int w = tid + j * kNT;
-      if ((WORDS % kNT == 0 || w < WORDS) && (w % R) < 16 * rb_n)
-        xstore(mine + w, (static_cast<u64>(tag) << 32) | __float_as_uint(tot[j]), wide);
-    }
-    MLORA_STAMP(3);  // producer: partial sums handed to the memory system
-    count_done();
-    MLORA_STAMP(15);  // role marker: producers leave slot 15 non-zero
-    return;
-  }
-
-  // ================================ consumer ====================================================
-  // ---- every load of the expand goes out first ----------------------------------------------------
+  // ================================ consumer part: loads =========================================
+  // ---- every load of the expand goes out first (before the shrink of a symmetric workgroup too) --
   const T* const Bs = static_cast<const T*>(sl.b[slice]) + static_cast<int64_t>(slot) * N * R;
   T* const ycols = static_cast<T*>(yv_) + sl.y_col[slice];
   const int eff8 = (eff + 7) >> 3;  // 8-rank chunks of a B row in use
@@ -288,6 +283,26 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   }
 
   MLORA_STAMP(4);  // consumer: every load of the expand is issued
+  // ================================ producer part ===============================================
+  if (producer && xok) {
+    float tot[WPT];
+    shrink_part(part, tot);
+    MLORA_STAMP(2);  // producer: its K part is multiplied and summed over the wavefronts
+    u64* mine = xchg + part * WORDS;
+#pragma unroll
+    for (int j = 0; j < WPT; ++j) {
+      const int w = tid + j * kNT;
+      if ((WORDS % kNT == 0 || w < WORDS) && (w % R) < 16 * rb_n)
+        xstore(mine + w, (static_cast<u64>(tag) << 32) | __float_as_uint(tot[j]), wide);
+    }
+    MLORA_STAMP(3);  // producer: partial sums handed to the memory system
+  }
+  if (!consumer || n0 >= n1) {  // nothing to expand here
+    if (xok) count_done();
+    MLORA_STAMP(15);  // role marker: pure producers leave slot 15 non-zero
+    return;
+  }
+
   // ---- the intermediate: from the producers, or computed here ---------------------------------------
   // lane l of wavefront 0 takes words l * WPL .. + WPL - 1 (token l / 4, ranks (l % 4) * WPL ..) of every part
   if (wave == 0) {
@@ -312,8 +327,9 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
         }
         ok = spin_ticks >= 0 && __builtin_amdgcn_ballot_w64(all) == ~0ull;
         if (ok || wall_clock64() - t0 >= spin_ticks) break;
-        __builtin_amdgcn_s_sleep(1);
+        if (!(wide & 32)) __builtin_amdgcn_s_sleep(1);
         if (wide & 8) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // drop what the L1 holds of the polled lines
+        if (wide & 16) asm volatile("buffer_inv sc0" ::: "memory");        // the same, this compute unit's L1 only
       }
       if (!ok && spin_ticks > 0 && lane == 0) atomicAdd(ws + kWsTimeoutsWord, 1u);  // diagnostic: a wait ran out
     }
@@ -463,16 +479,23 @@ __global__ __launch_bounds__(256) void workspace_init_kernel(uint32_t* ws) {
 struct SplitLaunch {
   const MloraAddArgs* a;
   dim3 grid;
-  int small_off, include_long, S, P, W, spin_ticks, wide, trusted;
+  int small_off, include_long, S, P, W, spin_ticks, wide, trusted, sym;
   SplitSlices sl;
 };
 
+template <typename T, int R, int NWP, bool MASKED>
+void launch_split_masked(const SplitLaunch& l) {
+  const MloraAddArgs* a = l.a;
+  hipLaunchKernelGGL((split_kernel<T, R, NWP, MASKED>), l.grid, dim3(kNT), 0, static_cast<hipStream_t>(a->stream), a->plan, a->x, a->y, a->x_stride,
+                     a->y_stride, static_cast<uint32_t*>(a->workspace), l.small_off, a->num_tokens, a->k, a->num_slots, a->scaling,
+                     l.include_long, l.S, l.P, l.W, l.spin_ticks, l.wide, l.trusted, l.sym, a->effective_rank, l.sl);
+}
+
+// With a rank vector the instance that reads it; without, the one that has no such code at all.
 template <typename T, int R, int NWP>
 void launch_split_one(const SplitLaunch& l) {
-  const MloraAddArgs* a = l.a;
-  hipLaunchKernelGGL((split_kernel<T, R, NWP>), l.grid, dim3(kNT), 0, static_cast<hipStream_t>(a->stream), a->plan, a->x, a->y, a->x_stride,
-                     a->y_stride, static_cast<uint32_t*>(a->workspace), l.small_off, a->num_tokens, a->k, a->num_slots, a->scaling,
-                     l.include_long, l.S, l.P, l.W, l.spin_ticks, l.wide, l.trusted, a->effective_rank, l.sl);
+  if (l.a->effective_rank) launch_split_masked<T, R, NWP, true>(l);
+  else launch_split_masked<T, R, NWP, false>(l);
 }
 
 template <typename T>
@@ -491,12 +514,16 @@ void launch_split_rank(const SplitLaunch& l, int nwp) {
 
 // Diagnostic knobs, read from the environment once per process.
 struct SplitKnobs {
-  int generation = -1, w, spin_ticks, wide, kpart;
+  int generation = -1, w, spin_ticks, wide, kpart, sym;
   void read() {
     generation = knob_generation();
     w = env_int("MLORA_SPLIT_W", 0);
     spin_ticks = env_int("MLORA_SPLIT_SPIN_TICKS", 20000);  // 200 us of the 100 MHz clock; negative: never accept published sums
-    wide = env_int("MLORA_SPLIT_WIDE", 7);
+    // loads and the arrival counts at device scope, stores in the L2 of the XCD on which every
+    // workgroup of a tile runs: were a tile ever spread over XCDs, its consumers would not see the
+    // stores, give up waiting and compute for themselves, and the generations would still advance
+    wide = env_int("MLORA_SPLIT_WIDE", 5);
+    sym = env_int("MLORA_SPLIT_SYM", -1);    // -1: symmetric roles when a tile's shrink has four or more K parts
     kpart = env_int("MLORA_SPLIT_KPART", 0);
   }
 };
@@ -589,8 +616,9 @@ int launch_split(const MloraAddArgs* a, bool include_long, bool trusted_workspac
   }
   l.sl.cons0[MLORA_MAX_SLICES] = consumers;
   l.W = w;
+  l.sym = knobs.sym >= 0 ? (knobs.sym ? 1 : 0) : (l.P >= 4 ? 1 : 0);
   // producers first: they are dispatched before the consumers that wait for them
-  l.grid = dim3(8, static_cast<unsigned>(l.S * l.P + consumers), static_cast<unsigned>(cap / 8));
+  l.grid = dim3(8, static_cast<unsigned>(l.sym ? l.S * l.P : l.S * l.P + consumers), static_cast<unsigned>(cap / 8));
   if (a->dtype == MLORA_DTYPE_BF16) launch_split_rank<__bf16>(l, nwp);
   else launch_split_rank<_Float16>(l, nwp);
   return check_launch("mlora_add_lora(small tiles, producers and consumers)");

@@ -145,22 +145,24 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
-@pytest.mark.parametrize("wide", [7, 8])
+@pytest.mark.parametrize("sym", [0, 1])
+@pytest.mark.parametrize("wide", [5, 7])
 @pytest.mark.parametrize("kpart", [512, 1024])
 @pytest.mark.parametrize("name,rank", [("down", 16), ("down", 64), ("qkv", 16), ("gate_up", 8), ("o", 32)])
-def test_split_form_producers_and_consumers(name, rank, kpart, wide, monkeypatch):
+def test_split_form_producers_and_consumers(name, rank, kpart, wide, sym, monkeypatch):
     """Small-tile form with the two products in different workgroups of one launch: producers
     publish the partial sums of their K part in the workspace, consumers pick them up (bounded
-    wait) and expand their column range; a consumer whose wait runs out computes the sums itself.
-    Checked: parity for both K-part widths and both access scopes, bit-identical results from one
+    wait) and expand their column range (sym: every workgroup is producer of a K part and consumer of
+    a column range); a consumer whose wait runs out computes the sums itself.
+    Checked: parity for both K-part widths, both role layouts and both access scopes, bit-identical results from one
     launch to the next and between accepting published sums, never accepting them and not waiting
     at all (the order of every sum is fixed, whatever the timing), slot -1 rows untouched, no wait
     running out in the ordinary runs, every tile's arrival count back at zero after each launch,
     and the same result from a workspace that was never initialised."""
     from nanovllm_voxcpm_amd import _hip, synthetic
 
-    print(f"split form {name} r={rank} kpart={kpart} wide={wide}", flush=True)
-    _knobs(monkeypatch, MLORA_SPLIT_KPART=kpart, MLORA_SPLIT_WIDE=wide, MLORA_SPLIT_W=128 if name == "qkv" else None)
+    print(f"split form {name} r={rank} kpart={kpart} wide={wide} sym={sym}", flush=True)
+    _knobs(monkeypatch, MLORA_SPLIT_KPART=kpart, MLORA_SPLIT_WIDE=wide, MLORA_SPLIT_SYM=sym, MLORA_SPLIT_W=128 if name == "qkv" else None)
     proj = _make(name, 12, rank, torch.bfloat16, seed=130 + rank)
     T = 90
     x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=131, device="cuda")
@@ -368,6 +370,26 @@ def test_auto_form_follows_rank_and_width(rank, expected):
     exact, mag = _exact(proj, x, y0, slots)
     _check(got, y0, exact, mag, slots, f"auto/r{rank}")
     assert torch.equal(got, _apply(expected, proj, x, y0.clone(), slots))
+
+
+@pytest.mark.parametrize("rank", [16, 32])
+def test_auto_takes_the_split_form_for_very_long_k(rank):
+    """K = 8192 (a model eight times as wide): a workgroup's K range no longer fits its registers as
+    one batch of loads, so AUTO lets the workgroups of a tile share the shrink.  Parity, and the
+    same bits as the form it is meant to pick."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"auto split r={rank}", flush=True)
+    shapes = {"wide_down": (8192, [1024, 264])}
+    proj = synthetic.make_projection("wide_down", 6, rank, torch.bfloat16, seed=340 + rank, device="cuda", shapes=shapes)
+    x, y0 = synthetic.make_activations(70, proj.k, sum(proj.widths), torch.bfloat16, seed=341, device="cuda")
+    g = torch.Generator().manual_seed(342)
+    slots = torch.randint(-1, 6, (70,), generator=g, dtype=torch.int32).cuda()
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"auto-split/r{rank}")
+    assert torch.equal(got, _apply("split", proj, x, y0.clone(), slots))
+    assert torch.allclose(got.float(), _apply("mfma", proj, x, y0.clone(), slots).float(), rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("seed", list(range(32)))
