@@ -272,8 +272,10 @@ def run_timeline(args) -> None:
     t0 = int(t[t[:, 0] != 0][:, 0].min())
     out = {"timeline_of": args.timeline, "form": args.form, "workgroups_launched": int((t[:, 0] != 0).sum()),
            "workgroups_with_work": int(rows.size(0)), "unit": "ns after the first workgroup entered", "kernels": {}}
-    groups = {"decode_kernel": rows[rows[:, 15] == 0]} if int((rows[:, 15] != 0).sum()) == 0 else {
-        "split_kernel producer": rows[rows[:, 15] != 0], "split_kernel consumer": rows[rows[:, 15] == 0]}
+    if int((rows[:, 15] != 0).sum()) == 0:
+        groups = {"decode_kernel": rows}
+    else:
+        groups = {"split_kernel producer": rows[rows[:, 15] != 0], "split_kernel consumer": rows[rows[:, 15] == 0]}
     for name, g in groups.items():
         entry = {}
         for i, label in enumerate(STAMPS[name]):

@@ -202,10 +202,19 @@ static_assert(kWsXchgOff + kWsXchgBytes == MLORA_WORKSPACE_HEAD_BYTES, "head siz
     if (threadIdx.x == 0 && trace_buf)                                                                       \
       trace_buf[(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 16ull + (i)] = wall_clock64(); \
   } while (0)
+// the same by thread `t` of the workgroup
+#define MLORA_STAMP_AT(i, t)                                                                                 \
+  do {                                                                                                       \
+    if (threadIdx.x == (t) && trace_buf)                                                                     \
+      trace_buf[(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * 16ull + (i)] = wall_clock64(); \
+  } while (0)
 #else
 #define MLORA_TRACE_DECL
 #define MLORA_STAMP(i) \
   do {                 \
+  } while (0)
+#define MLORA_STAMP_AT(i, t) \
+  do {                       \
   } while (0)
 #endif
 
