@@ -482,6 +482,35 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
     return result, (layers, slots, rank, step)
 
 
+def measure_unfused(layers, slots, name: str = "qkv") -> dict:
+    """The two-call form (lora_shrink into an fp32 intermediate, then lora_expand with add_inputs)
+    on one projection of the decode workload, beside the fused call on the same buffers: a graph
+    of the 24 layers' calls each, microseconds per projection call."""
+    import torch
+
+    from nanovllm_voxcpm_amd.lora_ops import lora_expand, lora_shrink
+
+    proj0 = layers[0][name][0]
+    n_slices, rank = len(proj0.widths), proj0.a[0].size(1)
+    h = torch.zeros((n_slices, slots.numel(), rank), dtype=torch.float32, device=slots.device)
+
+    def two_calls():
+        for entry in layers:
+            proj, x, y = entry[name]
+            lora_shrink(x, list(proj.a), h, slots, None, None, None, None, False, 0, 1.0)
+            lora_expand(h, list(proj.b), y, slots, None, None, None, None, False, 0, offset_start=0, add_inputs=True)
+
+    fused, calls = make_step(layers, slots, "auto", only=name)
+    out = {}
+    for key, fn in (("us_per_call_shrink_then_expand", two_calls), ("us_per_call_fused", fused)):
+        graph = capture(fn)
+        for _ in range(3):
+            graph.replay()
+        out[key] = round(time_region(graph.replay, 20) * 1e3 / calls, 2)
+    out["projection"] = name
+    return out
+
+
 def measure_floor(device: str, step_bytes: int, calls: int) -> dict:
     """What bounds a step of `calls` dependent launches on this machine, measured in this run:
     a replayed graph of as many kernels that do nothing (one wavefront each, then the grid of a
@@ -641,6 +670,7 @@ def main() -> None:
             extra[name]["unit"] = "GB/s"
             torch.cuda.empty_cache()
         extra["backbone"] = measure_backbone(10, 3)
+        extra["unfused_ops"] = measure_unfused(layers, slots)
         torch.cuda.empty_cache()
         out["extra"] = extra
     if not args.no_cpu_baseline and args.workload == "decode":

@@ -95,6 +95,37 @@ __global__ __launch_bounds__(kTokThreads) void token_shrink_kernel(TokenShrinkPa
   }
 }
 
+// The same shrink with 128-bit loads and packed dot products: a wavefront per rank row, each
+// lane eight consecutive elements of K at a time, then a 64-lane sum.  For 16-bit elements, K a
+// multiple of eight and 16-byte aligned rows (what the reference's tiled kernel,
+// lora_ops/triton_ops/lora_shrink_op.py:16-101, covers with its BLOCK_K loads).
+template <typename T, typename O>
+__global__ __launch_bounds__(kTokThreads) void token_shrink_vec_kernel(TokenShrinkParams p) {
+  const int t = blockIdx.x, i = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  O* out = static_cast<O*>(p.out) + (static_cast<int64_t>(i) * p.T + t) * p.r;
+  const int s = p.tts[t];
+  if (s < 0 || s >= p.num_slots) {
+    for (int j = tid; j < p.r; j += kTokThreads) out[j] = from_f32<O>(0.f);
+    return;
+  }
+  const T* x = static_cast<const T*>(p.x) + static_cast<int64_t>(t) * p.xs;
+  const T* A = static_cast<const T*>(p.a[i]) + static_cast<int64_t>(s) * p.r * p.K;
+  const int chunks = p.K / 8;
+  for (int j = wave; j < p.r; j += kTokWaves) {
+    const T* a = A + static_cast<int64_t>(j) * p.K;
+    float acc = 0.f;
+    for (int c = lane; c < chunks; c += kWave) {
+      Pack8 xv, av;
+      xv.raw = load128(x + c * 8);
+      av.raw = load128(a + c * 8);
+      acc = dot8<T>(xv, av, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) out[j] = from_f32<O>(acc * p.scaling);
+  }
+}
+
 struct TokenExpandParams {
   const void* h; void* y;
   int64_t ys;
@@ -128,6 +159,42 @@ __global__ __launch_bounds__(kTokThreads) void token_expand_kernel(TokenExpandPa
     const T* b = B + static_cast<int64_t>(n) * p.r;
     float acc = 0.f;
     for (int j = 0; j < p.r; ++j) acc += h[j] * to_f32(b[j]);
+    const T v = from_f32<T>(acc);
+    y[n] = p.add_inputs ? from_f32<T>(to_f32(y[n]) + to_f32(v)) : v;
+  }
+}
+
+// The same expand with 128-bit loads of the B rows: a thread per output column reads its row of r
+// elements eight at a time (r a multiple of eight, 16-bit elements, 16-byte aligned rows); the
+// roundings are those of the scalar kernel.
+template <typename T, typename H>
+__global__ __launch_bounds__(kTokThreads) void token_expand_vec_kernel(TokenExpandParams p) {
+  __shared__ float h[MLORA_MAX_RANK];
+  const int t = blockIdx.x, i = blockIdx.z;
+  const int s = p.tts[t];
+  if (s < 0 || s >= p.num_slots) return;
+  const int N = p.n[i];
+  const int chunk = (N + p.nsplit - 1) / p.nsplit;
+  const int n0 = blockIdx.y * chunk;
+  const int n1 = n0 + chunk < N ? n0 + chunk : N;
+  if (n0 >= n1) return;
+  const int tid = threadIdx.x;
+  const H* hin = static_cast<const H*>(p.h) + (static_cast<int64_t>(i) * p.T + t) * p.r;
+  for (int j = tid; j < p.r; j += kTokThreads) h[j] = to_f32(from_f32<T>(to_f32(hin[j])));
+  __syncthreads();
+  const T* B = static_cast<const T*>(p.b[i]) + static_cast<int64_t>(s) * N * p.r;
+  T* y = static_cast<T*>(p.y) + static_cast<int64_t>(t) * p.ys + p.col[i];
+  for (int n = n0 + tid; n < n1; n += kTokThreads) {
+    const T* b = B + static_cast<int64_t>(n) * p.r;
+    float acc = 0.f;
+    for (int j = 0; j < p.r; j += 8) {
+      Pack8 bv;
+      bv.raw = load128(b + j);
+      float f[8];
+      unpack8<T>(bv, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += h[j + e] * f[e];
+    }
     const T v = from_f32<T>(acc);
     y[n] = p.add_inputs ? from_f32<T>(to_f32(y[n]) + to_f32(v)) : v;
   }
@@ -207,6 +274,26 @@ void launch_shrink_out(const TokenShrinkParams& p, dim3 grid, int out_dtype, hip
 }
 
 template <typename T>
+void launch_shrink_vec_out(const TokenShrinkParams& p, dim3 grid, int out_dtype, hipStream_t st) {
+  switch (out_dtype) {
+    case MLORA_DTYPE_F32: hipLaunchKernelGGL((token_shrink_vec_kernel<T, float>), grid, dim3(kTokThreads), 0, st, p); break;
+    case MLORA_DTYPE_F16: hipLaunchKernelGGL((token_shrink_vec_kernel<T, _Float16>), grid, dim3(kTokThreads), 0, st, p); break;
+    default: hipLaunchKernelGGL((token_shrink_vec_kernel<T, __bf16>), grid, dim3(kTokThreads), 0, st, p); break;
+  }
+}
+
+template <typename T>
+void launch_expand_vec_h(const TokenExpandParams& p, dim3 grid, int h_dtype, hipStream_t st) {
+  switch (h_dtype) {
+    case MLORA_DTYPE_F32: hipLaunchKernelGGL((token_expand_vec_kernel<T, float>), grid, dim3(kTokThreads), 0, st, p); break;
+    case MLORA_DTYPE_F16: hipLaunchKernelGGL((token_expand_vec_kernel<T, _Float16>), grid, dim3(kTokThreads), 0, st, p); break;
+    default: hipLaunchKernelGGL((token_expand_vec_kernel<T, __bf16>), grid, dim3(kTokThreads), 0, st, p); break;
+  }
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+template <typename T>
 void launch_expand_h(const TokenExpandParams& p, dim3 grid, int h_dtype, hipStream_t st) {
   switch (h_dtype) {
     case MLORA_DTYPE_F32: hipLaunchKernelGGL((token_expand_kernel<T, float>), grid, dim3(kTokThreads), 0, st, p); break;
@@ -244,10 +331,12 @@ extern "C" int mlora_shrink(const MloraShrinkArgs* a) {
   }
   dim3 grid(a->num_tokens, a->num_slices);
   hipStream_t st = static_cast<hipStream_t>(a->stream);
+  bool vec = a->dtype != MLORA_DTYPE_F32 && a->k % 8 == 0 && a->x_stride % 8 == 0 && aligned16(a->x);
+  for (int i = 0; i < a->num_slices; ++i) vec = vec && aligned16(a->a[i]);
   switch (a->dtype) {
     case MLORA_DTYPE_F32: launch_shrink_out<float>(p, grid, a->out_dtype, st); break;
-    case MLORA_DTYPE_F16: launch_shrink_out<_Float16>(p, grid, a->out_dtype, st); break;
-    default: launch_shrink_out<__bf16>(p, grid, a->out_dtype, st); break;
+    case MLORA_DTYPE_F16: vec ? launch_shrink_vec_out<_Float16>(p, grid, a->out_dtype, st) : launch_shrink_out<_Float16>(p, grid, a->out_dtype, st); break;
+    default: vec ? launch_shrink_vec_out<__bf16>(p, grid, a->out_dtype, st) : launch_shrink_out<__bf16>(p, grid, a->out_dtype, st); break;
   }
   return check_launch("mlora_shrink");
 }
@@ -275,10 +364,12 @@ extern "C" int mlora_expand(const MloraExpandArgs* a) {
   p.nsplit = column_splits(n_max);
   dim3 grid(a->num_tokens, p.nsplit, a->num_slices);
   hipStream_t st = static_cast<hipStream_t>(a->stream);
+  bool vec = a->dtype != MLORA_DTYPE_F32 && a->r % 8 == 0;
+  for (int i = 0; i < a->num_slices; ++i) vec = vec && aligned16(a->b[i]);
   switch (a->dtype) {
     case MLORA_DTYPE_F32: launch_expand_h<float>(p, grid, a->h_dtype, st); break;
-    case MLORA_DTYPE_F16: launch_expand_h<_Float16>(p, grid, a->h_dtype, st); break;
-    default: launch_expand_h<__bf16>(p, grid, a->h_dtype, st); break;
+    case MLORA_DTYPE_F16: vec ? launch_expand_vec_h<_Float16>(p, grid, a->h_dtype, st) : launch_expand_h<_Float16>(p, grid, a->h_dtype, st); break;
+    default: vec ? launch_expand_vec_h<__bf16>(p, grid, a->h_dtype, st) : launch_expand_h<__bf16>(p, grid, a->h_dtype, st); break;
   }
   return check_launch("mlora_expand");
 }

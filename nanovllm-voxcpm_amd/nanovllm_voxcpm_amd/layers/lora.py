@@ -185,13 +185,16 @@ class _LoRALayerBase(nn.Module):
     def _wants_rank_masking(self) -> bool:
         """Whether the backend should be told the per-slot ranks: only buffers of more than one
         16-rank block can skip anything, and only when some resident adapter is below the padded
-        rank — or while a graph is captured, whose launches must serve adapters installed later.
-        Decided from the host mirror only."""
+        rank.  A graph captured while nothing is resident must serve whatever is installed later,
+        so it takes the rank-aware kernels; one captured over adapters that all fill the padded
+        rank takes the plain kernels, which stay correct for later installs because an install
+        zero-fills the ranks it does not use.  Decided from the host mirror only."""
         if self.max_lora_rank <= 16:
             return False
-        if _is_cuda_graph_capture():
+        resident = [rank for rank in self._effective_lora_rank_values if rank > 0]
+        if _is_cuda_graph_capture() and not resident:
             return True
-        return any(0 < rank < self.max_lora_rank for rank in self._effective_lora_rank_values)
+        return any(rank < self.max_lora_rank for rank in resident)
 
     def prime_lora_cache(self) -> None:
         if not self.supports_lora:

@@ -416,3 +416,19 @@ def test_rank_masking_is_requested_only_when_it_can_pay():
     assert wide._wants_rank_masking() is False  # only full-rank adapters
     wide.set_slot_lora(1, torch.ones(8, 8), torch.ones(4, 8), effective_rank=8, scaling=1.0)
     assert wide._wants_rank_masking() is True
+
+
+def test_rank_masking_under_graph_capture(monkeypatch):
+    """A graph captured with nothing resident gets the rank-aware kernels (it must serve what is
+    installed later); one captured over full-rank adapters gets the plain ones."""
+    from nanovllm_voxcpm_amd.layers import lora as lora_layers
+
+    monkeypatch.setattr(lora_layers, "_is_cuda_graph_capture", lambda: True)
+    wide = lora_layers.LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=64)
+    assert wide._wants_rank_masking() is True
+    wide.set_slot_lora(0, torch.ones(64, 8), torch.ones(4, 64), effective_rank=64, scaling=1.0)
+    assert wide._wants_rank_masking() is False
+    wide.set_slot_lora(1, torch.ones(8, 8), torch.ones(4, 8), effective_rank=8, scaling=1.0)
+    assert wide._wants_rank_masking() is True
+    narrow = lora_layers.LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=16)
+    assert narrow._wants_rank_masking() is False
