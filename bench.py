@@ -258,6 +258,8 @@ def run_timeline(args) -> None:
 
     device = "cuda:0"
     layers, slots, _ = build_workload("decode", device, args.rank or None)
+    if args.hot_layers > 0:
+        layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
     step, launches = make_step(layers, slots, args.form, args.timeline)
     for _ in range(3):
         step()
