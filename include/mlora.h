@@ -43,6 +43,9 @@ extern "C" {
 #define MLORA_FORM_SPLIT 5 /* small tiles, one launch: producer workgroups compute the rank-r intermediate of a
                               (tile, slice, K part) and publish it in the workspace, consumer workgroups take a
                               column range each, pick the intermediate up and expand; needs an initialised workspace */
+#define MLORA_FORM_FUSED 6 /* the tiles of MLORA_FORM_SGMV in one launch: the workgroups of a group of tiles share
+                              out its shrink, seal what they wrote to the workspace, wait for each other's seals
+                              and expand a column range each; needs an initialised workspace */
 
 /* error codes (negative) */
 #define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
@@ -276,8 +279,10 @@ void mlora_reload_knobs(void);
 /* Launches of known cost (measurement aid, no counterpart in the reference): kind 0 enqueues a
  * kernel that does nothing with the given grid and workgroup size (what a launch costs by itself);
  * kind 1 a read-modify-write stream over `bytes` of 16-bit elements at `buf` (every element read,
- * incremented, written back once: the access pattern of y); kind 2 a read-only stream over them.
- * bench.py quotes them beside the real kernels. */
+ * incremented, written back once: the access pattern of y); kind 2 a read-only stream over them;
+ * kind 3 a kernel of the given grid whose workgroups each write the number of the XCD they run on
+ * to `buf` (int32 per workgroup, linear workgroup order: the placement the kernels' grids of x
+ * extent 8 rely on can be checked).  bench.py quotes kinds 0-2 beside the real kernels. */
 int mlora_probe_launch(void* stream, int32_t kind, void* buf, int64_t bytes, int32_t grid_x, int32_t grid_y, int32_t grid_z,
                        int32_t threads);
 

@@ -78,12 +78,18 @@ namespace {
 
 // Diagnostic knobs, read from the environment once per process.
 struct ApiKnobs {
-  int generation = -1, small_batch_tokens, force_form, no_split, split_min_k;
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_k, auto_fused;
   void read() {
     generation = knob_generation();
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
     force_form = env_int("MLORA_FORCE_FORM", 0);
     no_split = env_int("MLORA_NO_SPLIT", 0);
+    // Measured on the prefill batch (7605 tokens, rank 64) and the mixed one: the one-launch
+    // long-segment form takes 4214 us per step against 3858 for two launches (mixed: 6496 against
+    // 5467).  Its workgroups are all resident at once, so the whole grid first shrinks (a chain of
+    // dependent slab fetches per workgroup, HBM nearly idle) and then expands; the saved launch
+    // does not pay for the wait on the slowest role of each unit.  AUTO keeps the two launches.
+    auto_fused = env_int("MLORA_AUTO_FUSED", 0);
     // Measured on the decode batch (32 tiles): at K = 4096 one workgroup per (tile, column range)
     // takes 6.9 us per call, the split form 8.0 (what producers publish reaches the consumers 1.6 us
     // later, two trips through the memory system; that is more than spreading the shrink saves), at
@@ -135,7 +141,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (a->dtype != MLORA_DTYPE_F32 && a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) {
     set_error("mlora_add_lora: unknown dtype %d", a->dtype); return MLORA_E_INVALID;
   }
-  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_SPLIT) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
+  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_FUSED) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
   if (a->num_slices > MLORA_MAX_SLICES) { set_error("mlora_add_lora: %d slices exceed %d", a->num_slices, MLORA_MAX_SLICES); return MLORA_E_TOO_LARGE; }
   if (a->r > MLORA_MAX_RANK) { set_error("mlora_add_lora: rank %d exceeds %d", a->r, MLORA_MAX_RANK); return MLORA_E_TOO_LARGE; }
   if (a->num_slots > MLORA_MAX_SLOTS) { set_error("mlora_add_lora: %d slots exceed %d", a->num_slots, MLORA_MAX_SLOTS); return MLORA_E_TOO_LARGE; }
@@ -161,7 +167,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   const bool vec = vector_ok(a);
   if (form == MLORA_FORM_AUTO) {
     const int forced = knobs().force_form;
-    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_SPLIT && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
+    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_FUSED && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
   }
   if (form == MLORA_FORM_AUTO) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
@@ -178,6 +184,9 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
       (knobs().no_split || !split_supported(a) || (a->k < knobs().split_min_k && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;
+  // long-segment batches in one launch, on request
+  if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))
+    form = MLORA_FORM_FUSED;
   switch (form) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
@@ -187,6 +196,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
       if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
       return launch_bgmv(a, /*include_long=*/true);
     case MLORA_FORM_SGMV:
+    case MLORA_FORM_FUSED:
     case MLORA_FORM_SPLIT:
     case MLORA_FORM_MFMA: {
       if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
@@ -204,6 +214,14 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
         set_error("mlora_add_lora: SGMV form needs a 16-byte aligned workspace of %zu bytes and no empty slice",
                   sgmv_workspace_bytes(a->num_tokens, a->num_slices, a->r, a->dtype));
         return MLORA_E_INVALID;
+      }
+      if (form == MLORA_FORM_FUSED) {
+        if (!fused_supported(a)) {
+          set_error("mlora_add_lora: the one-launch long-segment form needs K %% 256 == 0, at most %d groups of tiles and a workspace "
+                    "whose head holds their seals", kWsTiles);
+          return MLORA_E_UNSUPPORTED;
+        }
+        return launch_fused(a, trusted_workspace);
       }
       return launch_sgmv(a);
     }
@@ -296,6 +314,7 @@ extern "C" int mlora_trace_set(void* buf) {
 #ifdef MLORA_TRACE
   decode_trace_set(buf);
   split_trace_set(buf);
+  fused_trace_set(buf);
   return 0;
 #else
   (void)buf;

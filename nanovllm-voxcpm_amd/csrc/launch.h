@@ -38,8 +38,14 @@ bool sgmv_workspace_ok(const MloraAddArgs* a);
 size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype);
 int launch_sgmv(const MloraAddArgs* a);
 
+// fused.hip: the same tiles, shrink and expand in one launch (workgroups of a unit exchange the
+// intermediate through the workspace under seals kept in its head).
+bool fused_supported(const MloraAddArgs* a);
+int launch_fused(const MloraAddArgs* a, bool trusted_workspace);
+
 // in-kernel timeline of trace builds (no-ops otherwise)
 void decode_trace_set(void* buf);
 void split_trace_set(void* buf);
+void fused_trace_set(void* buf);
 
 }  // namespace mlora

@@ -39,6 +39,13 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const i32x4* __restrict
   if (acc == 0x5a5a5a5a && sink) *sink = acc;
 }
 
+// kind 3: every workgroup of a (grid_x, grid_y, grid_z) grid records the XCD it runs on (one int32
+// per workgroup, in linear workgroup order): what the kernels assume about grids whose x extent
+// is 8 (blockIdx.x names the XCD) can be checked on the machine at hand.
+__global__ void probe_xcd_kernel(int32_t* __restrict__ out) {
+  if (threadIdx.x == 0) out[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = static_cast<int32_t>(xcc_id());
+}
+
 }  // namespace
 
 }  // namespace mlora
@@ -52,6 +59,12 @@ extern "C" int mlora_probe_launch(void* stream, int32_t kind, void* buf, int64_t
     if (grid_x < 1 || grid_y < 1 || grid_z < 1 || threads < 1 || threads > 1024) { set_error("mlora_probe_launch: bad launch shape"); return MLORA_E_INVALID; }
     hipLaunchKernelGGL(probe_empty_kernel, dim3(grid_x, grid_y, grid_z), dim3(threads), 0, st);
     return check_launch("mlora_probe_launch(empty)");
+  }
+  if (kind == 3) {
+    if (grid_x < 1 || grid_y < 1 || grid_z < 1 || threads < 1 || threads > 1024) { set_error("mlora_probe_launch: bad launch shape"); return MLORA_E_INVALID; }
+    if (!buf || bytes < static_cast<int64_t>(grid_x) * grid_y * grid_z * 4) { set_error("mlora_probe_launch: one int32 per workgroup is needed"); return MLORA_E_INVALID; }
+    hipLaunchKernelGGL(probe_xcd_kernel, dim3(grid_x, grid_y, grid_z), dim3(threads), 0, st, static_cast<int32_t*>(buf));
+    return check_launch("mlora_probe_launch(xcd)");
   }
   if (kind != 1 && kind != 2) { set_error("mlora_probe_launch: unknown kind %d", kind); return MLORA_E_INVALID; }
   if (!buf || bytes < 16 || (reinterpret_cast<uintptr_t>(buf) & 15)) { set_error("mlora_probe_launch: a 16-byte aligned buffer is needed"); return MLORA_E_INVALID; }

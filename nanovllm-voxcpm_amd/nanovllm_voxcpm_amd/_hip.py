@@ -22,8 +22,9 @@ MAX_SLOTS = 1024
 MAX_RANK = 256
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
-FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT = 0, 1, 2, 3, 4, 5
-FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA, "split": FORM_SPLIT}
+FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT, FORM_FUSED = 0, 1, 2, 3, 4, 5, 6
+FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA, "split": FORM_SPLIT,
+         "fused": FORM_FUSED}
 
 PLAN_HEADER_WORDS = 16
 (
@@ -568,7 +569,9 @@ def reload_knobs() -> None:
 def probe_launch(kind: int, buf: torch.Tensor | None = None, grid: tuple[int, int, int] = (1, 1, 1), threads: int = 64,
                  device: torch.device | None = None) -> None:
     """Enqueue a launch of known cost on torch's current stream: kind 0 an empty kernel of the given
-    shape, kind 1 a read-modify-write stream over ``buf``, kind 2 a read-only stream over it."""
+    shape, kind 1 a read-modify-write stream over ``buf``, kind 2 a read-only stream over it, kind 3
+    a kernel of the given shape whose workgroups each write the XCD they run on into ``buf`` (int32
+    per workgroup, linear workgroup order)."""
     dev = buf.device if buf is not None else (device or torch.device("cuda", torch.cuda.current_device()))
     nbytes = buf.numel() * buf.element_size() if buf is not None else 0
     with _on(dev):

@@ -352,6 +352,90 @@ def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
         assert torch.equal(y._base[:, :16], yw[:, :16]) and torch.equal(y._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
 
 
+def test_workgroups_of_one_blockidx_x_share_an_xcd():
+    """Grids of x extent 8: the kernels treat blockIdx.x as the XCD (column ranges of a tile share
+    an L2; workgroups that hand each other partial sums through it check the XCD they ran on).
+    Every workgroup records its XCD: one XCD per blockIdx.x, whatever y and z."""
+    from nanovllm_voxcpm_amd import _hip
+
+    grid = (8, 5, 37)
+    out = torch.full((grid[0] * grid[1] * grid[2],), -1, dtype=torch.int32, device="cuda")
+    _hip.probe_launch(3, out, grid=grid, threads=256)
+    torch.cuda.synchronize()
+    xcd = out.cpu().view(grid[2], grid[1], grid[0])
+    assert (xcd >= 0).all()
+    for bx in range(8):
+        assert xcd[:, :, bx].unique().numel() == 1, f"blockIdx.x = {bx} ran on XCDs {xcd[:, :, bx].unique().tolist()}"
+    print("XCD of blockIdx.x 0..7:", [int(xcd[0, 0, bx]) for bx in range(8)], flush=True)
+
+
+@pytest.mark.parametrize("knobs", [{}, {"MLORA_SGMV_KSPLIT": "1", "MLORA_SGMV_GROUP": "4"}, {"MLORA_SGMV_KSPLIT": "4", "MLORA_SGMV_GROUP": "1", "MLORA_SGMV_NT": "512"},
+                                   {"MLORA_SGMV_ALL_SLICES": "2", "MLORA_SGMV_GROUP": "4", "MLORA_SGMV_NT": "512"}])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [8, 16, 32, 64])
+def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
+    """The one-launch form of the long-segment kernels: the workgroups of a group of tiles share
+    out its shrink, seal what they wrote, wait for each other's seals (bounded) and expand a column
+    range each.  Same batch as for the two-launch form (segments of 1..130 tokens, rows without
+    adapter, ragged widths, strided views).  Checked: parity; the bits of the two-launch form where
+    neither cuts K (same sums, same order); the same bits on a second launch, when no seal is ever accepted
+    (every workgroup computes what it needs itself) and on a workspace without the signature; no
+    wait running out in the ordinary runs; every unit's arrival count back at zero."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
+
+    print(f"one-launch long form r={rank} {dtype} {knobs}", flush=True)
+    for key, value in knobs.items():
+        monkeypatch.setenv(key, value)
+    _knobs(monkeypatch)
+    shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520]), "t": (768, [264]), "u": (1536, [136]), "v": (2048, [64])}
+    lengths = [130, 1, 64, 15, 16, 65, 3, 128, 17, 7]
+    slot_of = [2, 0, 5, 1, 3, -1, 4, 2, -1, 6]  # slot 2 twice: two segments merge into one of 258
+    slots = torch.cat([torch.full((n,), s, dtype=torch.int32) for n, s in zip(lengths, slot_of)])
+    slots = slots[torch.randperm(slots.numel(), generator=torch.Generator().manual_seed(9))].cuda()
+    T = slots.numel()
+    for name in shapes:
+        proj = synthetic.make_projection(name, 7, rank, dtype, seed=900 + rank, device="cuda", shapes=shapes)
+        xw, yw = synthetic.make_activations(T, proj.k + 24, sum(proj.widths) + 40, dtype, seed=901, device="cuda")
+        x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 16 : 16 + sum(proj.widths)]  # 16-byte aligned views of wider buffers
+        backend = _backend("fused")
+        meta = _metadata(slots)
+
+        def run():
+            y = yw.clone()[:, 16 : 16 + sum(proj.widths)]
+            blocks = list(y.split(proj.widths, dim=-1))
+            backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=meta, scaling=0.75, y_packed=y if len(blocks) > 1 else None)
+            return y
+
+        runs = []
+        for spin in (50000, 50000, -1):
+            _knobs(monkeypatch, MLORA_FUSED_SPIN_TICKS=spin)
+            runs.append(run())
+            if spin > 0:
+                assert _waits_run_out(backend) == 0, "a workgroup gave up waiting for its unit's seals"
+        got = runs[0]
+        exact, mag = _exact(proj, x, y0, slots, scaling=0.75)
+        _check(got, y0, exact, mag, slots, f"one-launch/{name}/r{rank}/{dtype}/{knobs}")
+        assert torch.equal(got._base[:, :16], yw[:, :16]) and torch.equal(got._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
+        for other in runs[1:]:
+            assert torch.equal(got, other)
+        two = _apply("sgmv", proj, x, yw.clone()[:, 16 : 16 + sum(proj.widths)], slots, scaling=0.75)
+        if knobs.get("MLORA_SGMV_KSPLIT") == "1":  # K uncut in both forms: the same sums in the same order
+            assert torch.equal(got, two)
+        else:
+            assert torch.allclose(got.float(), two.float(), rtol=RTOL, atol=ATOL)
+        (scratch,) = backend._scratch.values()
+        head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
+        state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} per unit
+        assert all(arrivals == 0 for _, arrivals in state)
+        assert any(generation > 0 for generation, _ in state)
+        # a workspace without the signature: nobody seals, nobody waits, same bits
+        scratch[:4].zero_()
+        _knobs(monkeypatch, MLORA_FUSED_SPIN_TICKS=50000)
+        assert torch.equal(run(), got)
+        assert _waits_run_out(backend) == 0
+        assert head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist() == state
+
+
 @pytest.mark.parametrize("rank,expected", [(16, "mfma"), (64, "sgmv")])
 def test_auto_form_follows_rank_and_width(rank, expected):
     """A 3000-token prefill of three sequences through the o projection: at rank 16 the one-launch
