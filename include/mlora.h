@@ -129,14 +129,15 @@ int mlora_add_lora_static(const MloraAddArgs* args);
 size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);
 
 /* A workspace starts with a head of MLORA_WORKSPACE_HEAD_BYTES bytes: a signature word, one
- * {generation, arrivals} pair per small tile and the area in which producer workgroups of
- * MLORA_FORM_SPLIT leave the intermediate for the consumers, every word tagged with its tile's
- * generation.  mlora_workspace_init enqueues one kernel that clears the head and writes the
+ * {generation, arrivals} pair per small tile (or group of 64-token tiles), the area in which
+ * producer workgroups of MLORA_FORM_SPLIT leave the intermediate for the consumers, every word
+ * tagged with its tile's generation, and the seals (generation and XCD of the writer) that the
+ * workgroups of MLORA_FORM_FUSED put on the partial sums they wrote.  mlora_workspace_init enqueues one kernel that clears the head and writes the
  * signature; call it once after allocation (it is a kernel, not a memset, so it may be recorded
  * into a graph).  Launches leave the head ready for the next launch.  A workspace whose head
  * does not carry the signature is still safe to pass: the kernels then compute every
  * intermediate locally and never read the exchange area.  No counterpart in the reference. */
-#define MLORA_WORKSPACE_HEAD_BYTES (16384 + (1 << 20))
+#define MLORA_WORKSPACE_HEAD_BYTES (16384 + (1 << 20) + (64 << 10))
 int mlora_workspace_init(void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0

@@ -188,12 +188,12 @@ constexpr int kWsTileOff = 256;
 constexpr int kWsTiles = 1024;
 constexpr int kWsXchgOff = 16384;
 constexpr int kWsXchgBytes = 1 << 20;
-// the last 64 KiB of the exchange area: one 64-bit seal per (unit, shrink role) of the one-launch
+// behind the exchange area: one 64-bit seal per (unit, shrink role) of the one-launch
 // long-segment form: {generation of the unit + 1, XCD of the writer}
 constexpr int kWsSealBytes = 64 << 10;
-constexpr int kWsSealOff = kWsXchgOff + kWsXchgBytes - kWsSealBytes;
+constexpr int kWsSealOff = kWsXchgOff + kWsXchgBytes;
 static_assert(kWsTileOff + 8 * kWsTiles <= kWsXchgOff, "tile state overlaps the exchange area");
-static_assert(kWsXchgOff + kWsXchgBytes == MLORA_WORKSPACE_HEAD_BYTES, "head size");
+static_assert(kWsSealOff + kWsSealBytes == MLORA_WORKSPACE_HEAD_BYTES, "head size");
 
 // The XCD (accelerator die) this wavefront runs on: bits 3:0 of hardware register XCC_ID (id 20).
 __device__ __forceinline__ uint32_t xcc_id() { return __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15u; }

@@ -553,7 +553,7 @@ static int pick_kpart(const MloraAddArgs* a, int wanted) {
   for (int kp : order) {
     if (kp != 512 && kp != 1024) continue;
     if (a->k % kp != 0 || a->k / kp > 8) continue;
-    if (static_cast<int64_t>(lay.cap_small) * a->num_slices * (a->k / kp) * 16 * a->r * 8 <= kWsXchgBytes - kWsSealBytes) return kp;
+    if (static_cast<int64_t>(lay.cap_small) * a->num_slices * (a->k / kp) * 16 * a->r * 8 <= kWsXchgBytes) return kp;
   }
   return 0;
 }
