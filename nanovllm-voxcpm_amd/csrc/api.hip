@@ -315,6 +315,7 @@ extern "C" int mlora_trace_set(void* buf) {
   decode_trace_set(buf);
   split_trace_set(buf);
   fused_trace_set(buf);
+  sgmv_trace_set(buf);
   return 0;
 #else
   (void)buf;

@@ -30,8 +30,6 @@ namespace mlora {
 namespace {
 
 constexpr int kFusedThreads = 256;
-
-MLORA_TRACE_DECL
 static_assert(kFusedThreads == kShrinkWaves * kWave && kFusedThreads == kExpandWaves * kWave, "both products run with four wavefronts");
 
 
@@ -181,11 +179,11 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
     fused_shrink_role<T, R, KR, XW, DB>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, gs, gstart,
                                         gm, ge);
   }
-  MLORA_STAMP(2);  // own role multiplied, its stores issued
+  MLORA_STAMP(10);  // own role multiplied, its stores issued
   // the partial sums written above have been acknowledged by the L2 ...
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  MLORA_STAMP(3);  // ... by every wavefront
+  MLORA_STAMP(11);  // ... by every wavefront
   // ... and only then is the role sealed
   if (xok && have_role && tid == 0) __hip_atomic_store(seals + c, seal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
@@ -210,7 +208,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
     }
   }
   __syncthreads();
-  MLORA_STAMP(4);  // the wait is over
+  MLORA_STAMP(12);  // the wait is over
   const uint64_t todo = (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(s_todo[1])) << 32) | static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(s_todo[0]));
   if (todo) {
     // seals that did not arrive (or a workspace whose head cannot be used): those roles are computed here
@@ -230,7 +228,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   // ---- expand ---------------------------------------------------------------------------------------
   fused_expand<T, R, CPL, TPF, G>(s_h, s_row, s_slot, s_m, s_eff, s_start, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt, sp);
 
-  MLORA_STAMP(5);  // expanded (wavefront 0)
+  MLORA_STAMP(13);  // expanded (wavefront 0)
   // ---- the last member of the unit to get here advances its generation ---------------------------------
   if (xok && tid == 0) {
     const uint32_t before = __hip_atomic_fetch_add(ustate + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -47,5 +47,6 @@ int launch_fused(const MloraAddArgs* a, bool trusted_workspace);
 void decode_trace_set(void* buf);
 void split_trace_set(void* buf);
 void fused_trace_set(void* buf);
+void sgmv_trace_set(void* buf);
 
 }  // namespace mlora

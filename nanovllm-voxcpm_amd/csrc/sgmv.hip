@@ -49,8 +49,10 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   // registers (its K part is a single batch then), instead of one workgroup per slice
   const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
   const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  MLORA_STAMP(0);  // first instruction
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
   if (!tr.ok) return;
+  MLORA_STAMP(1);  // tile record here
   // rank of the adapter in this slot (a second, dependent fetch, only with the vector given)
   int eff = R;
   if (R > 16 && eff_rank) {
@@ -64,6 +66,11 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   else
     shrink_body<T, R, KR, XW, DB, false>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart,
                                          tr.slot, tr.start, tr.m, eff);
+#ifdef MLORA_TRACE
+  MLORA_STAMP(6);  // partial sums issued
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  MLORA_STAMP(7);  // ... and acknowledged
+#endif
 }
 
 template <typename T, int R, int CPL, int TPF, int G>
@@ -205,6 +212,14 @@ size_t sgmv_workspace_bytes(int num_tokens, int num_slices, int r, int dtype) {
   (void)dtype;
   if (num_tokens <= 0 || num_slices <= 0 || r <= 0) return 0;
   return MLORA_WORKSPACE_HEAD_BYTES + kMaxKSplit * partial_bytes(num_tokens, num_slices, r);
+}
+
+void sgmv_trace_set(void* buf) {
+#ifdef MLORA_TRACE
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(trace_buf), &buf, sizeof(buf));
+#else
+  (void)buf;
+#endif
 }
 
 bool sgmv_supported(const MloraAddArgs* a) { return a->k % 128 == 0 && a->k >= 128; }

@@ -9,6 +9,8 @@ namespace mlora {
 
 namespace {
 
+MLORA_TRACE_DECL
+
 constexpr int kMaxSplits = 64;
 constexpr int kExpandWaves = 4;
 constexpr int kMaxKSplit = 4;  // most K parts the shrink ever uses (the workspace has room for them)
@@ -102,6 +104,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
   // MFMA harmlessly and are never written back)
   const int ti = wave * 16 + lr;
   const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
+  MLORA_STAMP(2);  // shrink: token rows requested
   const T* xptr = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + k0 + lg * 8;
   const int64_t aoff = static_cast<int64_t>(slot) * R * K + k0;
 
@@ -143,6 +146,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
       if (!first) __syncthreads();  // everyone is done reading the previous slab
       first = false;
       store_slab();
+      if (b == 0 && s == 0 && si == 0) MLORA_STAMP(4);  // shrink: first slab arrived and is on its way to LDS
       __syncthreads();
       // the slab after this one: same batch, next batch, or the first of the next slice
       if (s + 1 < SPB) request_slab(A + b * XW + (s + 1) * KR);
@@ -169,6 +173,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
 
   request_slab(static_cast<const T*>(sl.a[slice0]) + aoff);
   if (active) request_x(xa, 0);
+  MLORA_STAMP(3);  // shrink: first slab and first x batch requested (the token rows are here)
   for (int si = 0; si < nsl; ++si) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -180,6 +185,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
     } else {
       for (int b = 0; b < nbatch; ++b) run_batch(xa, xa, si, b);
     }
+    if (si == 0) MLORA_STAMP(5);  // shrink: first slice multiplied
     // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
     if (active && ti < m) {
       float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice0 + si) * R;
