@@ -460,6 +460,7 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
         "tflops": round(step_flops / (ms * 1e-3) / 1e12, 2),
         "pct_of_mfma_bf16_peak": round(100 * step_flops / (ms * 1e-3) / 1e12 / MFMA_BF16_TFLOPS, 3),
         "calls_per_step": calls,
+        "algorithmic_bytes_per_call_by_projection": per_proj,
         "us_per_call_by_projection": per_proj_us,
         "gbs_by_projection": {n: round(per_proj[n] / (per_proj_us[n] * 1e-6) / 1e9, 1) for n in per_proj_us},
         "roofline": {
