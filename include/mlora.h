@@ -137,7 +137,7 @@ size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t
  * into a graph).  Launches leave the head ready for the next launch.  A workspace whose head
  * does not carry the signature is still safe to pass: the kernels then compute every
  * intermediate locally and never read the exchange area.  No counterpart in the reference. */
-#define MLORA_WORKSPACE_HEAD_BYTES (16384 + (1 << 20) + (64 << 10))
+#define MLORA_WORKSPACE_HEAD_BYTES (16384 + (4 << 20) + (64 << 10))
 int mlora_workspace_init(void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Unfused shrink:  out[i, t, 0:r] = scaling * x[t] . A_i[s_t]^T  for s_t >= 0, and 0

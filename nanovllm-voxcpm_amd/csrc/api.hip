@@ -78,7 +78,7 @@ namespace {
 
 // Diagnostic knobs, read from the environment once per process.
 struct ApiKnobs {
-  int generation = -1, small_batch_tokens, force_form, no_split, split_min_k, auto_fused;
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, auto_fused;
   void read() {
     generation = knob_generation();
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
@@ -90,12 +90,14 @@ struct ApiKnobs {
     // dependent slab fetches per workgroup, HBM nearly idle) and then expands; the saved launch
     // does not pay for the wait on the slowest role of each unit.  AUTO keeps the two launches.
     auto_fused = env_int("MLORA_AUTO_FUSED", 0);
-    // Measured on the decode batch (32 tiles): at K = 4096 one workgroup per (tile, column range)
-    // takes 6.9 us per call, the split form 8.0 (what producers publish reaches the consumers 1.6 us
-    // later, two trips through the memory system; that is more than spreading the shrink saves), at
-    // K = 1024 4.2-7.4 against 6.9-11.5.  From K = 8192 on a workgroup's K range no longer fits its
-    // registers in one batch of loads, and the split form takes over.
-    split_min_k = env_int("MLORA_SPLIT_MIN_K", 8192);
+    // The split form pays when A[slot], which every workgroup of a tile would otherwise fetch whole,
+    // is large: rank x K >= 131072 elements (256 KB).  Measured on the decode batch (256 tokens, 32
+    // adapters), one workgroup per (tile, column range) against the split form, us per call: rank 16,
+    // K = 4096: 6.9 / 8.0 (what producers publish reaches the consumers 1.6 us later, two trips
+    // through the memory system; more than spreading 128 KB saves); rank 32, K = 4096: 15.5 / 10.5;
+    // rank 32, K = 1024: 4.9-10.0 / 8.1-17.1; rank 16, K = 8192: the K range of a workgroup no
+    // longer fits its registers as one batch of loads.
+    split_min_rk = env_int("MLORA_SPLIT_MIN_RK", 131072);
   }
 };
 const ApiKnobs& knobs() {
@@ -179,10 +181,10 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     else if (small_tiles) form = MLORA_FORM_SPLIT;
     else form = MLORA_FORM_BGMV;
   }
-  // the split form where it pays (very long K) and shape and workspace allow it, else one
+  // the split form where it pays (a large A[slot]) and shape and workspace allow it, else one
   // workgroup per (tile, column range)
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
-      (knobs().no_split || !split_supported(a) || (a->k < knobs().split_min_k && knobs().force_form != MLORA_FORM_SPLIT)))
+      (knobs().no_split || !split_supported(a) || (static_cast<long long>(a->r) * a->k < knobs().split_min_rk && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;
   // long-segment batches in one launch, on request
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))

@@ -187,7 +187,7 @@ constexpr int kWsTimeoutsWord = 1;
 constexpr int kWsTileOff = 256;
 constexpr int kWsTiles = 1024;
 constexpr int kWsXchgOff = 16384;
-constexpr int kWsXchgBytes = 1 << 20;
+constexpr int kWsXchgBytes = 4 << 20;
 // behind the exchange area: one 64-bit seal per (unit, shrink role) of the one-launch
 // long-segment form: {generation of the unit + 1, XCD of the writer}
 constexpr int kWsSealBytes = 64 << 10;

@@ -44,7 +44,7 @@ PLAN_MAGIC_VALUE = 0x4D4C5031
 SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 16, 64
 SMALL_TILE_WORDS, SMALL_TILE_ROWS, BIG_TILE_WORDS = 32, 4, 4
 STATIC_SCRATCH_BYTES = 16 << 20
-WORKSPACE_HEAD_BYTES = 16384 + (1 << 20) + (64 << 10)
+WORKSPACE_HEAD_BYTES = 16384 + (4 << 20) + (64 << 10)
 WORKSPACE_TIMEOUTS_WORD = 1  # uint32 index in the workspace head: waits of the split form that ran out
 
 _DTYPES = {torch.float32: DTYPE_F32, torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}

@@ -66,7 +66,7 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
                          ("MLORA_TILE_SMALL", 16), ("MLORA_SMALL_TILE_WORDS", _hip.SMALL_TILE_WORDS), ("MLORA_BIG_TILE_WORDS", _hip.BIG_TILE_WORDS), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
                          ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS), ("MLORA_FORM_SPLIT", _hip.FORM_SPLIT)):
         assert re.search(rf"#define {macro} {value}\b", text), macro
-    assert re.search(r"#define MLORA_WORKSPACE_HEAD_BYTES \(16384 \+ \(1 << 20\) \+ \(64 << 10\)\)", text) and _hip.WORKSPACE_HEAD_BYTES == 16384 + (1 << 20) + (64 << 10)
+    assert re.search(r"#define MLORA_WORKSPACE_HEAD_BYTES \(16384 \+ \(4 << 20\) \+ \(64 << 10\)\)", text) and _hip.WORKSPACE_HEAD_BYTES == 16384 + (4 << 20) + (64 << 10)
     assert re.search(r"#define MLORA_STATIC_SCRATCH_BYTES \(16u << 20\)", text) and _hip.STATIC_SCRATCH_BYTES == 16 << 20
 
 
