@@ -128,10 +128,10 @@ int mlora_add_lora_static(const MloraAddArgs* args);
  * splits K less, or AUTO does not choose it). */
 size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t r, int32_t dtype);
 
-/* A workspace starts with a head of MLORA_WORKSPACE_HEAD_BYTES bytes: a signature word, one
- * {generation, arrivals} pair per small tile (or group of 64-token tiles), the area in which
- * producer workgroups of MLORA_FORM_SPLIT leave the intermediate for the consumers, every word
- * tagged with its tile's generation, and the seals (generation and XCD of the writer) that the
+/* A workspace starts with a head of MLORA_WORKSPACE_HEAD_BYTES bytes: a signature word, the
+ * workspace's {generation, arrivals} pair (advanced once per launch that uses the head), the area
+ * in which producer workgroups of MLORA_FORM_SPLIT leave the intermediate for the consumers, every
+ * word tagged with the generation, and the seals (generation and XCD of the writer) that the
  * workgroups of MLORA_FORM_FUSED put on the partial sums they wrote.  mlora_workspace_init enqueues one kernel that clears the head and writes the
  * signature; call it once after allocation (it is a kernel, not a memset, so it may be recorded
  * into a graph).  Launches leave the head ready for the next launch.  A workspace whose head

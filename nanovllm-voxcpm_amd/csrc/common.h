@@ -179,9 +179,13 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
 }
 
 // ---- workspace head (see MLORA_WORKSPACE_HEAD_BYTES in mlora.h) -------------------------------
-// uint32 words:  [0] signature | [1] waits that ran out (diagnostic) | ... ; at byte kWsTileOff one
-// {generation, arrivals} pair per small tile; at byte kWsXchgOff the exchange area of the split
-// form: 64-bit words {fp32 bits, tag}, valid when tag == generation of the tile + 1.
+// uint32 words:  [0] signature | [1] waits that ran out (diagnostic) | ... ; at byte kWsTileOff the
+// {generation, arrivals} pair of the workspace (every workgroup of a split or one-launch
+// long-segment grid reports once when it is done, the last one advances the generation; the rest of
+// the 8 KiB behind it is reserved); at byte kWsXchgOff the exchange area of the split form: 64-bit
+// words {fp32 bits, tag}, valid when tag == generation + 1.  One generation for the whole
+// workspace: whatever an earlier launch left anywhere in the area, in whatever layout, carries a
+// tag below the current one.
 constexpr uint32_t kWsMagic = 0x4d4c5733u;  // "MLW3"
 constexpr int kWsTimeoutsWord = 1;
 constexpr int kWsTileOff = 256;

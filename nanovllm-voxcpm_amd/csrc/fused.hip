@@ -21,8 +21,9 @@
 // will free its compute-unit slots without outside help; a unit's members wait only for each
 // other.  Should a seal still be missing after `spin_ticks` (or the workspace head be
 // uninitialised), the waiting workgroup computes the missing roles itself: the same arithmetic in
-// the same order, so the words it writes are the ones the late producer writes.  The last member
-// to finish advances the unit's generation, which makes every seal of this launch stale.
+// the same order, so the words it writes are the ones the late producer writes.  The last
+// workgroup of the grid to finish advances the workspace's generation, which makes every seal of
+// this launch stale.
 #include "sgmv_body.h"
 
 namespace mlora {
@@ -112,7 +113,9 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   for (int g = 0; g < G; ++g) big[g] = reinterpret_cast<const i32x4*>(plan + big_off)[is_big ? unit * G + g : 0];
   const ExpandSplit sp = splits.split[c];
   const uint32_t signature = ws[0];
-  uint32_t* const ustate = ws + kWsTileOff / 4 + 2 * unit;  // {generation, arrivals}; unit < kWsTiles (host)
+  // {generation, arrivals} of the workspace: one pair for the whole launch, so that every seal any
+  // earlier launch left anywhere (whatever its layout was) carries a tag below this launch's
+  uint32_t* const ustate = ws + kWsTileOff / 4;
   const uint32_t tag = ustate[0] + 1u;
   const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
   int slot[G], start[G], m[G], any = 0;
@@ -136,11 +139,25 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
     }
     any |= m[g];
   }
-  // One exit test, the same for every workgroup of a unit (they count each other at the end)
+  // One exit test, the same for every workgroup of a unit
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0);
-  if (!usable) return;
   const bool xok = trusted | (signature == kWsMagic);  // seals and generations can be used
+  // every workgroup of the grid reports exactly once that it is done (also the ones without work);
+  // the last one advances the generation, which makes every seal of this launch stale
+  auto count_done = [&]() {
+    if (xok && tid == 0) {
+      const uint32_t before = __hip_atomic_fetch_add(ustate + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (before + 1u == gridDim.x * gridDim.y * gridDim.z) {
+        __hip_atomic_store(ustate + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(ustate, tag == 0xffffffffu ? 0u : tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // generation + 1, the next tag, is never 0
+      }
+    }
+  };
+  if (!usable) {
+    count_done();
+    return;
+  }
   MLORA_STAMP(1);  // records, ranks and generation are here
 
   if (tid == 0) {
@@ -229,14 +246,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   fused_expand<T, R, CPL, TPF, G>(s_h, s_row, s_slot, s_m, s_eff, s_start, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt, sp);
 
   MLORA_STAMP(13);  // expanded (wavefront 0)
-  // ---- the last member of the unit to get here advances its generation ---------------------------------
-  if (xok && tid == 0) {
-    const uint32_t before = __hip_atomic_fetch_add(ustate + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (before + 1u == static_cast<uint32_t>(W)) {
-      __hip_atomic_store(ustate + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(ustate, tag == 0xffffffffu ? 0u : tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // generation + 1, the next tag, is never 0
-    }
-  }
+  count_done();
 }
 
 // Diagnostic knobs, read from the environment once and again after mlora_reload_knobs().

@@ -110,7 +110,10 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
   const uint32_t signature = ws[0];
   const RankPrefetch ranks = rank_prefetch(MASKED ? eff_rank : nullptr, num_slots, lane);
-  uint32_t* const tstate = ws + kWsTileOff / 4 + 2 * tile;  // {generation, arrivals}; tile < kWsTiles (host)
+  // {generation, arrivals} of the workspace: one pair for the whole launch, so that every tagged
+  // word any earlier launch left anywhere in the exchange area (whatever its layout was) carries a
+  // tag below this launch's
+  uint32_t* const tstate = ws + kWsTileOff / 4;
   const uint32_t tag = tstate[0] + 1u;
   const int slot = rec0[0], m = rec0[1];
   const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
@@ -118,15 +121,34 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
                      int(slot < num_slots);
-  if (!usable) return;
-  MLORA_STAMP(1);  // tile record, plan header and tile generation are here
   const bool xok = trusted | (signature == kWsMagic);  // the exchange area can be used
+  // Every workgroup of the grid reports exactly once that it is done with the exchange area (also
+  // the ones without work); the last one advances the generation.  Counted by the last wavefront,
+  // which has the least other work: the count comes back from the memory system long after it was
+  // sent, and whoever sent it has to wait for it.
+  auto count_done = [&]() {
+    if (xok && tid == kNT - kWave) {
+      const uint32_t before = xadd(tstate + 1, 1u, wide);
+      if (before + 1u == gridDim.x * gridDim.y * gridDim.z) {
+        xstore32(tstate + 1, 0u, wide);
+        xstore32(tstate, tag == 0xffffffffu ? 0u : tag, wide);  // so that generation + 1, the next tag, is never 0
+      }
+    }
+  };
+  if (!usable) {
+    count_done();
+    return;
+  }
+  MLORA_STAMP(1);  // tile record, plan header and generation are here
 
   // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
   // (MASKED = false is the instance for callers that gave no rank vector: eff is the constant R
   // there and every test on it below folds away)
   const int eff = MASKED ? rank_pick(ranks, eff_rank, num_slots, slot, R) : R;
-  if (MASKED && eff == 0) return;  // nothing resident: the same for every workgroup of the tile
+  if (MASKED && eff == 0) {  // nothing resident: the same for every workgroup of the tile
+    count_done();
+    return;
+  }
   const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
 
   // Roles.  Asymmetric launch: S * P producers (slice, K part), then the consumers (slice, column
@@ -144,7 +166,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
       n0 = part * ws_cols < sl.n[slice] ? part * ws_cols : sl.n[slice];
       n1 = n0 + ws_cols < sl.n[slice] ? n0 + ws_cols : sl.n[slice];
     } else if (!xok) {
-      return;  // nobody would read what this workgroup publishes
+      return;  // nobody would read what this workgroup publishes (and nobody counts)
     }
   } else {
     const int c = role - S * P;
@@ -218,19 +240,6 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
     __syncthreads();  // s_red may be rewritten by the next part
   };
 
-  // Generation of the tile advanced by the last of its workgroups to be done with the exchange area.
-  // Counted by the last wavefront, which has the least other work: the count comes back from the
-  // memory system long after it was sent, and whoever sent it has to wait for it.
-  auto count_done = [&]() {
-    if (tid == kNT - kWave) {
-      const uint32_t before = xadd(tstate + 1, 1u, wide);
-      if (before + 1u == gridDim.y) {
-        xstore32(tstate + 1, 0u, wide);
-        xstore32(tstate, tag == 0xffffffffu ? 0u : tag, wide);  // so that generation + 1, the next tag, is never 0
-      }
-    }
-  };
-
   // ================================ consumer part: loads =========================================
   // ---- every load of the expand goes out first (before the shrink of a symmetric workgroup too) --
   const T* const Bs = static_cast<const T*>(sl.b[slice]) + static_cast<int64_t>(slot) * N * R;
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
     MLORA_STAMP(3);  // producer: partial sums handed to the memory system
   }
   if (!consumer || n0 >= n1) {  // nothing to expand here
-    if (xok) count_done();
+    count_done();
     MLORA_STAMP(15);  // role marker: pure producers leave slot 15 non-zero
     return;
   }
@@ -379,7 +388,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
       if (c0 < n1) load_span(c0, bop[s], yq[s]);
     }
   }
-  if (xok) count_done();  // this workgroup reads the exchange area no more
+  count_done();  // this workgroup reads the exchange area no more
   MLORA_STAMP(6);  // consumer: the intermediate is in LDS, the arrival counted
 
   // ---- expand ---------------------------------------------------------------------------------------

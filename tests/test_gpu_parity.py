@@ -157,7 +157,7 @@ def test_split_form_producers_and_consumers(name, rank, kpart, wide, sym, monkey
     Checked: parity for both K-part widths, both role layouts and both access scopes, bit-identical results from one
     launch to the next and between accepting published sums, never accepting them and not waiting
     at all (the order of every sum is fixed, whatever the timing), slot -1 rows untouched, no wait
-    running out in the ordinary runs, every tile's arrival count back at zero after each launch,
+    running out in the ordinary runs, the arrival count back at zero and the generation one step on after each launch,
     and the same result from a workspace that was never initialised."""
     from nanovllm_voxcpm_amd import _hip, synthetic
 
@@ -192,15 +192,51 @@ def test_split_form_producers_and_consumers(name, rank, kpart, wide, sym, monkey
         assert torch.equal(runs[0], other)
     (scratch,) = backend._scratch.values()
     head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
-    state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} per tile
+    state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} of the workspace, then reserved words
     assert all(arrivals == 0 for _, arrivals in state)
-    assert any(generation > 0 for generation, _ in state)
+    assert state[0][0] == len(runs) and all(generation == 0 for generation, _ in state[1:])  # one step per launch
     # a workspace without the signature: same bits, nothing published, nobody waits
     scratch[:4].zero_()
     _knobs(monkeypatch, MLORA_SPLIT_SPIN_TICKS=20000)
     assert torch.equal(run(), runs[0])
     assert _waits_run_out(backend) == 0
     assert head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist() == state
+
+
+def test_split_form_ignores_what_a_launch_of_another_layout_left():
+    """Two projections of different shape share one workspace, as the layers of a model do.  The
+    first launch (three slices, few tiles) leaves tagged sums all over the exchange area; the second
+    (one slice, long K, more tiles, among them tiles the first never had) lays its own sums out
+    differently over the same bytes.  Its consumers must not take any of the old words for new ones:
+    same bits as on a workspace nobody used before, in either order of the two launches."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    shapes = {"three": (1024, [512, 128, 128]), "long": (4096, [1024])}
+    projs = {n: synthetic.make_projection(n, 24, 32, torch.bfloat16, seed=150, device="cuda", shapes=shapes) for n in shapes}
+    g = torch.Generator().manual_seed(151)
+    few = torch.randint(0, 3, (40,), generator=g, dtype=torch.int32).cuda()      # three slots: three or four tiles
+    many = torch.randint(-1, 24, (200,), generator=g, dtype=torch.int32).cuda()  # every slot: thirty tiles or so
+    batches = {"three": few, "long": many}
+    data = {n: synthetic.make_activations(batches[n].numel(), projs[n].k, sum(projs[n].widths), torch.bfloat16, seed=152, device="cuda") for n in shapes}
+
+    def run(backend, n):
+        x, y0 = data[n]
+        y = y0.clone()
+        blocks = list(y.split(projs[n].widths, dim=-1))
+        backend.add_lora(blocks, x, projs[n].a, projs[n].b, indices=batches[n], metadata=_metadata(batches[n]), scaling=1.0,
+                         y_packed=y if len(blocks) > 1 else None)
+        return y
+
+    fresh = {n: run(_backend("split"), n) for n in shapes}
+    for order in (("three", "long"), ("long", "three"), ("three", "three", "long", "long", "three")):
+        shared = _backend("split")
+        for n in order:
+            assert torch.equal(run(shared, n), fresh[n]), f"{n} after {order}"
+        assert _waits_run_out(shared) == 0
+    for n in shapes:
+        x, y0 = data[n]
+        exact, mag = _exact(projs[n], x, y0, batches[n])
+        _check(fresh[n], y0, exact, mag, batches[n], f"split/shared-workspace/{n}")
 
 
 def test_config2_matches_reference_torch_loop():
@@ -380,7 +416,8 @@ def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
     adapter, ragged widths, strided views).  Checked: parity; the bits of the two-launch form where
     neither cuts K (same sums, same order); the same bits on a second launch, when no seal is ever accepted
     (every workgroup computes what it needs itself) and on a workspace without the signature; no
-    wait running out in the ordinary runs; every unit's arrival count back at zero."""
+    wait running out in the ordinary runs; the arrival count back at zero and the generation one
+    step on after each launch."""
     from nanovllm_voxcpm_amd import _hip, synthetic
 
     print(f"one-launch long form r={rank} {dtype} {knobs}", flush=True)
@@ -425,9 +462,9 @@ def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
             assert torch.allclose(got.float(), two.float(), rtol=RTOL, atol=ATOL)
         (scratch,) = backend._scratch.values()
         head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
-        state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} per unit
+        state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} of the workspace, then reserved words
         assert all(arrivals == 0 for _, arrivals in state)
-        assert any(generation > 0 for generation, _ in state)
+        assert state[0][0] == len(runs) and all(generation == 0 for generation, _ in state[1:])  # one step per launch
         # a workspace without the signature: nobody seals, nobody waits, same bits
         scratch[:4].zero_()
         _knobs(monkeypatch, MLORA_FUSED_SPIN_TICKS=50000)
