@@ -514,6 +514,27 @@ def measure_unfused(layers, slots, name: str = "qkv") -> dict:
     return out
 
 
+def measure_long_form_latency(layers, slots) -> dict:
+    """What a call of the two-launch long-segment form costs before it moves any data to speak of:
+    the prefill step's 96 calls (same buffers, same grids) on a batch in which no token has an
+    adapter slot (both launches find nothing to do) and on one in which a single token has one (one
+    workgroup per launch walks the whole chain: record, token rows, operands, multiply, store).
+    Microseconds per call, graph replay."""
+    import torch
+
+    out = {}
+    none = torch.full_like(slots, -1)
+    one = none.clone()
+    one[0] = 0
+    for key, batch in (("us_per_call_no_token_has_a_slot", none), ("us_per_call_one_token_has_a_slot", one)):
+        step, calls = make_step(layers, batch, "sgmv")
+        graph = capture(step)
+        for _ in range(3):
+            graph.replay()
+        out[key] = round(time_region(graph.replay, 10) * 1e3 / calls, 2)
+    return out
+
+
 def measure_floor(device: str, step_bytes: int, calls: int) -> dict:
     """What bounds a step of `calls` dependent launches on this machine, measured in this run:
     a replayed graph of as many kernels that do nothing (one wavefront each, then the grid of a
@@ -667,10 +688,13 @@ def main() -> None:
         out["floor"] = measure_floor(device, res["algorithmic_bytes_per_step"], res["calls_per_step"])
         extra = {}
         for name in ("prefill", "mixed"):
-            r, _ = measure_workload(name, device, "auto", 5, 2, per_projection=True)
+            r, (wl_layers, wl_slots, _, _) = measure_workload(name, device, "auto", 5, 2, per_projection=True)
             extra[name] = {k: r[k] for k in ("config", "us_per_step", "value", "pct_of_hbm_peak", "tflops", "pct_of_mfma_bf16_peak",
                                              "algorithmic_bytes_per_step", "us_per_call_by_projection", "roofline")}
             extra[name]["unit"] = "GB/s"
+            if name == "prefill":
+                extra[name]["latency"] = measure_long_form_latency(wl_layers, wl_slots)
+            del wl_layers, wl_slots
             torch.cuda.empty_cache()
         extra["backbone"] = measure_backbone(10, 3)
         extra["unfused_ops"] = measure_unfused(layers, slots)
