@@ -78,7 +78,7 @@ namespace {
 
 // Diagnostic knobs, read from the environment once per process.
 struct ApiKnobs {
-  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, auto_fused;
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, split_max_tokens, auto_fused;
   void read() {
     generation = knob_generation();
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
@@ -98,6 +98,9 @@ struct ApiKnobs {
     // rank 32, K = 1024: 4.9-10.0 / 8.1-17.1; rank 16, K = 8192: the K range of a workgroup no
     // longer fits its registers as one batch of loads.
     split_min_rk = env_int("MLORA_SPLIT_MIN_RK", 131072);
+    // ... and while the batch has few tiles: K = 4096, rank 32 / 64, 1011 tokens: 12.0 / 17.7 us against
+    // 14.8 / 23.1; 1620 tokens: 17.6 / 26.8 against 15.8 / 24.7
+    split_max_tokens = env_int("MLORA_SPLIT_MAX_TOKENS", 1280);
   }
 };
 const ApiKnobs& knobs() {
@@ -109,20 +112,23 @@ const ApiKnobs& knobs() {
 }  // namespace
 
 // Where the one-launch form over 16-token tiles stops paying.  Its cost per token grows with the
-// rank (every tile fetches A[slot] again, every column range repeats its tile's shrink) while the
-// two-launch form pays about 10 us up front; measured per projection shape, single- and
-// multi-adapter batches of 512..16384 tokens, the two meet where tokens x (slices x K + columns)
-// reaches 8.4e7 for ranks up to 16, 1.7e7 for rank 32 and about 1.2e7 for rank 64 (rank 64: 850
-// tokens for gate_up, 2200 for down, 3500 for qkv, 7500 for o; rank 16: 8200 for gate_up, never
-// below 16384 for o and qkv).
+// rank (every tile fetches A[slot] and B[slot] again, every column range repeats its tile's shrink)
+// while a two-launch call pays 11.6 us before it moves any data (3.5 us for one launch over small
+// tiles).  Measured per projection shape on prefill batches of 1011..9392 tokens (1..16 sequences,
+// up to 8 adapters), the two forms meet where tokens x width reaches about 1.4e7 at rank 64 and
+// 2.4e7 at rank 32, with width = slices x K x max(1, K / 2048) + columns x max(1, columns / 4096):
+// long K and wide outputs cost the small tiles more than their share (tokens at the
+// crossing, rank 64 / rank 32: qkv 5000 / 6500, o 8500 / 11000, gate_up 1000 / 1300, down
+// 1200 / 2100).  At rank 16 and below only gate_up crosses before 16384 tokens (at 8200).
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
 static bool small_batch(const MloraAddArgs* a) {
   const int fixed = knobs().small_batch_tokens;
   if (fixed > 0) return a->num_tokens <= fixed;
-  long long width = static_cast<long long>(a->num_slices) * a->k;
-  for (int i = 0; i < a->num_slices; ++i) width += a->slices[i].n;
-  const long long limit = a->r <= 16 ? 84000000LL : a->r <= 32 ? 17000000LL : 12000000LL;
-  return static_cast<long long>(a->num_tokens) * width <= limit;
+  double cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+  const double width = static_cast<double>(a->num_slices) * a->k * (a->k > 2048 ? a->k / 2048.0 : 1.0) + cols * (cols > 4096 ? cols / 4096.0 : 1.0);
+  const double limit = a->r <= 16 ? 1.5e8 : a->r <= 32 ? 2.4e7 : 1.4e7;
+  return a->num_tokens * width <= limit;
 }
 
 namespace {
@@ -184,7 +190,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   // the split form where it pays (a large A[slot]) and shape and workspace allow it, else one
   // workgroup per (tile, column range)
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
-      (knobs().no_split || !split_supported(a) || (static_cast<long long>(a->r) * a->k < knobs().split_min_rk && knobs().force_form != MLORA_FORM_SPLIT)))
+      (knobs().no_split || !split_supported(a) || ((static_cast<long long>(a->r) * a->k < knobs().split_min_rk || a->num_tokens > knobs().split_max_tokens) && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;
   // long-segment batches in one launch, on request
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))

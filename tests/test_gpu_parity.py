@@ -477,10 +477,10 @@ def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
 def test_auto_form_follows_rank_and_width(rank, expected):
     """A 3000-token prefill of three sequences through the o projection: at rank 16 the one-launch
     small-tile form is the faster one up to far larger batches, at rank 64 the two-launch form
-    takes over near 6000 tokens.  AUTO gives the oracle's result in both cases
+    takes over near 8500 tokens (here 12000).  AUTO gives the oracle's result in both cases
     and exactly what the form it is meant to pick gives."""
     print(f"auto form r={rank}", flush=True)
-    T = 3000 if rank == 16 else 7000
+    T = 3000 if rank == 16 else 12000
     proj = _make("o", 4, rank, torch.bfloat16, seed=330 + rank)
     slots = torch.cat([torch.full((T // 2,), 1, dtype=torch.int32), torch.full((T // 4,), -1, dtype=torch.int32),
                        torch.full((T - T // 2 - T // 4,), 3, dtype=torch.int32)]).cuda()
