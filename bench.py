@@ -72,7 +72,7 @@ def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int, token_r
     return 2 * (t_lora * rank if token_rank_sum is None else token_rank_sum) * (len(widths) * k + sum(widths))
 
 
-def build_workload(name: str, device: str, rank: int | None = None):
+def build_workload(name: str, device: str, rank: int | None = None, sequences: int = 0):
     """Per-layer (projection weights, x, y) for the distinct layers of the workload and the
     batch's slot vector.  Layers beyond the distinct ones reuse buffers round-robin (the distinct
     set alone exceeds the 256 MB last-level cache)."""
@@ -86,7 +86,7 @@ def build_workload(name: str, device: str, rank: int | None = None):
         slots = synthetic.decode_slots(256, spec["slots"], seed=7)
         ranks = None
     elif name == "prefill":
-        slots, _ = synthetic.prefill_slots(16, spec["slots"], seed=301)
+        slots, _ = synthetic.prefill_slots(sequences or 16, spec["slots"], seed=301)
         ranks = None
     else:
         slots = synthetic.mixed_slots(seed=402)
@@ -385,14 +385,14 @@ def recorded_traffic(workload: str):
 
 
 def measure_workload(name: str, device: str, form: str, steps: int, warmup: int, *, only=None, rank=0, hot_layers=0, eager=False,
-                     per_projection=True, rank_vector=True) -> tuple[dict, tuple]:
+                     per_projection=True, rank_vector=True, sequences=0) -> tuple[dict, tuple]:
     """Time one workload: its step replayed as a captured graph (or eagerly), per-projection steps,
     bytes, flops and the roofline object.  Returns (result, (layers, slots, rank, step))."""
     import torch
 
     spec = WORKLOADS[name]
     rank = rank or spec["rank"]
-    layers, slots, eff = build_workload(name, device, rank)
+    layers, slots, eff = build_workload(name, device, rank, sequences)
     if not rank_vector:
         eff = None
     if hot_layers > 0:
@@ -441,7 +441,7 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
     calls = launches
     launch_bytes = step_bytes / calls
     call_us = ms * 1e3 / calls
-    default_shape = form == "auto" and not only and not hot_layers and rank == spec["rank"]
+    default_shape = form == "auto" and not only and not hot_layers and rank == spec["rank"] and not sequences
     result = {
         "value": round(value, 2),
         "ms_per_step": round(ms, 5),
@@ -610,6 +610,9 @@ def main() -> None:
                          "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
     ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
                     help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
+    ap.add_argument("--sequences", type=int, default=0,
+                    help="diagnostic (prefill workload): a batch of N sequences drawn like the 16 (1: 1011 tokens, "
+                         "2: 1620, 4: 2098, 8: 4511); 0 = all 16")
     ap.add_argument("--no-rank-vector", action="store_true",
                     help="diagnostic (mixed workload): do not tell the kernels the adapters' true ranks; the zero "
                          "padding of the rank-64 buffers is then read and multiplied like any other data")
@@ -654,7 +657,8 @@ def main() -> None:
     warmup = args.warmup if not heavy else max(1, min(args.warmup, 3))
     rank = args.rank if args.workload in ("decode", "prefill") else 0
     res, (layers, slots, rank, step) = measure_workload(args.workload, device, args.form, steps, warmup, only=args.only, rank=rank,
-                                                        hot_layers=args.hot_layers, eager=args.eager, rank_vector=not args.no_rank_vector)
+                                                        hot_layers=args.hot_layers, eager=args.eager, rank_vector=not args.no_rank_vector,
+                                                        sequences=args.sequences if args.workload == "prefill" else 0)
     out = {
         "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
         "value": res["value"],
