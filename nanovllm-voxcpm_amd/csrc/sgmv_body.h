@@ -250,7 +250,8 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
 // Body of the expand for the tiles of one workgroup.  MASKED: some tile's slot holds an adapter of
 // fewer ranks than the buffers: chunks of the intermediate the shrink did not write are not read,
 // ranks at or above the adapter's are zero in the intermediate, B columns from that rank on are
-// neither fetched nor multiplied.  The unmasked instance is the code without any of those tests.
+// not fetched (zeros take their place in the operand).  The unmasked instance is the code without
+// any of those tests.
 //
 // SC1: the partial sums are fetched with agent-scope loads (past the compute unit's and the XCD's
 // caches): they were written by other workgroups of the same launch.
@@ -308,7 +309,6 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   };
   Pack8 bop[CPL][KSTEPS];
   int b_slot = -1, b_c0 = -1;  // what bop holds
-  int b_ks = KSTEPS;  // k-steps of the slot bop holds
   auto load_b = [&](int c0, int sg, int eg) {
     // the B rows of the span (lanes whose chunk lies beyond the rank fetch a valid chunk anyway,
     // their H operand is zero; columns past the range repeat the last one and are never stored)
@@ -346,7 +346,6 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     }
     b_slot = sg;
     b_c0 = c0;
-    if constexpr (MASKED) b_ks = (eg + 31) >> 5;
   };
   auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
     const int g = st / NB, tp = (st % NB) * TPF;
@@ -377,9 +376,6 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
         out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          if constexpr (MASKED && KSTEPS > 1) {
-            if (ks >= b_ks) continue;
-          }
           out[j] = Mma<T>::run(hlo[ks], bop[j][ks], out[j]);
           out[j] = Mma<T>::run(hop[ks], bop[j][ks], out[j]);
         }
