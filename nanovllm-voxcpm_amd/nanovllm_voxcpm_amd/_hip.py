@@ -296,9 +296,18 @@ def plan_workspace_words(num_tokens: int, max_slots: int) -> int:
     return (load().mlora_plan_workspace_bytes(num_tokens, max_slots) + 3) // 4
 
 
+_WORKSPACE_BYTES: dict = {}
+
+
 def add_workspace_bytes(num_tokens: int, num_slices: int, r: int, dtype: torch.dtype) -> int:
     """Bytes of scratch that let the fused apply use every form it has for this shape."""
-    return int(load().mlora_add_workspace_bytes(num_tokens, num_slices, r, dtype_code(dtype)))
+    key = (num_tokens, num_slices, r, dtype)
+    n = _WORKSPACE_BYTES.get(key)
+    if n is None:  # asked on every call with the handful of shapes a model has
+        if len(_WORKSPACE_BYTES) >= 256:
+            _WORKSPACE_BYTES.clear()
+        n = _WORKSPACE_BYTES[key] = int(load().mlora_add_workspace_bytes(num_tokens, num_slices, r, dtype_code(dtype)))
+    return n
 
 
 def workspace_init(workspace: torch.Tensor, stream: int | None = None) -> None:
@@ -336,12 +345,17 @@ def add_lora(
     lib = load()
     if len(a_slices) > MAX_SLICES:
         raise ValueError(f"at most {MAX_SLICES} slices per call, got {len(a_slices)}")
-    for name, t in (("y", y), ("token_to_slot", token_to_slot), *((f"lora_a[{i}]", a) for i, a in enumerate(a_slices)),
-                    *((f"lora_b[{i}]", b) for i, b in enumerate(b_slices))):
-        if t.device != x.device:
-            raise ValueError(f"{name} lives on {t.device}, x on {x.device}")
-        if name != "token_to_slot" and t.dtype != x.dtype:
-            raise ValueError(f"{name} has element type {t.dtype}, x has {x.dtype}")
+    dev, dt = x.device, x.dtype  # (names of the offenders are only put together when one is found: this runs per call)
+    if token_to_slot.device != dev:
+        raise ValueError(f"token_to_slot lives on {token_to_slot.device}, x on {dev}")
+    if y.device != dev or y.dtype != dt or any(t.device != dev or t.dtype != dt for t in a_slices) or \
+            any(t.device != dev or t.dtype != dt for t in b_slices):
+        for name, t in (("y", y), *((f"lora_a[{i}]", a) for i, a in enumerate(a_slices)),
+                        *((f"lora_b[{i}]", b) for i, b in enumerate(b_slices))):
+            if t.device != dev:
+                raise ValueError(f"{name} lives on {t.device}, x on {dev}")
+            if t.dtype != dt:
+                raise ValueError(f"{name} has element type {t.dtype}, x has {dt}")
     if token_to_slot.dtype != torch.int32 or not token_to_slot.is_contiguous():
         raise ValueError("token_to_slot must be a contiguous int32 tensor")
     if token_to_slot.numel() < x.size(0):
