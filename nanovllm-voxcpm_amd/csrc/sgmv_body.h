@@ -634,7 +634,11 @@ inline SgmvShape sgmv_shape(const MloraAddArgs* a, bool one_launch = false) {
   // expand: consecutive tiles per workgroup (they share their B rows when they share their
   // slot), then column ranges so that the grid has about 2048 workgroups
   int group = sgmv_knobs().group;
-  if (group != 1 && group != 2 && group != 4) group = (cols >= 4096 && est_tiles >= 64) ? 4 : 1;  // wide projections only: narrow ones need the workgroups
+  // wide projections only: narrow ones need the workgroups.  Two tiles per workgroup, not four: on
+  // the prefill batch (8 adapters) gate_up takes 72.2 against 73.2 us per call, on the mixed batch
+  // (126 adapters, many of them with fewer than four tiles) 105.8 against 110.4
+  if (group != 1 && group != 2 && group != 4) group = (cols >= 4096 && est_tiles >= 64) ? 2 : 1;
+  if (one_launch && group == 2) group = 4;  // the one-launch kernel exists for one tile and for four
   const int target = sgmv_knobs().wgs;
   int nt = sgmv_knobs().nt;
   if (nt <= 0) {
