@@ -134,6 +134,116 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
     for (int i = 0; i < XK; ++i) buf[i].raw = load128(xptr + kc + i * 32);
   };
 
+  // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
+  auto write_partials = [&](const f32x4(&part)[RB], int si) {
+    if (active && ti < m) {
+      float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice0 + si) * R;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int r0 = rb * 16 + 4 * lg;
+        if (r0 < R && (!MASKED || rb < rb_n)) {
+          if constexpr (SC1) {
+            uint64_t* q = reinterpret_cast<uint64_t*>(dst + r0);
+            __hip_atomic_store(q, (static_cast<uint64_t>(__float_as_uint(part[rb][1])) << 32) | __float_as_uint(part[rb][0]), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(q + 1, (static_cast<uint64_t>(__float_as_uint(part[rb][3])) << 32) | __float_as_uint(part[rb][2]), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+          } else {
+            *reinterpret_cast<f32x4*>(dst + r0) = part[rb];
+          }
+        }
+      }
+    }
+  };
+
+  if constexpr (!DB && KR == XW && KR >= 256) {
+    // A batch that is one slab: slab and batch are requested in NS column pieces, piece after
+    // piece (A piece, then the x columns it meets), all of them up front; a piece is copied to LDS
+    // and multiplied as soon as it is there, while the later ones are still on their way.  A piece
+    // of the slab has its own place in LDS and NS - 1 barriers lie between two uses of a place, so
+    // one barrier per piece is enough; a piece's registers take the next slab's piece (next batch
+    // or next slice) as soon as they are stored.
+    constexpr int NS = MASKED ? 2 : 4, SW = KR / NS, SCPR = SW / 8, STOTAL = R * SCPR, SCH = (STOTAL + NT - 1) / NT, KSS = KS / NS;
+    static_assert(KS % NS == 0, "pieces of whole k-steps");
+    i32x4 v[NS][SCH];
+    Pack8 xa[XK];
+    f32x4 acc[RB];
+    auto request_piece = [&](const T* Aslab, int s, i32x4(&buf)[SCH]) {
+#pragma unroll
+      for (int i = 0; i < SCH; ++i) {
+        const int c = i * NT + tid;
+        if constexpr (MASKED) {
+          if (i * (NT / SCPR) >= rows_used) continue;  // rows beyond the adapter's rank (the same for every thread)
+        }
+        if (STOTAL % NT == 0 || c < STOTAL) buf[i] = load128(Aslab + static_cast<int64_t>(c / SCPR) * K + s * SW + (c % SCPR) * 8);
+      }
+    };
+    auto store_piece = [&](int s, const i32x4(&buf)[SCH]) {
+#pragma unroll
+      for (int i = 0; i < SCH; ++i) {
+        const int c = i * NT + tid;
+        if constexpr (MASKED) {
+          if (i * (NT / SCPR) >= rows_used) continue;
+        }
+        if (STOTAL % NT == 0 || c < STOTAL) *reinterpret_cast<i32x4*>(&s_a[(c / SCPR) * ASTRIDE + s * SW + (c % SCPR) * 8]) = buf[i];
+      }
+    };
+    auto request_x_piece = [&](int kc, int s) {
+#pragma unroll
+      for (int i = 0; i < KSS; ++i) xa[s * KSS + i].raw = load128(xptr + kc + (s * KSS + i) * 32);
+    };
+    {
+      const T* A0 = static_cast<const T*>(sl.a[slice0]) + aoff;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        // (piece by piece: with every A piece ahead of the x columns the prefill step takes 3816
+        // against 3753 us)
+        request_piece(A0, s, v[s]);
+        if (active) request_x_piece(0, s);
+      }
+    }
+    MLORA_STAMP(3);  // shrink: first slab and first x batch requested (the token rows are here)
+    for (int si = 0; si < nsl; ++si) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int b = 0; b < nbatch; ++b) {
+        // the slab after this one: next batch, or the first of the next slice
+        const T* An = nullptr;
+        if (b + 1 < nbatch) An = static_cast<const T*>(sl.a[slice0 + si]) + aoff + (b + 1) * XW;
+        else if (si + 1 < nsl) An = static_cast<const T*>(sl.a[slice0 + si + 1]) + aoff;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          store_piece(s, v[s]);
+          if (b == 0 && s == 0 && si == 0) MLORA_STAMP(4);  // shrink: first piece arrived and is on its way to LDS
+          if (An) request_piece(An, s, v[s]);
+          __syncthreads();
+          if (active) {
+#pragma unroll
+            for (int i = s * KSS; i < (s + 1) * KSS; ++i) {
+#pragma unroll
+              for (int rb = 0; rb < RB; ++rb) {
+                if constexpr (MASKED) {
+                  if (rb >= rb_n) continue;
+                }
+                const int rr = rb * 16 + lr;
+                Pack8 aw;
+                aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + i * 32 + lg * 8]);
+                acc[rb] = Mma<T>::run(aw, xa[i], acc[rb]);
+              }
+            }
+          }
+        }
+        if (active && b + 1 < nbatch) {
+#pragma unroll
+          for (int s = 0; s < NS; ++s) request_x_piece((b + 1) * XW, s);
+        }
+      }
+      if (si == 0) MLORA_STAMP(5);  // shrink: first slice multiplied
+      write_partials(acc, si);
+    }
+    return;
+  }
+
   Pack8 xa[XK], xb[DB ? XK : 1];
   f32x4 acc[RB];
   bool first = true;
@@ -186,25 +296,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
       for (int b = 0; b < nbatch; ++b) run_batch(xa, xa, si, b);
     }
     if (si == 0) MLORA_STAMP(5);  // shrink: first slice multiplied
-    // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
-    if (active && ti < m) {
-      float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice0 + si) * R;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int r0 = rb * 16 + 4 * lg;
-        if (r0 < R && (!MASKED || rb < rb_n)) {
-          if constexpr (SC1) {
-            uint64_t* q = reinterpret_cast<uint64_t*>(dst + r0);
-            __hip_atomic_store(q, (static_cast<uint64_t>(__float_as_uint(acc[rb][1])) << 32) | __float_as_uint(acc[rb][0]), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(q + 1, (static_cast<uint64_t>(__float_as_uint(acc[rb][3])) << 32) | __float_as_uint(acc[rb][2]), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-          } else {
-            *reinterpret_cast<f32x4*>(dst + r0) = acc[rb];
-          }
-        }
-      }
-    }
+    write_partials(acc, si);
   }
 }
 
@@ -274,14 +366,73 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
 
-  // token rows -> LDS (entries past the end of a tile repeat its last token: a valid row to read,
-  // never written)
+  // The partial sums of a tile's intermediate: requested (every K part together), then summed,
+  // scaled, split and written to LDS.  The first tile's are requested before anything else: they
+  // depend on the tile record alone, and are on their way while the token rows make theirs.
+  const int64_t hrow = static_cast<int64_t>(num_slices) * R;
+  const int64_t part = static_cast<int64_t>(T_) * hrow;
+  f32x4 t[HC][kMaxKSplit][2];
+  auto request_h = [&](int g) {
+    const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
-    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
-  }
-  __syncthreads();
+    for (int h = 0; h < HC; ++h) {
+      const int c = h * NT + tid;
+      int tok = c / CPR;
+      tok = tok < m[g] ? tok : m[g] - 1;
+      const float* q = src + tok * hrow + (c % CPR) * 8;
+      const bool used = !MASKED || (c % CPR) * 8 < ((eff[g] + 15) & ~15);  // the shrink wrote this chunk
+#pragma unroll
+      for (int kp = 0; kp < kMaxKSplit; ++kp) {
+        if (kp < ksplit) {
+          if (used && SC1) {
+            const uint64_t* q8 = reinterpret_cast<const uint64_t*>(q + kp * part);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              const uint64_t pair = __hip_atomic_load(q8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              t[h][kp][w >> 1][2 * (w & 1)] = __uint_as_float(static_cast<uint32_t>(pair));
+              t[h][kp][w >> 1][2 * (w & 1) + 1] = __uint_as_float(static_cast<uint32_t>(pair >> 32));
+            }
+          } else if (used) {
+            t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
+            t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
+          } else {
+            t[h][kp][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            t[h][kp][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+      }
+    }
+  };
+  auto stage_h = [&](int g) {
+#pragma unroll
+    for (int h = 0; h < HC; ++h) {
+      const int c = h * NT + tid, tok = c / CPR, ch = c % CPR;
+      if ((MLORA_TILE_BIG * CPR) % NT != 0 && c >= MLORA_TILE_BIG * CPR) continue;
+      f32x4 s0 = t[h][0][0], s1 = t[h][0][1];
+#pragma unroll
+      for (int kp = 1; kp < kMaxKSplit; ++kp) {
+        if (kp < ksplit) {
+          s0[0] += t[h][kp][0][0]; s0[1] += t[h][kp][0][1]; s0[2] += t[h][kp][0][2]; s0[3] += t[h][kp][0][3];
+          s1[0] += t[h][kp][1][0]; s1[1] += t[h][kp][1][1]; s1[2] += t[h][kp][1][2]; s1[3] += t[h][kp][1][3];
+        }
+      }
+      Pack8 hi, lo;
+      float v[8], back[8], rem[8];
+      const float live = tok < m[g] ? scaling : 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = (!MASKED || ch * 8 + i < eff[g]) ? s0[i] * live : 0.f;  // ranks the adapter does not have contribute nothing
+        v[4 + i] = (!MASKED || ch * 8 + 4 + i < eff[g]) ? s1[i] * live : 0.f;
+      }
+      pack8<T>(v, hi);
+      unpack8<T>(hi, back);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
+      pack8<T>(rem, lo);
+      *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
+      *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
+    }
+  };
 
   // A wavefront's work is a sequence of items: for each of its spans of 16 * CPL columns, the
   // (tile, y batch) steps that hold tokens.  The y rows of the item after the current one are
@@ -293,7 +444,7 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
       if (s_m[st / NB] > (st % NB) * TPF * 16) break;
     return st;
   };
-  const int first_step = next_step(-1);  // exists: some tile holds tokens
+  int first_step = 0;  // (set once the tiles' sizes are in LDS)
   auto column = [&](int c0) {  // first of this lane's CPL columns, clamped into the range
     const int c = c0 + CPL * lr;
     return c < sp.n1 ? c : sp.n1 - 8;
@@ -395,8 +546,28 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   };
 
   YVec<T, CPL> ya[TPF][4], yb[TPF][4];
-  int c0 = sp.n0 + wave * SPAN, st = first_step;
+  int c0 = sp.n0 + wave * SPAN;
   const bool has_work = c0 < sp.n1;
+
+  // The token rows go out first: they are what the y rows wait for.  Entries of the row list past
+  // the end of a tile repeat its last token (a valid row to read, never written).  The partial
+  // sums of the first tile hang on the tile record alone and are on their way meanwhile (the B
+  // rows of the first span could be too, but they are 16 KB per wavefront and hold the token
+  // rows up: the prefill step 3748 -> 3858 us).
+  int rowv[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
+    rowv[g] = 0;
+    if (m[g] > 0 && tid < MLORA_TILE_BIG) rowv[g] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
+  }
+  if (m[0] > 0) request_h(0);
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = rowv[g];
+  __syncthreads();
+  first_step = next_step(-1);  // exists: some tile holds tokens
+  int st = first_step;
   if (has_work) {
     load_b(c0, s_slot[st / NB], s_eff[st / NB]);
     issue_y(ya, c0, st);
@@ -404,71 +575,11 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
 
   // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
   // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
-  {
-    const int64_t hrow = static_cast<int64_t>(num_slices) * R;
-    const int64_t part = static_cast<int64_t>(T_) * hrow;
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      if (m[g] == 0) continue;
-      const float* src = hws + static_cast<int64_t>(start[g]) * hrow + sp.slice * R;
-      f32x4 t[HC][kMaxKSplit][2];
-#pragma unroll
-      for (int h = 0; h < HC; ++h) {
-        const int c = h * NT + tid;
-        int tok = c / CPR;
-        tok = tok < m[g] ? tok : m[g] - 1;
-        const float* q = src + tok * hrow + (c % CPR) * 8;
-        const bool used = !MASKED || (c % CPR) * 8 < ((eff[g] + 15) & ~15);  // the shrink wrote this chunk
-#pragma unroll
-        for (int kp = 0; kp < kMaxKSplit; ++kp) {
-          if (kp < ksplit) {
-            if (used && SC1) {
-              const uint64_t* q8 = reinterpret_cast<const uint64_t*>(q + kp * part);
-#pragma unroll
-              for (int w = 0; w < 4; ++w) {
-                const uint64_t pair = __hip_atomic_load(q8 + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                t[h][kp][w >> 1][2 * (w & 1)] = __uint_as_float(static_cast<uint32_t>(pair));
-                t[h][kp][w >> 1][2 * (w & 1) + 1] = __uint_as_float(static_cast<uint32_t>(pair >> 32));
-              }
-            } else if (used) {
-              t[h][kp][0] = *reinterpret_cast<const f32x4*>(q + kp * part);
-              t[h][kp][1] = *reinterpret_cast<const f32x4*>(q + kp * part + 4);
-            } else {
-              t[h][kp][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-              t[h][kp][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int h = 0; h < HC; ++h) {
-        const int c = h * NT + tid, tok = c / CPR, ch = c % CPR;
-        if ((MLORA_TILE_BIG * CPR) % NT != 0 && c >= MLORA_TILE_BIG * CPR) continue;
-        f32x4 s0 = t[h][0][0], s1 = t[h][0][1];
-#pragma unroll
-        for (int kp = 1; kp < kMaxKSplit; ++kp) {
-          if (kp < ksplit) {
-            s0[0] += t[h][kp][0][0]; s0[1] += t[h][kp][0][1]; s0[2] += t[h][kp][0][2]; s0[3] += t[h][kp][0][3];
-            s1[0] += t[h][kp][1][0]; s1[1] += t[h][kp][1][1]; s1[2] += t[h][kp][1][2]; s1[3] += t[h][kp][1][3];
-          }
-        }
-        Pack8 hi, lo;
-        float v[8], back[8], rem[8];
-        const float live = tok < m[g] ? scaling : 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          v[i] = (!MASKED || ch * 8 + i < eff[g]) ? s0[i] * live : 0.f;  // ranks the adapter does not have contribute nothing
-          v[4 + i] = (!MASKED || ch * 8 + 4 + i < eff[g]) ? s1[i] * live : 0.f;
-        }
-        pack8<T>(v, hi);
-        unpack8<T>(hi, back);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) rem[i] = v[i] - back[i];
-        pack8<T>(rem, lo);
-        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + ch * 8]) = hi.raw;
-        *reinterpret_cast<i32x4*>(&s_h[(g * MLORA_TILE_BIG + tok) * HSTRIDE + R + ch * 8]) = lo.raw;
-      }
-    }
+  for (int g = 0; g < G; ++g) {
+    if (m[g] == 0) continue;
+    if (g > 0) request_h(g);
+    stage_h(g);
   }
   __syncthreads();
   if (!has_work) return;
