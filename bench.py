@@ -243,6 +243,12 @@ STAMPS = {
     "split_kernel producer": ["entry", "record here", "K part summed", "partials published"],
     "split_kernel consumer": ["entry", "record here", None, None, "loads issued", "wait over", "intermediate in LDS",
                               "wave 0 first spans stored", "wave 0 stores acknowledged", "all waves done"],
+    "sgmv_shrink_kernel": ["entry", "record here", "token rows requested", "first slab and x batch requested",
+                           "first piece of the slab on its way to LDS", "first slice multiplied", "partial sums issued",
+                           "partial sums acknowledged"],
+    # (the expand's stamps sit in columns 8.. of the same rows)
+    "sgmv_expand_kernel": ["entry", "records here", "token rows and first partial sums here", "intermediate in LDS",
+                           "wave 0 last item stored", "wave 0 stores acknowledged", "wave 0 first item stored"],
 }
 
 
@@ -257,10 +263,10 @@ def run_timeline(args) -> None:
     from nanovllm_voxcpm_amd import _hip
 
     device = "cuda:0"
-    layers, slots, _ = build_workload("decode", device, args.rank or None)
+    layers, slots, eff = build_workload(args.workload, device, args.rank or None, args.sequences)
     if args.hot_layers > 0:
         layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
-    step, launches = make_step(layers, slots, args.form, args.timeline)
+    step, launches = make_step(layers, slots, args.form, args.timeline, eff=None if args.no_rank_vector else eff)
     for _ in range(3):
         step()
     torch.cuda.synchronize()
@@ -272,18 +278,26 @@ def run_timeline(args) -> None:
     t = buf.cpu()
     rows = t[t[:, 1] != 0]  # workgroups that found a tile
     t0 = int(t[t[:, 0] != 0][:, 0].min())
-    out = {"timeline_of": args.timeline, "form": args.form, "workgroups_launched": int((t[:, 0] != 0).sum()),
-           "workgroups_with_work": int(rows.size(0)), "unit": "ns after the first workgroup entered", "kernels": {}}
-    if int((rows[:, 15] != 0).sum()) == 0:
+    out = {"timeline_of": args.timeline, "workload": args.workload, "form": args.form,
+           "workgroups_launched": int((t[:, 0] != 0).sum()), "workgroups_with_work": int(rows.size(0)),
+           "unit": "ns after the first workgroup of the kernel entered", "kernels": {}}
+    first = {}  # column of a group's first stamp when it is not column 0
+    if int((t[:, 8] != 0).sum()) > 0 and int((t[:, 15] != 0).sum()) == 0 and int((t[:, 9] != 0).sum()) > 0 and args.form != "fused":
+        groups = {"sgmv_shrink_kernel": rows, "sgmv_expand_kernel": t[t[:, 9] != 0]}
+        first["sgmv_expand_kernel"] = 8
+    elif int((rows[:, 15] != 0).sum()) == 0:
         groups = {"decode_kernel": rows}
     else:
         groups = {"split_kernel producer": rows[rows[:, 15] != 0], "split_kernel consumer": rows[rows[:, 15] == 0]}
     for name, g in groups.items():
         entry = {}
+        c0 = first.get(name, 0)
+        if c0:
+            t0 = int(t[t[:, c0] != 0][:, c0].min())
         for i, label in enumerate(STAMPS[name]):
             if label is None:
                 continue
-            col = g[:, i]
+            col = g[:, c0 + i]
             col = (col[col != 0] - t0) * 10
             if col.numel():
                 entry[label] = [int(col.min()), int(col.median()), int(col.max())]
@@ -617,7 +631,7 @@ def main() -> None:
                     help="diagnostic (mixed workload): do not tell the kernels the adapters' true ranks; the zero "
                          "padding of the rank-64 buffers is then read and multiplied like any other data")
     ap.add_argument("--timeline", default=None, choices=ORDER,
-                    help="diagnostic: in-kernel timeline of one projection's launch on the decode workload "
+                    help="diagnostic: in-kernel timeline of one projection's launch (decode, prefill or mixed workload) "
                          "(needs the trace build of the library)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "

@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   // A workgroup takes G consecutive 64-token tiles (consecutive tiles mostly belong to one slot,
   // whose B rows then stay in registers across them), or, past `big_units`, one short segment.
   const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  MLORA_STAMP(8);  // expand: first instruction
   const bool is_big = unit < big_units;
   const int sidx = is_big ? 0 : unit - big_units;
 
@@ -128,6 +129,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
   if (!usable) return;
+  MLORA_STAMP(9);  // expand: tile records here
 
   bool masked = false;
 #pragma unroll

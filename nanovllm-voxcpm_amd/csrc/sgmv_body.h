@@ -566,11 +566,25 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   for (int g = 0; g < G; ++g)
     if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = rowv[g];
   __syncthreads();
+  if constexpr (!SC1) MLORA_STAMP(10);  // expand: token rows (and the first partial sums) here
   first_step = next_step(-1);  // exists: some tile holds tokens
   int st = first_step;
+  auto advance = [&](int fc0, int fst, int& nc0, int& nst) {  // item after (fc0, fst); false when there is none
+    nst = next_step(fst);
+    nc0 = fc0;
+    if (nst >= STEPS) {
+      nst = first_step;
+      nc0 = fc0 + kExpandWaves * SPAN;
+    }
+    return nc0 < sp.n1;
+  };
+  int c1 = 0, st1 = 0;
+  bool more1 = false;
   if (has_work) {
     load_b(c0, s_slot[st / NB], s_eff[st / NB]);
     issue_y(ya, c0, st);
+    more1 = advance(c0, st, c1, st1);
+    if (more1) issue_y(yb, c1, st1);
   }
 
   // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
@@ -582,33 +596,31 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     stage_h(g);
   }
   __syncthreads();
+  if constexpr (!SC1) MLORA_STAMP(11);  // expand: intermediate in LDS
   if (!has_work) return;
 
-  // two y buffers, used in turn
-  auto advance = [&](int& nc0, int& nst) {  // item after (c0, st); false when there is none
-    nst = next_step(st);
-    nc0 = c0;
-    if (nst >= STEPS) {
-      nst = first_step;
-      nc0 = c0 + kExpandWaves * SPAN;
-    }
-    return nc0 < sp.n1;
-  };
-  for (;;) {
-    int nc0, nst;
-    bool more = advance(nc0, nst);
-    if (more) issue_y(yb, nc0, nst);
-    process(ya, c0, st);
-    if (!more) break;
-    c0 = nc0;
-    st = nst;
-    more = advance(nc0, nst);
-    if (more) issue_y(ya, nc0, nst);
-    process(yb, c0, st);
-    if (!more) break;
-    c0 = nc0;
-    st = nst;
+  // two y buffers, used in turn, both on their way whenever the wavefront has two more items
+  process(ya, c0, st);
+  if constexpr (!SC1) MLORA_STAMP(14);  // expand: wavefront 0 has stored its first item
+  for (bool again = false;; again = true) {
+    if (again) process(ya, c0, st);
+    if constexpr (!SC1) MLORA_STAMP(12);  // expand: wavefront 0 has stored an item (the last stamp taken stays)
+    if (!more1) break;
+    int c2, st2;
+    const bool more2 = advance(c1, st1, c2, st2);
+    if (more2) issue_y(ya, c2, st2);
+    process(yb, c1, st1);
+    if constexpr (!SC1) MLORA_STAMP(12);
+    if (!more2) break;
+    c0 = c2;
+    st = st2;
+    more1 = advance(c0, st, c1, st1);
+    if (more1) issue_y(yb, c1, st1);
   }
+#ifdef MLORA_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if constexpr (!SC1) MLORA_STAMP(13);  // expand: wavefront 0's stores acknowledged
+#endif
 }
 
 // The fp32 partials of the intermediate live behind the head of the workspace.
