@@ -356,7 +356,8 @@ def test_config3_prefill_bf16(name, form):
 
 
 @pytest.mark.parametrize("knobs", [{}, {"MLORA_SGMV_KSPLIT": "1", "MLORA_SGMV_GROUP": "2"}, {"MLORA_SGMV_KR": "128", "MLORA_SGMV_KSPLIT": "4", "MLORA_SGMV_GROUP": "4", "MLORA_SGMV_CPL": "4"},
-                                   {"MLORA_SGMV_ALL_SLICES": "2", "MLORA_SGMV_KR": "256", "MLORA_SGMV_NT": "512"}])
+                                   {"MLORA_SGMV_ALL_SLICES": "2", "MLORA_SGMV_KR": "256", "MLORA_SGMV_NT": "512"},
+                                   {"MLORA_SGMV_XDB": "0", "MLORA_SGMV_KSPLIT": "1"}])  # K parts of several one-slab batches
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rank", [8, 16, 32, 64])
 def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
