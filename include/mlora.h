@@ -209,7 +209,10 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
  * needs from one load: words {slot, token count, first position in sorted_idx, 0}, then 16
  * token indices (the tile's tokens in order; entries past the count repeat them cyclically, so
  * all sixteen name rows of the tile itself), then padding.
- * A big tile is four words {slot, first position in sorted_idx, token count, 0}. */
+ * A big tile is four words {slot, first position in sorted_idx, token count, 0}; behind the
+ * big-tile records lies one list of MLORA_TILE_BIG token indices per big tile (its tokens in
+ * order, repeated cyclically past the count), at a place that follows from the tile's number
+ * alone: a workgroup requests it together with the record. */
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
 #define MLORA_BIG_TILE_WORDS 4

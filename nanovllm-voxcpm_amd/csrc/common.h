@@ -154,10 +154,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---- plan workspace layout ------------------------------------------------------------
-// int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles
-// Small tiles are 32-word records (128-byte aligned), big tiles four words; see mlora.h.
+// int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles | big-tile rows
+// Small tiles are 32-word records (128-byte aligned), big tiles four words, their row lists 64 words; see mlora.h.
 struct PlanLayout {
-  int sorted_off, counts_off, offsets_off, small_off, big_off, cap_small, cap_big, total_words;
+  int sorted_off, counts_off, offsets_off, small_off, big_off, bigrows_off, cap_small, cap_big, total_words;
 };
 
 __host__ __device__ inline int round_up4(int v) { return (v + 3) & ~3; }
@@ -174,7 +174,8 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   p.cap_small = ((T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs + 7) & ~7;
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
   p.cap_big = (T / MLORA_TILE_BIG + segs + 31) & ~31;  // groups of up to four tiles, eight groups abreast
-  p.total_words = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;
+  p.bigrows_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;  // (a multiple of 32 words again)
+  p.total_words = p.bigrows_off + MLORA_TILE_BIG * p.cap_big;
   return p;
 }
 

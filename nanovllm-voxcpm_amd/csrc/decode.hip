@@ -97,20 +97,23 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   const int row = rec[MLORA_SMALL_TILE_ROWS + lr];
   const i32x4 rows4 = *reinterpret_cast<const i32x4*>(rec + MLORA_SMALL_TILE_ROWS + 4 * lg);  // tokens 4*lg .. 4*lg+3
   const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);       // slot, count, start, 0
-  const i32x4 hdr0 = *reinterpret_cast<const i32x4*>(plan);      // magic, T, L, ...
-  const i32x4 hdr1 = *reinterpret_cast<const i32x4*>(plan + 4);  // ..., short tiles
-  const i32x4 hdr2 = *reinterpret_cast<const i32x4*>(plan + 8);  // long small tiles, ...
+  typedef int i32x16 __attribute__((ext_vector_type(16)));
   const DecodeSplit sp = splits.split[split_id];
+  const i32x16 hdr = *reinterpret_cast<const i32x16*>(plan);  // the whole header in one scalar load
   const RankPrefetch ranks = rank_prefetch(MASKED ? eff_rank : nullptr, num_slots, lane);
+  // (everything above is requested before anything below is scheduled: left to itself the
+  // compiler requests this launch's column range only after the header has arrived)
+  __builtin_amdgcn_sched_barrier(0);
   const int slot = rec0[0], m = rec0[1];
-  const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
+  const int n_tiles = hdr[MLORA_PLAN_TILES_SHORT] + hdr[MLORA_PLAN_TILES_LONG_SMALL] * include_long;
   // One exit test, evaluated without short-circuit, that consumes everything fetched above
   // (the token index through its first lane), so that all of it is requested here, together,
   // instead of piece by piece behind a chain of branches.
-  const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
-                     int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) &
+  const int usable = int(hdr[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr[MLORA_PLAN_NUM_TOKENS] == T_) &
+                     int(hdr[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) &
                      int(slot < num_slots) & int(sp.n0 < sp.n1) & int(sp.a != nullptr) & int(sp.b != nullptr) &
-                     int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0);
+                     int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0) &
+                     int(__builtin_amdgcn_readfirstlane(rows4[0]) >= 0);
   if (!usable) return;
   MLORA_STAMP(1);  // tile record and plan header are here
 

@@ -41,12 +41,13 @@ template <typename T, int R, int KR, int XW, bool DB>
 __device__ __forceinline__ void fused_shrink_role(T* __restrict__ s_a, const int32_t* __restrict__ plan, const void* __restrict__ xv, float* __restrict__ hws, int64_t xs, int sorted_off,
                                                             int T_, int K, int num_slices, int krange, int all_slices, const ShrinkSlices& sl,
                                                             int slice0, int kpart, int slot, int start, int m, int eff) {
+  // token row of this lane (positions past the end of the tile repeat its last token)
+  const int ti = (threadIdx.x / kWave) * 16 + (threadIdx.x & 15);
+  const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
   if (R > 16 && ((eff + 15) >> 4) < (R + 15) / 16)
-    shrink_body<T, R, KR, XW, DB, true, false>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, slot,
-                                               start, m, eff);
+    shrink_body<T, R, KR, XW, DB, true, false>(s_a, xv, hws, xs, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, slot, start, m, eff, row);
   else
-    shrink_body<T, R, KR, XW, DB, false, false>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, slot,
-                                                start, m, eff);
+    shrink_body<T, R, KR, XW, DB, false, false>(s_a, xv, hws, xs, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, slot, start, m, eff, row);
 }
 
 // The same for the roles a workgroup computes because their seals did not arrive: the exception, so
@@ -62,20 +63,23 @@ template <typename T, int R, int CPL, int TPF, int G>
 __device__ __forceinline__ void fused_expand(T* s_h, int* s_row, int* s_slot, int* s_m, int* s_eff, const int* s_start,
                                                        const int32_t* plan, const float* hws, void* yv_, int64_t ys, int sorted_off, int T_,
                                                        int num_slices, int ksplit, float scaling, int nt, const ExpandSplit& sp) {
-  int slot[G], start[G], m[G], eff[G];
+  int slot[G], start[G], m[G], eff[G], rowv[G];
   bool masked = false;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     slot[g] = s_slot[g]; start[g] = s_start[g]; m[g] = s_m[g]; eff[g] = s_eff[g];
     masked |= m[g] > 0 && eff[g] < R;
+    // token row at position tid of the tile (positions past its end repeat its last token)
+    const int tid = threadIdx.x;
+    rowv[g] = (m[g] > 0 && tid < MLORA_TILE_BIG) ? plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)] : 0;
   }
   __syncthreads();  // expand_body rewrites the arrays read above
   if (masked)
-    expand_body<T, R, CPL, TPF, G, true, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
-                                               sp, slot, start, m, eff);
+    expand_body<T, R, CPL, TPF, G, true, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+                                               m, eff, rowv);
   else
-    expand_body<T, R, CPL, TPF, G, false, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
-                                                sp, slot, start, m, eff);
+    expand_body<T, R, CPL, TPF, G, false, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+                                                m, eff, rowv);
 }
 
 template <typename T, int R, int KR, int XW, bool DB, int CPL, int TPF, int G>

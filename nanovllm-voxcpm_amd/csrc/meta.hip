@@ -266,6 +266,13 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
           const int n = left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL;
           for (int pos = r % MLORA_TILE_SMALL; pos < MLORA_TILE_SMALL; pos += n)
             p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + pos] = t;
+          if (c >= MLORA_SEGMENT_THRESHOLD) {
+            // the same for the row list of the segment's 64-token tile
+            const int qb = ts_big[key] + r / MLORA_TILE_BIG;
+            const int leftb = c - (r / MLORA_TILE_BIG) * MLORA_TILE_BIG;
+            const int nb = leftb < MLORA_TILE_BIG ? leftb : MLORA_TILE_BIG;
+            for (int pos = r % MLORA_TILE_BIG; pos < MLORA_TILE_BIG; pos += nb) p.plan[lay.bigrows_off + qb * MLORA_TILE_BIG + pos] = t;
+          }
         }
         if (p.sorted_idx) p.sorted_idx[n_neg + off[key] + r] = t;
       } else if (p.sorted_idx) {

@@ -40,7 +40,7 @@ namespace {
 template <typename T, int R, int KR, int XW, bool DB>
 __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                                              float* __restrict__ hws, int64_t xs, int big_off,
-                                                                             int small_off, int big_cap, int sorted_off, int T_, int K,
+                                                                             int small_off, int big_cap, int bigrows_off, int T_, int K,
                                                                              int num_slots, int num_slices, int ksplit, int krange,
                                                                              int all_slices, const int32_t* __restrict__ eff_rank, ShrinkSlices sl) {
   constexpr int ASTRIDE = KR + 8;  // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -50,6 +50,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
   const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
   MLORA_STAMP(0);  // first instruction
+  const int row = tile_row(plan, bigrows_off, small_off, big_cap, tile, (threadIdx.x / kWave) * 16 + (threadIdx.x & 15));
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
   if (!tr.ok) return;
   MLORA_STAMP(1);  // tile record here
@@ -61,11 +62,11 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
     if (eff == 0) return;
   }
   if (R > 16 && ((eff + 15) >> 4) < (R + 15) / 16)
-    shrink_body<T, R, KR, XW, DB, true>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart,
-                                        tr.slot, tr.start, tr.m, eff);
+    shrink_body<T, R, KR, XW, DB, true>(s_a, xv, hws, xs, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, tr.slot, tr.start, tr.m,
+                                        eff, row);
   else
-    shrink_body<T, R, KR, XW, DB, false>(s_a, plan, xv, hws, xs, sorted_off, T_, K, num_slices, krange, all_slices, sl, slice0, kpart,
-                                         tr.slot, tr.start, tr.m, eff);
+    shrink_body<T, R, KR, XW, DB, false>(s_a, xv, hws, xs, T_, K, num_slices, krange, all_slices, sl, slice0, kpart, tr.slot, tr.start, tr.m,
+                                         eff, row);
 #ifdef MLORA_TRACE
   MLORA_STAMP(6);  // partial sums issued
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
 template <typename T, int R, int CPL, int TPF, int G>
 __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                                                              void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
-                                                                             int big_units, int sorted_off, int T_, int num_slots,
+                                                                             int big_units, int bigrows_off, int T_, int num_slots,
                                                                              int num_slices, int ksplit, float scaling, int nt,
                                                                              const int32_t* __restrict__ eff_rank, ExpandSplits splits) {
   constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
@@ -102,6 +103,17 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   i32x4 big[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) big[g] = reinterpret_cast<const i32x4*>(plan + big_off)[is_big ? unit * G + g : 0];
+  // the token rows of the tiles: where they lie follows from the unit's number, so they are
+  // requested here, with the records (threads 0..63 hold one position of every tile each)
+  int rowv[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    rowv[g] = 0;
+    if (tid < MLORA_TILE_BIG) {
+      if (is_big) rowv[g] = plan[bigrows_off + (unit * G + g) * MLORA_TILE_BIG + tid];
+      else if (g == 0) rowv[g] = plan[small_off + sidx * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (tid & (MLORA_TILE_SMALL - 1))];
+    }
+  }
   const ExpandSplit sp = splits.split[blockIdx.y];
   const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
   int slot[G], start[G], m[G], any = 0;
@@ -135,11 +147,11 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
 #pragma unroll
   for (int g = 0; g < G; ++g) masked |= m[g] > 0 && eff[g] < R;
   if (masked)
-    expand_body<T, R, CPL, TPF, G, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
-                                         sp, slot, start, m, eff);
+    expand_body<T, R, CPL, TPF, G, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+                                         m, eff, rowv);
   else
-    expand_body<T, R, CPL, TPF, G, false>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt,
-                                          sp, slot, start, m, eff);
+    expand_body<T, R, CPL, TPF, G, false>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+                                          m, eff, rowv);
 }
 
 struct ShrinkLaunch {
@@ -157,7 +169,7 @@ void launch_shrink_one(const ShrinkLaunch& l) {
   dim3 grid(8, static_cast<unsigned>(l.all_slices ? l.ksplit : a->num_slices * l.ksplit), static_cast<unsigned>(l.tiles8));
   hipLaunchKernelGGL((sgmv_shrink_kernel<T, R, KR, XW, DB>), grid, dim3(kShrinkWaves * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, partials_of(a), a->x_stride, l.lay.big_off, l.lay.small_off, l.big_cap,
-                     l.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, a->effective_rank, l.sl);
+                     l.lay.bigrows_off, a->num_tokens, a->k, a->num_slots, a->num_slices, l.ksplit, l.krange, l.all_slices, a->effective_rank, l.sl);
 }
 
 // (slab width, x batch width): 128/128 and 256/256 with two x buffers, 256/512 and 512/512 with one
@@ -187,7 +199,7 @@ void launch_expand_group(const MloraAddArgs* a, const PlanLayout& lay, int big_u
   const int nt = sgmv_knobs().nt_hint;
 #define MLORA_EXPAND(CPL_, TPF_, G_)                                                                                       \
   hipLaunchKernelGGL((sgmv_expand_kernel<T, R, CPL_, TPF_, G_>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, \
-                     a->y_stride, lay.big_off, lay.small_off, big_units, lay.sorted_off, a->num_tokens, a->num_slots,      \
+                     a->y_stride, lay.big_off, lay.small_off, big_units, lay.bigrows_off, a->num_tokens, a->num_slots,      \
                      a->num_slices, ksplit, a->scaling, nt, a->effective_rank, sp)
   if (cpl == 4) {
     if (group == 4) MLORA_EXPAND(4, 4, 4); else if (group == 2) MLORA_EXPAND(4, 4, 2); else MLORA_EXPAND(4, 4, 1);

@@ -58,6 +58,17 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
   return t;
 }
 
+// Token row at position `ti` of tile `tile`.  Where it lies follows from the tile's number alone (a
+// 64-token tile has its row list behind the big-tile records, a short segment carries its rows in
+// its record), so it is requested together with the record instead of after it.  Positions past
+// the tile's count hold rows of the tile as well (a valid row to read, never written).
+__device__ __forceinline__ int tile_row(const int32_t* __restrict__ plan, int bigrows_off, int small_off, int big_cap, int tile, int ti) {
+  const bool is_big = tile < big_cap;
+  const int at = is_big ? bigrows_off + tile * MLORA_TILE_BIG + ti
+                        : small_off + (tile - big_cap) * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + (ti & (MLORA_TILE_SMALL - 1));
+  return plan[at];
+}
+
 // ---- shrink -------------------------------------------------------------------------------------
 // grid (8, slices * K parts, tiles / 8), four wavefronts of sixteen tokens each.  The workgroup's
 // K part is walked in x batches of XW columns (a wavefront holds the batch of its sixteen token
@@ -77,9 +88,9 @@ constexpr int kShrinkWaves = 4;
 // SC1: the partial sums leave with agent-scope stores (they pass the compute unit's and the XCD's
 // caches on their way), for readers in other workgroups of the same launch.
 template <typename T, int R, int KR, int XW, bool DB, bool MASKED, bool SC1 = false>
-__device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* __restrict__ plan, const void* __restrict__ xv,
-                                            float* __restrict__ hws, int64_t xs, int sorted_off, int T_, int K, int num_slices, int krange,
-                                            int all_slices, const ShrinkSlices& sl, int slice0, int kpart, int slot, int start, int m, int eff) {
+__device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __restrict__ xv, float* __restrict__ hws, int64_t xs, int T_, int K,
+                                            int num_slices, int krange, int all_slices, const ShrinkSlices& sl, int slice0, int kpart, int slot,
+                                            int start, int m, int eff, int row) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -100,11 +111,11 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const int32_t* 
   const int k0 = kpart * krange;
   const int nbatch = krange / XW;
   const bool active = wave * 16 < m;  // this wavefront's token block exists
-  // token row of this lane (lanes past the end of the tile repeat its last token: they feed the
-  // MFMA harmlessly and are never written back)
+  // `row`: token row of this lane, position wave * 16 + lane % 16 of the tile (positions past the
+  // end of the tile name rows of the tile too: they feed the MFMA harmlessly and are never
+  // written back)
   const int ti = wave * 16 + lr;
-  const int row = plan[sorted_off + start + (ti < m ? ti : m - 1)];
-  MLORA_STAMP(2);  // shrink: token rows requested
+  MLORA_STAMP(2);  // shrink: body entered (the token rows were requested with the record)
   const T* xptr = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + k0 + lg * 8;
   const int64_t aoff = static_cast<int64_t>(slot) * R * K + k0;
 
@@ -320,23 +331,26 @@ template <int N> struct YRaw;
 template <> struct YRaw<4> { typedef u32x2 type; };
 template <> struct YRaw<8> { typedef u32x4 type; };
 
-// y is touched once per launch: with `nt` it is moved with the non-temporal hint so that it does
-// not push the B rows, which every tile of a slot re-reads, out of the L2.
+// y is touched once per launch (a non-temporal hint on its accesses measured no gain).  An item
+// stays the raw vectors it was fetched as until it is used: unpacked where it is requested, its
+// arithmetic is scheduled ahead of the barrier that ends the staging of the intermediate, and the
+// wavefront waits for the item in front of work that could have run meanwhile.
 template <typename T, int N>
-__device__ __forceinline__ YVec<T, N> load_y(const T* p, int nt) {
-  typedef typename YRaw<N>::type Raw;
+__device__ __forceinline__ typename YRaw<N>::type load_y(const T* p) {
+  return *reinterpret_cast<const typename YRaw<N>::type*>(p);
+}
+template <typename T, int N>
+__device__ __forceinline__ YVec<T, N> unpack_y(const typename YRaw<N>::type& r) {
   YVec<T, N> v;
-  Raw r = nt ? __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p)) : *reinterpret_cast<const Raw*>(p);
   __builtin_memcpy(&v, &r, sizeof(r));
   return v;
 }
 template <typename T, int N>
-__device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
+__device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v) {
   typedef typename YRaw<N>::type Raw;
   Raw r;
   __builtin_memcpy(&r, &v, sizeof(r));
-  if (nt) __builtin_nontemporal_store(r, reinterpret_cast<Raw*>(p));
-  else *reinterpret_cast<Raw*>(p) = r;
+  *reinterpret_cast<Raw*>(p) = r;
 }
 
 // Body of the expand for the tiles of one workgroup.  MASKED: some tile's slot holds an adapter of
@@ -350,9 +364,9 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v, int nt) {
 template <typename T, int R, int CPL, int TPF, int G, bool MASKED, bool SC1 = false>
 __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict__ s_row, int* __restrict__ s_slot, int* __restrict__ s_m,
                                             int* __restrict__ s_eff, const int32_t* __restrict__ plan, const float* __restrict__ hws,
-                                            void* __restrict__ yv_, int64_t ys, int sorted_off, int T_, int num_slices, int ksplit,
+                                            void* __restrict__ yv_, int64_t ys, int T_, int num_slices, int ksplit,
                                             float scaling, int nt, const ExpandSplit& sp, const int (&slot)[G], const int (&start)[G],
-                                            const int (&m)[G], const int (&eff)[G]) {
+                                            const int (&m)[G], const int (&eff)[G], const int (&rowv)[G]) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int NB = TB / TPF;           // y batches per tile
   constexpr int STEPS = G * NB;          // (tile, batch) steps of a span
@@ -449,13 +463,14 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     const int c = c0 + CPL * lr;
     return c < sp.n1 ? c : sp.n1 - 8;
   };
-  auto issue_y = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+  typedef typename YRaw<CPL>::type YItem[TPF][4];  // a y item as it was fetched: 16 * TPF tokens x 16 * CPL columns of a wavefront
+  auto issue_y = [&](YItem& buf, int c0, int st) {
     const int g = st / NB, tp = (st % NB) * TPF, cl = column(c0);
 #pragma unroll
     for (int u = 0; u < TPF; ++u) {
       const i32x4 rows = *reinterpret_cast<const i32x4*>(&s_row[g * MLORA_TILE_BIG + (tp + u) * 16 + 4 * lg]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) buf[u][i] = load_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + cl, nt);
+      for (int i = 0; i < 4; ++i) buf[u][i] = load_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + cl);
     }
   };
   Pack8 bop[CPL][KSTEPS];
@@ -498,10 +513,9 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     b_slot = sg;
     b_c0 = c0;
   };
-  auto process = [&](YVec<T, CPL>(&buf)[TPF][4], int c0, int st) {
+  auto process = [&](YItem& buf, int c0, int st) {
     const int g = st / NB, tp = (st % NB) * TPF;
-    const int mg = s_m[g], sg = s_slot[g];
-    if (sg != b_slot || c0 != b_c0) load_b(c0, sg, s_eff[g]);
+    const int mg = s_m[g];
     const T* hg = s_h + g * MLORA_TILE_BIG * HSTRIDE;
     const int c = c0 + CPL * lr;
     const bool col_ok = c < sp.n1;
@@ -536,35 +550,32 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (col_ok && tb * 16 + 4 * lg + i < mg) {
+          const YVec<T, CPL> yv = unpack_y<T, CPL>(buf[u][i]);
           YVec<T, CPL> r;
 #pragma unroll
-          for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(buf[u][i].e[j]) + out[j][i]);
-          store_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + c, r, nt);
+          for (int j = 0; j < CPL; ++j) r.e[j] = from_f32<T>(to_f32(yv.e[j]) + out[j][i]);
+          store_y<T, CPL>(ybase + static_cast<int64_t>(rows[i]) * ys + c, r);
         }
       }
     }
   };
 
-  YVec<T, CPL> ya[TPF][4], yb[TPF][4];
+  YItem ya, yb;
   int c0 = sp.n0 + wave * SPAN;
   const bool has_work = c0 < sp.n1;
 
-  // The token rows go out first: they are what the y rows wait for.  Entries of the row list past
-  // the end of a tile repeat its last token (a valid row to read, never written).  The partial
-  // sums of the first tile hang on the tile record alone and are on their way meanwhile (the B
-  // rows of the first span could be too, but they are 16 KB per wavefront and hold the token
-  // rows up: the prefill step 3748 -> 3858 us).
-  int rowv[G];
+  // `rowv[g]` (threads 0..63): token row at position tid of tile g, requested by the caller
+  // together with the tile records.  Entries past the end of a tile name rows of the tile too (a
+  // valid row to read, never written).  The partial sums of the first tile hang on the tile
+  // record alone; they are requested before the barrier the rows pass through, so that they and
+  // the y rows are on their way together.  (The B rows of the first span could go out there too,
+  // but they are 16 KB per wavefront and hold everything behind them up: prefill 3748 -> 3858 us.)
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
-    rowv[g] = 0;
-    if (m[g] > 0 && tid < MLORA_TILE_BIG) rowv[g] = plan[sorted_off + start[g] + (tid < m[g] ? tid : m[g] - 1)];
+    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = rowv[g];
   }
   if (m[0] > 0) request_h(0);
-#pragma unroll
-  for (int g = 0; g < G; ++g)
-    if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = rowv[g];
   __syncthreads();
   if constexpr (!SC1) MLORA_STAMP(10);  // expand: token rows (and the first partial sums) here
   first_step = next_step(-1);  // exists: some tile holds tokens
@@ -578,44 +589,86 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     }
     return nc0 < sp.n1;
   };
-  int c1 = 0, st1 = 0;
-  bool more1 = false;
-  if (has_work) {
-    load_b(c0, s_slot[st / NB], s_eff[st / NB]);
-    issue_y(ya, c0, st);
-    more1 = advance(c0, st, c1, st1);
-    if (more1) issue_y(yb, c1, st1);
-  }
-
   // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
   // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
+  auto stage_all = [&]() {
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    if (m[g] == 0) continue;
-    if (g > 0) request_h(g);
-    stage_h(g);
+    for (int g = 0; g < G; ++g) {
+      if (m[g] == 0) continue;
+      if (g > 0) request_h(g);
+      stage_h(g);
+    }
+  };
+  // the B rows of an item's span and slot, if the registers do not hold them already
+  auto ensure_b = [&](int c0, int st) {
+    const int g = st / NB, sg = s_slot[g];
+    if (sg != b_slot || c0 != b_c0) load_b(c0, sg, s_eff[g]);
+  };
+  // The B rows and the first two y items go out, then the intermediate is staged while they are
+  // on their way.  The staging is written out once per path (no work / one item / two items) so
+  // that each is straight-line code from the requests to the staging: the compiler then waits for
+  // the partial sums alone, not for everything requested after them.
+  // (Every path passes the one barrier that ends the staging in its own copy: a wavefront counts
+  // at the barrier wherever its program counter is.  The markers keep the compiler from merging
+  // the ends of the copies into one block, where it would have to wait for every load again.)
+  if (!has_work) {
+    stage_all();
+    asm volatile("; staged, no item" ::: "memory");
+    __syncthreads();
+    if constexpr (!SC1) MLORA_STAMP(11);  // expand: intermediate in LDS
+    return;
   }
-  __syncthreads();
-  if constexpr (!SC1) MLORA_STAMP(11);  // expand: intermediate in LDS
-  if (!has_work) return;
-
-  // two y buffers, used in turn, both on their way whenever the wavefront has two more items
-  process(ya, c0, st);
-  if constexpr (!SC1) MLORA_STAMP(14);  // expand: wavefront 0 has stored its first item
-  for (bool again = false;; again = true) {
-    if (again) process(ya, c0, st);
+  int c1 = 0, st1 = 0;
+  load_b(c0, s_slot[st / NB], s_eff[st / NB]);
+  issue_y(ya, c0, st);
+  if (!advance(c0, st, c1, st1)) {
+    stage_all();
+    asm volatile("; staged behind one item" ::: "memory");
+    __syncthreads();
+    if constexpr (!SC1) MLORA_STAMP(11);
+    process(ya, c0, st);
+    if constexpr (!SC1) MLORA_STAMP(14);  // expand: wavefront 0 has stored its first item
     if constexpr (!SC1) MLORA_STAMP(12);  // expand: wavefront 0 has stored an item (the last stamp taken stays)
-    if (!more1) break;
-    int c2, st2;
-    const bool more2 = advance(c1, st1, c2, st2);
-    if (more2) issue_y(ya, c2, st2);
-    process(yb, c1, st1);
+  } else {
+    issue_y(yb, c1, st1);
+    stage_all();
+    asm volatile("; staged behind two items" ::: "memory");
+    __syncthreads();
+    if constexpr (!SC1) MLORA_STAMP(11);
+    // Two y buffers, used in turn, both on their way whenever the wavefront has two more items.
+    // The order inside the loop is what lets the compiler count the loads in flight instead of
+    // waiting for all of them: an item's B rows are looked after (a reload only when span or slot
+    // change, behind a branch) BEFORE the item after it is requested, so whatever waits for B
+    // rows or for a y item knows how many requests are younger; the paths that run out of items
+    // leave the loop where they find out, with their own copy of the last step.
+    process(ya, c0, st);
+    if constexpr (!SC1) MLORA_STAMP(14);
     if constexpr (!SC1) MLORA_STAMP(12);
-    if (!more2) break;
-    c0 = c2;
-    st = st2;
-    more1 = advance(c0, st, c1, st1);
-    if (more1) issue_y(yb, c1, st1);
+    for (;;) {
+      // here: (c1, st1) is on its way in yb; ya is free
+      int c2, st2;
+      const bool more2 = advance(c1, st1, c2, st2);
+      ensure_b(c1, st1);
+      if (!more2) {
+        process(yb, c1, st1);
+        if constexpr (!SC1) MLORA_STAMP(12);
+        break;
+      }
+      issue_y(ya, c2, st2);
+      process(yb, c1, st1);
+      if constexpr (!SC1) MLORA_STAMP(12);
+      // here: (c2, st2) is on its way in ya; yb is free
+      const bool more3 = advance(c2, st2, c1, st1);
+      ensure_b(c2, st2);
+      if (!more3) {
+        process(ya, c2, st2);
+        if constexpr (!SC1) MLORA_STAMP(12);
+        break;
+      }
+      issue_y(yb, c1, st1);
+      process(ya, c2, st2);
+      if constexpr (!SC1) MLORA_STAMP(12);
+    }
   }
 #ifdef MLORA_TRACE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -860,7 +860,9 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     small_off = (offsets_off + r4(L + 2) + 31) & ~31
     cap_small = ((T + 15) // 16 + min(L, T) + 7) & ~7
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
-    assert len(ws) == big_off + 4 * ((T // 64 + min(L, T) + 31) & ~31)
+    cap_big = (T // 64 + min(L, T) + 31) & ~31
+    bigrows_off = big_off + 4 * cap_big
+    assert len(ws) == bigrows_off + 64 * cap_big
     assert ws[sorted_off : sorted_off + len(s)] == s
     dense = [0] * (L + 1)
     for slot, n in zip(a, c):
@@ -873,6 +875,9 @@ def test_metadata_bit_exact_random(T, L, p_neg):
         own = s[start : start + count]
         assert rec[4:20] == [own[j % count] for j in range(16)] and rec[20:] == [0] * 12  # cyclic repeats past the count
     assert [tuple(ws[big_off + 4 * i : big_off + 4 * i + 3]) for i in range(len(long_big))] == long_big
+    for q, (slot, start, count) in enumerate(long_big):  # the tile's tokens, repeated cyclically past its count
+        own = s[start : start + count]
+        assert ws[bigrows_off + 64 * q : bigrows_off + 64 * (q + 1)] == [own[j % count] for j in range(64)]
 
 
 def test_metadata_flags_bad_slot_ids():
