@@ -208,10 +208,14 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
   for (int s = 0; s < kSpansAhead; ++s) {
     const int c0 = sp.n0 + (wave + s * kNW) * 64;
-    if (c0 < sp.n1) {
-      if constexpr (TR) {
-        load_span_tr(c0, bop[s], yq[s]);
-      } else {
+    if constexpr (TR) {
+      // requested whether the span exists or not (the addresses of one that does not are clamped
+      // into the range: a cache line or two, never stored): values that are requested in a branch
+      // and used in a later one are unpacked by the compiler where they are requested, and the
+      // wavefront then waits for them before it has requested anything else
+      load_span_tr(c0, bop[s], yq[s]);
+    } else if (c0 < sp.n1) {
+      {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           int n = c0 + 16 * (lr >> 2) + 4 * j + (lr & 3);
@@ -400,6 +404,11 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
       }
     }
     const int c = c0 + 4 * lr;
+    // (the y values are taken as they are only here: left to itself the compiler unpacks them
+    // where they were requested, and the wavefront then waits for their arrival before it has
+    // requested its other spans and before the shrink)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(yy[i].x), "+v"(yy[i].y));
     if (c < sp.n1) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {

@@ -2,6 +2,8 @@
 // shrink of one (tile, slices, K part) and the expand of one (group of tiles, column range) as
 // device functions, and the host-side helpers both launchers use.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
 
@@ -255,13 +257,19 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
     return;
   }
 
+  // (Written once for wavefronts whose token block exists and once for those without one, which
+  // only help with the slabs: a branch on `active` around the x requests keeps the compiler from
+  // counting the loads in flight, and the wait for a slab then is a wait for the x batch requested
+  // after it as well.)
+  auto batches = [&](auto act_tag) {
+  constexpr bool ACT = decltype(act_tag)::value;
   Pack8 xa[XK], xb[DB ? XK : 1];
   f32x4 acc[RB];
   bool first = true;
   // One x batch: `cur` holds it (or is about to), `nxt` receives the following one meanwhile.
   auto run_batch = [&](Pack8(&cur)[XK], Pack8(&nxt)[XK], int si, int b) {
     const T* A = static_cast<const T*>(sl.a[slice0 + si]) + aoff;
-    if (DB && active && b + 1 < nbatch) request_x(nxt, (b + 1) * XW);
+    if (DB && ACT && b + 1 < nbatch) request_x(nxt, (b + 1) * XW);
 #pragma unroll
     for (int s = 0; s < SPB; ++s) {
       if (!first) __syncthreads();  // everyone is done reading the previous slab
@@ -273,7 +281,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
       if (s + 1 < SPB) request_slab(A + b * XW + (s + 1) * KR);
       else if (b + 1 < nbatch) request_slab(A + (b + 1) * XW);
       else if (si + 1 < nsl) request_slab(static_cast<const T*>(sl.a[slice0 + si + 1]) + aoff);
-      if (active) {
+      if (ACT) {
 #pragma unroll
         for (int i = 0; i < KS; ++i) {
 #pragma unroll
@@ -289,26 +297,69 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
         }
       }
     }
-    if (!DB && active && b + 1 < nbatch) request_x(cur, (b + 1) * XW);
+    if (!DB && ACT && b + 1 < nbatch) request_x(cur, (b + 1) * XW);
   };
 
   request_slab(static_cast<const T*>(sl.a[slice0]) + aoff);
-  if (active) request_x(xa, 0);
+  if (ACT) request_x(xa, 0);
   MLORA_STAMP(3);  // shrink: first slab and first x batch requested (the token rows are here)
   for (int si = 0; si < nsl; ++si) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
     if constexpr (DB) {
-      for (int b = 0; b < nbatch; b += 2) {
-        run_batch(xa, xb, si, b);
-        if (b + 1 < nbatch) run_batch(xb, xa, si, b + 1);
+      // Two x buffers, one slab per batch.  A batch that has a successor (MORE) requests the
+      // successor's x batch, waits for its own slab alone, and requests the successor's slab
+      // after the barrier; the last batch of the K part is a copy of its own without those
+      // requests.  Written that way (instead of tests on b inside one body) every wait counts
+      // the requests younger than what it waits for: the x batch that was just requested stays
+      // in flight while the current one is multiplied.
+      auto batch = [&](auto more_tag, Pack8(&cur)[XK], Pack8(&nxt)[XK], int b) __attribute__((always_inline)) {
+        constexpr bool MORE = decltype(more_tag)::value;
+        static_assert(SPB == 1, "one slab per batch");
+        const T* A = static_cast<const T*>(sl.a[slice0 + si]) + aoff;
+        if (MORE && ACT) request_x(nxt, (b + 1) * XW);
+        __syncthreads();  // everyone is done reading the previous slab
+        store_slab();
+        if (b == 0 && si == 0) MLORA_STAMP(4);  // shrink: first slab arrived and is on its way to LDS
+        __syncthreads();
+        if constexpr (MORE) request_slab(A + (b + 1) * XW);
+        else if (si + 1 < nsl) request_slab(static_cast<const T*>(sl.a[slice0 + si + 1]) + aoff);
+        if (ACT) {
+#pragma unroll
+          for (int i = 0; i < KS; ++i) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+              if constexpr (MASKED) {
+                if (rb >= rb_n) continue;
+              }
+              const int rr = rb * 16 + lr;
+              Pack8 aw;
+              aw.raw = *reinterpret_cast<const i32x4*>(&s_a[(rr < R ? rr : R - 1) * ASTRIDE + i * 32 + lg * 8]);
+              acc[rb] = Mma<T>::run(aw, cur[i], acc[rb]);
+            }
+          }
+        }
+      };
+      int b = 0;
+      for (; b + 2 < nbatch; b += 2) {
+        batch(std::true_type{}, xa, xb, b);
+        batch(std::true_type{}, xb, xa, b + 1);
+      }
+      if (b + 1 < nbatch) {
+        batch(std::true_type{}, xa, xb, b);
+        batch(std::false_type{}, xb, xa, b + 1);
+      } else {
+        batch(std::false_type{}, xa, xb, b);
       }
     } else {
       for (int b = 0; b < nbatch; ++b) run_batch(xa, xa, si, b);
     }
     if (si == 0) MLORA_STAMP(5);  // shrink: first slice multiplied
-    write_partials(acc, si);
+    if (ACT) write_partials(acc, si);
   }
+  };
+  if (active) batches(std::true_type{});
+  else batches(std::false_type{});
 }
 
 // ---- expand -------------------------------------------------------------------------------------
