@@ -113,21 +113,21 @@ const ApiKnobs& knobs() {
 
 // Where the one-launch form over 16-token tiles stops paying.  Its cost per token grows with the
 // rank (every tile fetches A[slot] and B[slot] again, every column range repeats its tile's shrink)
-// while a two-launch call pays 11.6 us before it moves any data (3.5 us for one launch over small
-// tiles).  Measured per projection shape on prefill batches of 1011..9392 tokens (1..16 sequences,
-// up to 8 adapters), the two forms meet where tokens x width reaches about 1.4e7 at rank 64 and
-// 2.4e7 at rank 32, with width = slices x K x max(1, K / 2048) + columns x max(1, columns / 4096):
-// long K and wide outputs cost the small tiles more than their share (tokens at the
-// crossing, rank 64 / rank 32: qkv 5000 / 6500, o 8500 / 11000, gate_up 1000 / 1300, down
-// 1200 / 2100).  At rank 16 and below only gate_up crosses before 16384 tokens (at 8200).
+// while a two-launch call pays about 10 us before it moves any data (3.5 us for one launch over
+// small tiles).  Measured per projection shape on prefill batches of 1011..9392 tokens (1..16
+// sequences, up to 8 adapters), the two forms meet where tokens x width reaches about 1.7e7 at
+// rank 64, 2.6e7 at rank 32 and 8.3e7 at rank 16, with width = slices x K x max(1, K / 1024) +
+// columns x max(1, columns / 4096): long K and wide outputs cost the small tiles more than their
+// share (tokens at the crossing, rank 64 / 32 / 16: qkv 4000 / 6000 / 19000, o 8300 / 12700 / -,
+// gate_up 900 / 1400 / 4500, down 1000 / 1500 / 4800).
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
 static bool small_batch(const MloraAddArgs* a) {
   const int fixed = knobs().small_batch_tokens;
   if (fixed > 0) return a->num_tokens <= fixed;
   double cols = 0;
   for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
-  const double width = static_cast<double>(a->num_slices) * a->k * (a->k > 2048 ? a->k / 2048.0 : 1.0) + cols * (cols > 4096 ? cols / 4096.0 : 1.0);
-  const double limit = a->r <= 16 ? 1.5e8 : a->r <= 32 ? 2.4e7 : 1.4e7;
+  const double width = static_cast<double>(a->num_slices) * a->k * (a->k > 1024 ? a->k / 1024.0 : 1.0) + cols * (cols > 4096 ? cols / 4096.0 : 1.0);
+  const double limit = a->r <= 16 ? 8.3e7 : a->r <= 32 ? 2.6e7 : 1.7e7;
   return a->num_tokens * width <= limit;
 }
 
