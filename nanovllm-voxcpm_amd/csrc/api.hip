@@ -115,11 +115,13 @@ const ApiKnobs& knobs() {
 // rank (every tile fetches A[slot] and B[slot] again, every column range repeats its tile's shrink)
 // while a two-launch call pays about 10 us before it moves any data (3.5 us for one launch over
 // small tiles).  Measured per projection shape on prefill batches of 1011..9392 tokens (1..16
-// sequences, up to 8 adapters), the two forms meet where tokens x width reaches about 1.7e7 at
-// rank 64, 2.6e7 at rank 32 and 8.3e7 at rank 16, with width = slices x K x max(1, K / 1024) +
+// sequences, up to 8 adapters), the two forms meet where tokens x width reaches about 1.5e7-1.7e7
+// at rank 64, 2.6e7 at rank 32 and 8.3e7 at rank 16, with width = slices x K x max(1, K / 1024) +
 // columns x max(1, columns / 4096): long K and wide outputs cost the small tiles more than their
 // share (tokens at the crossing, rank 64 / 32 / 16: qkv 4000 / 6000 / 19000, o 8300 / 12700 / -,
 // gate_up 900 / 1400 / 4500, down 1000 / 1500 / 4800).
+// The rank-64 limit is 1.5e7: with many adapters in the batch the small tiles lose earlier (the
+// mixed batch, 8192 tokens and 128 adapters: o 28.8 us per call on small tiles, 23.0 in two launches).
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
 static bool small_batch(const MloraAddArgs* a) {
   const int fixed = knobs().small_batch_tokens;
@@ -127,7 +129,7 @@ static bool small_batch(const MloraAddArgs* a) {
   double cols = 0;
   for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
   const double width = static_cast<double>(a->num_slices) * a->k * (a->k > 1024 ? a->k / 1024.0 : 1.0) + cols * (cols > 4096 ? cols / 4096.0 : 1.0);
-  const double limit = a->r <= 16 ? 8.3e7 : a->r <= 32 ? 2.6e7 : 1.7e7;
+  const double limit = a->r <= 16 ? 8.3e7 : a->r <= 32 ? 2.6e7 : 1.5e7;
   return a->num_tokens * width <= limit;
 }
 
