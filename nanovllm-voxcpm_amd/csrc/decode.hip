@@ -186,7 +186,6 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         int n = c0 + 32 * h + (lane >> 1);
         n = n < sp.n1 ? n : sp.n1 - 1;
         bo[h][0].raw = load128(B + static_cast<int64_t>(n) * R + (lane & 1) * 8);
-        if (MASKED && eff < R) mask_ranks(bo[h][0], (lane & 1) * 8, eff);
       }
     } else {
 #pragma unroll
@@ -197,7 +196,6 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-          if (MASKED && eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
     }
@@ -226,7 +224,6 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
             // zero, and an unconditional load keeps the whole batch of loads in flight together
             const int kc = (lg + 4 * ks) & (R / 8 - 1);
             bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-            if (MASKED && eff < R) mask_ranks(bop[s][j][ks], kc * 8, eff);
           }
         }
 #pragma unroll
@@ -338,8 +335,19 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     }
   }
 
+  // Ranks at or above the adapter's are cleared in the B operands where they are used, not where
+  // they were requested: cleared at the request, every load is waited for on the spot.
+  auto mask_b = [&](Pack8(&bo)[4][KSTEPS]) {
+    if (MASKED && eff < R) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) mask_ranks(bo[j][ks], ((lg + 4 * ks) & (R / 8 - 1)) * 8, eff);
+    }
+  };
   auto finish_span = [&](int c0, Pack8(&bo)[4][KSTEPS], Pack8(&yy)[2]) {
     f32x4 out[4];
+    mask_b(bo);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -377,6 +385,10 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
     f32x4 out[4];
     uint2 pieces[4];
     if constexpr (K16) {
+      if (MASKED && eff < R) {
+        mask_ranks(bo[0][0], (lane & 1) * 8, eff);
+        mask_ranks(bo[1][0], (lane & 1) * 8, eff);
+      }
       // B rows -> operand pieces through the wavefront's LDS block: four rows (128 bytes) per
       // group, groups 144 bytes apart so that the sixteen lanes of a piece read hit every bank
       // once.  MFMA j of lane (lr, lg) takes ranks 4*lg .. 4*lg+3 of column c0 + 4*lr + j.
@@ -387,6 +399,8 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
       for (int j = 0; j < 4; ++j) pieces[j] = *reinterpret_cast<const uint2*>(blk + lr * 144 + j * 32 + lg * 8);
       __builtin_amdgcn_wave_barrier();
+    } else {
+      mask_b(bo);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -447,7 +461,6 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const int kc = (lg + 4 * ks) & (R / 8 - 1);
           bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
-          if (MASKED && eff < R) mask_ranks(bo[j][ks], kc * 8, eff);
         }
       }
 #pragma unroll
