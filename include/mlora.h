@@ -211,7 +211,7 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
  * all sixteen name rows of the tile itself), then padding.
  * A big tile is four words {slot, first position in sorted_idx, token count, 0}; behind the
  * big-tile records lies one list of MLORA_TILE_BIG token indices per big tile (its tokens in
- * order, repeated cyclically past the count), at a place that follows from the tile's number
+ * order, 0 past the count: a valid row to read), at a place that follows from the tile's number
  * alone: a workgroup requests it together with the record. */
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */

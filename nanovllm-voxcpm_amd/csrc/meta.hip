@@ -73,18 +73,35 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   const int beg = wave * span;
   const int end = beg + span < T ? beg + span : T;
 
-  // (the slot id of the next step is requested before the current one is counted)
-  int s_next = beg + lane < end ? p.tts[beg + lane] : -1;
-  for (int base = beg; base < end; base += kWave) {
-    const int t = base + lane;
-    const int s = s_next;
-    if (t + kWave < end) s_next = p.tts[t + kWave];
+  // A wavefront walks its span in steps of 64 tokens with the slot ids of the next four steps
+  // requested ahead: a step is a few hundred cycles of work and a request to memory takes several
+  // times that, so with one step in flight the walk runs at the pace of the memory's latency.
+  constexpr int kAhead = 4;
+  auto walk = [&](auto&& step) {
+    int q[kAhead];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      const int t = beg + j * kWave + lane;
+      q[j] = t < end ? p.tts[t] : -1;
+    }
+    for (int base = beg; base < end; base += kAhead * kWave) {
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) {
+        const int t = base + j * kWave + lane;
+        const int s = q[j];
+        const int tn = t + kAhead * kWave;
+        q[j] = tn < end ? p.tts[tn] : -1;
+        if (base + j * kWave < end) step(t, s);
+      }
+    }
+  };
+  walk([&](int t, int s) {
     if (t < end) {
       int key = (s >= 0 && s < L) ? s + 1 : 0;
       if (s >= L) s_bad = 1;
       atomicAdd(&hist[wave * NB + key], 1);
     }
-  }
+  });
   if (p.padded_tts) {
     for (int i = tid; i < p.padded_len; i += kMetaThreads) p.padded_tts[i] = i < T ? p.tts[i] : -1;
   }
@@ -225,6 +242,9 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       int left = c - j * MLORA_TILE_BIG;
       big[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
     }
+    // row lists of the big tiles: cleared, the scatter below enters the tokens
+    i32x4* rows = reinterpret_cast<i32x4*>(p.plan + lay.bigrows_off);
+    for (int q = tid; q < n_big * (MLORA_TILE_BIG / 4); q += kMetaThreads) rows[q] = i32x4{0, 0, 0, 0};
   }
   __syncthreads();
 
@@ -232,13 +252,9 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   // among the equal keys of its 64-token step is counted lane against lane; the running cursor
   // of (wave, key) lives in hist and is advanced once per distinct key per step.
   int32_t* plan_sorted = p.plan ? p.plan + lay.sorted_off : nullptr;
-  s_next = beg + lane < end ? p.tts[beg + lane] : -1;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
   const int key_bits = 32 - __builtin_clz(NB);  // keys are 0 .. NB - 1
-  for (int base = beg; base < end; base += kWave) {
-    const int t = base + lane;
-    const int s = s_next;
-    if (t + kWave < end) s_next = p.tts[t + kWave];
+  walk([&](int t, int s) {
     int key = -1;
     if (t < end) key = (s >= 0 && s < L) ? s + 1 : 0;
     const bool take = key >= 1 || (key == 0 && p.no_lora_bucket && !reset_only);
@@ -266,13 +282,10 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
           const int n = left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL;
           for (int pos = r % MLORA_TILE_SMALL; pos < MLORA_TILE_SMALL; pos += n)
             p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + pos] = t;
-          if (c >= MLORA_SEGMENT_THRESHOLD) {
-            // the same for the row list of the segment's 64-token tile
-            const int qb = ts_big[key] + r / MLORA_TILE_BIG;
-            const int leftb = c - (r / MLORA_TILE_BIG) * MLORA_TILE_BIG;
-            const int nb = leftb < MLORA_TILE_BIG ? leftb : MLORA_TILE_BIG;
-            for (int pos = r % MLORA_TILE_BIG; pos < MLORA_TILE_BIG; pos += nb) p.plan[lay.bigrows_off + qb * MLORA_TILE_BIG + pos] = t;
-          }
+          // its entry in the row list of the segment's 64-token tile (entries past a tile's count
+          // stay 0, a valid row: only the last tile of a segment has any, and repeating its tokens
+          // there as in the small records is a loop of up to 64 stores in one lane)
+          if (c >= MLORA_SEGMENT_THRESHOLD) p.plan[lay.bigrows_off + (ts_big[key] + r / MLORA_TILE_BIG) * MLORA_TILE_BIG + r % MLORA_TILE_BIG] = t;
         }
         if (p.sorted_idx) p.sorted_idx[n_neg + off[key] + r] = t;
       } else if (p.sorted_idx) {
@@ -283,7 +296,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       if (before == group - 1) hist[wave * NB + key] = cursor + group;
     }
     __builtin_amdgcn_wave_barrier();
-  }
+  });
 }
 
 }  // namespace

@@ -63,7 +63,8 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
 // Token row at position `ti` of tile `tile`.  Where it lies follows from the tile's number alone (a
 // 64-token tile has its row list behind the big-tile records, a short segment carries its rows in
 // its record), so it is requested together with the record instead of after it.  Positions past
-// the tile's count hold rows of the tile as well (a valid row to read, never written).
+// the tile's count hold a valid row as well (a tile's own in a short segment's record, row 0 in a
+// big tile's list): read, never written.
 __device__ __forceinline__ int tile_row(const int32_t* __restrict__ plan, int bigrows_off, int small_off, int big_cap, int tile, int ti) {
   const bool is_big = tile < big_cap;
   const int at = is_big ? bigrows_off + tile * MLORA_TILE_BIG + ti
@@ -114,7 +115,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
   const int nbatch = krange / XW;
   const bool active = wave * 16 < m;  // this wavefront's token block exists
   // `row`: token row of this lane, position wave * 16 + lane % 16 of the tile (positions past the
-  // end of the tile name rows of the tile too: they feed the MFMA harmlessly and are never
+  // end of the tile name valid rows too: they feed the MFMA harmlessly and are never
   // written back)
   const int ti = wave * 16 + lr;
   MLORA_STAMP(2);  // shrink: body entered (the token rows were requested with the record)
@@ -616,7 +617,7 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   const bool has_work = c0 < sp.n1;
 
   // `rowv[g]` (threads 0..63): token row at position tid of tile g, requested by the caller
-  // together with the tile records.  Entries past the end of a tile name rows of the tile too (a
+  // together with the tile records.  Entries past the end of a tile name valid rows too (a
   // valid row to read, never written).  The partial sums of the first tile hang on the tile
   // record alone; they are requested before the barrier the rows pass through, so that they and
   // the y rows are on their way together.  (The B rows of the first span could go out there too,

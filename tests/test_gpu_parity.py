@@ -875,9 +875,9 @@ def test_metadata_bit_exact_random(T, L, p_neg):
         own = s[start : start + count]
         assert rec[4:20] == [own[j % count] for j in range(16)] and rec[20:] == [0] * 12  # cyclic repeats past the count
     assert [tuple(ws[big_off + 4 * i : big_off + 4 * i + 3]) for i in range(len(long_big))] == long_big
-    for q, (slot, start, count) in enumerate(long_big):  # the tile's tokens, repeated cyclically past its count
+    for q, (slot, start, count) in enumerate(long_big):  # the tile's tokens, then zeros (a valid row to read)
         own = s[start : start + count]
-        assert ws[bigrows_off + 64 * q : bigrows_off + 64 * (q + 1)] == [own[j % count] for j in range(64)]
+        assert ws[bigrows_off + 64 * q : bigrows_off + 64 * (q + 1)] == own + [0] * (64 - count)
 
 
 def test_metadata_flags_bad_slot_ids():
