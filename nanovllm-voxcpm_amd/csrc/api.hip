@@ -85,8 +85,8 @@ struct ApiKnobs {
     force_form = env_int("MLORA_FORCE_FORM", 0);
     no_split = env_int("MLORA_NO_SPLIT", 0);
     // Measured on the prefill batch (7605 tokens, rank 64) and the mixed one: the one-launch
-    // long-segment form takes 4214 us per step against 3858 for two launches (mixed: 6496 against
-    // 5467).  Its workgroups are all resident at once, so the whole grid first shrinks (a chain of
+    // long-segment form takes 4060 us per step against 3586 for two launches (mixed: 6090 against
+    // 4992).  Its workgroups are all resident at once, so the whole grid first shrinks (a chain of
     // dependent slab fetches per workgroup, HBM nearly idle) and then expands; the saved launch
     // does not pay for the wait on the slowest role of each unit.  AUTO keeps the two launches.
     auto_fused = env_int("MLORA_AUTO_FUSED", 0);
