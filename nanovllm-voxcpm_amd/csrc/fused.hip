@@ -62,7 +62,7 @@ __device__ __attribute__((noinline)) void fused_shrink_role_late(T* s_a, const i
 template <typename T, int R, int CPL, int TPF, int G>
 __device__ __forceinline__ void fused_expand(T* s_h, int* s_row, int* s_slot, int* s_m, int* s_eff, const int* s_start,
                                                        const int32_t* plan, const float* hws, void* yv_, int64_t ys, int sorted_off, int T_,
-                                                       int num_slices, int ksplit, float scaling, int nt, const ExpandSplit& sp) {
+                                                       int num_slices, int ksplit, float scaling, const ExpandSplit& sp) {
   int slot[G], start[G], m[G], eff[G], rowv[G];
   bool masked = false;
 #pragma unroll
@@ -75,10 +75,10 @@ __device__ __forceinline__ void fused_expand(T* s_h, int* s_row, int* s_slot, in
   }
   __syncthreads();  // expand_body rewrites the arrays read above
   if (masked)
-    expand_body<T, R, CPL, TPF, G, true, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+    expand_body<T, R, CPL, TPF, G, true, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, sp, slot, start,
                                                m, eff, rowv);
   else
-    expand_body<T, R, CPL, TPF, G, false, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+    expand_body<T, R, CPL, TPF, G, false, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, sp, slot, start,
                                                 m, eff, rowv);
 }
 
@@ -86,7 +86,7 @@ template <typename T, int R, int KR, int XW, bool DB, int CPL, int TPF, int G>
 __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
     const int32_t* __restrict__ plan, const void* __restrict__ xv, void* __restrict__ yv_, uint32_t* __restrict__ ws,
     float* __restrict__ hws, int64_t xs, int64_t ys, int big_off, int small_off, int big_units, int sorted_off, int T_, int K,
-    int num_slots, int num_slices, int ksplit, int krange, int all_slices, float scaling, int nt, int spin_ticks, int trusted,
+    int num_slots, int num_slices, int ksplit, int krange, int all_slices, float scaling, int spin_ticks, int trusted,
     const int32_t* __restrict__ eff_rank, ShrinkSlices sl, ExpandSplits splits) {
   constexpr int HSTRIDE = 2 * R + 8;
   constexpr int kShrinkLds = R * (KR + 8) * static_cast<int>(sizeof(T));
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   // (every path to here ends in a barrier: the slab buffer is free for the intermediate)
 
   // ---- expand ---------------------------------------------------------------------------------------
-  fused_expand<T, R, CPL, TPF, G>(s_h, s_row, s_slot, s_m, s_eff, s_start, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, nt, sp);
+  fused_expand<T, R, CPL, TPF, G>(s_h, s_row, s_slot, s_m, s_eff, s_start, plan, hws, yv_, ys, sorted_off, T_, num_slices, ksplit, scaling, sp);
 
   MLORA_STAMP(13);  // expanded (wavefront 0)
   count_done();
@@ -281,7 +281,7 @@ void launch_fused_one(const FusedLaunch& l) {
   hipLaunchKernelGGL((sgmv_fused_kernel<T, R, KR, XW, DB, 8, 2, G>), grid, dim3(kFusedThreads), 0, static_cast<hipStream_t>(a->stream), a->plan,
                      a->x, a->y, static_cast<uint32_t*>(a->workspace), partials_of(a), a->x_stride, a->y_stride, sh.lay.big_off,
                      sh.lay.small_off, sh.big_units, sh.lay.sorted_off, a->num_tokens, a->k, a->num_slots, a->num_slices, sh.ksplit,
-                     sh.krange, sh.all_slices, a->scaling, sgmv_knobs().nt_hint, fused_knobs().spin_ticks, l.trusted, a->effective_rank,
+                     sh.krange, sh.all_slices, a->scaling, fused_knobs().spin_ticks, l.trusted, a->effective_rank,
                      sh.sl, sh.splits);
 }
 

@@ -78,7 +78,7 @@ template <typename T, int R, int CPL, int TPF, int G>
 __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                                                              void* __restrict__ yv_, int64_t ys, int big_off, int small_off,
                                                                              int big_units, int bigrows_off, int T_, int num_slots,
-                                                                             int num_slices, int ksplit, float scaling, int nt,
+                                                                             int num_slices, int ksplit, float scaling,
                                                                              const int32_t* __restrict__ eff_rank, ExpandSplits splits) {
   constexpr int HSTRIDE = 2 * R + 8;     // padded LDS row: R leading parts, R remainders
   __shared__ __attribute__((aligned(16))) T s_h[G * MLORA_TILE_BIG * HSTRIDE];
@@ -147,10 +147,10 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
 #pragma unroll
   for (int g = 0; g < G; ++g) masked |= m[g] > 0 && eff[g] < R;
   if (masked)
-    expand_body<T, R, CPL, TPF, G, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+    expand_body<T, R, CPL, TPF, G, true>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, sp, slot, start,
                                          m, eff, rowv);
   else
-    expand_body<T, R, CPL, TPF, G, false>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, nt, sp, slot, start,
+    expand_body<T, R, CPL, TPF, G, false>(s_h, s_row, s_slot, s_m, s_eff, plan, hws, yv_, ys, T_, num_slices, ksplit, scaling, sp, slot, start,
                                           m, eff, rowv);
 }
 
@@ -196,11 +196,10 @@ void launch_expand_group(const MloraAddArgs* a, const PlanLayout& lay, int big_u
                          const ExpandSplits& sp) {
   hipStream_t st = static_cast<hipStream_t>(a->stream);
   const float* h = partials_of(a);
-  const int nt = sgmv_knobs().nt_hint;
 #define MLORA_EXPAND(CPL_, TPF_, G_)                                                                                       \
   hipLaunchKernelGGL((sgmv_expand_kernel<T, R, CPL_, TPF_, G_>), grid, dim3(kExpandWaves* kWave), 0, st, a->plan, h, a->y, \
                      a->y_stride, lay.big_off, lay.small_off, big_units, lay.bigrows_off, a->num_tokens, a->num_slots,      \
-                     a->num_slices, ksplit, a->scaling, nt, a->effective_rank, sp)
+                     a->num_slices, ksplit, a->scaling, a->effective_rank, sp)
   if (cpl == 4) {
     if (group == 4) MLORA_EXPAND(4, 4, 4); else if (group == 2) MLORA_EXPAND(4, 4, 2); else MLORA_EXPAND(4, 4, 1);
   } else {

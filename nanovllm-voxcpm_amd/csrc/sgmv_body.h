@@ -417,7 +417,7 @@ template <typename T, int R, int CPL, int TPF, int G, bool MASKED, bool SC1 = fa
 __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict__ s_row, int* __restrict__ s_slot, int* __restrict__ s_m,
                                             int* __restrict__ s_eff, const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                             void* __restrict__ yv_, int64_t ys, int T_, int num_slices, int ksplit,
-                                            float scaling, int nt, const ExpandSplit& sp, const int (&slot)[G], const int (&start)[G],
+                                            float scaling, const ExpandSplit& sp, const int (&slot)[G], const int (&start)[G],
                                             const int (&m)[G], const int (&eff)[G], const int (&rowv)[G]) {
   constexpr int TB = MLORA_TILE_BIG / 16;
   constexpr int NB = TB / TPF;           // y batches per tile
@@ -736,10 +736,9 @@ size_t partials_room(const MloraAddArgs* a) {
 
 // Diagnostic knobs, read from the environment once and again after mlora_reload_knobs().
 struct SgmvKnobs {
-  int generation = -1, nt_hint, kr, ksplit, all_slices, xdb, group, wgs, nt, cpl;
+  int generation = -1, kr, ksplit, all_slices, xdb, group, wgs, nt, cpl;
   void read() {
     generation = knob_generation();
-    nt_hint = env_int("MLORA_SGMV_NT_HINT", 0);
     kr = env_int("MLORA_SGMV_KR", 0);
     ksplit = env_int("MLORA_SGMV_KSPLIT", 0);
     all_slices = env_int("MLORA_SGMV_ALL_SLICES", 3);
