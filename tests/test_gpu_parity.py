@@ -145,6 +145,31 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
+@pytest.mark.parametrize("rank", [16, 64])
+@pytest.mark.parametrize("name", ["gate_up", "o"])
+def test_small_tile_form_is_the_same_for_every_column_range_width(name, rank, monkeypatch):
+    """The small-tile kernel exists in an instance that requests one output span per wavefront up
+    front (column ranges of at most 512 columns) and one that requests two (wider ranges); with
+    ranges of 128..1024 columns both are taken, with and without the spans that wide ranges walk
+    in a loop.  Every width gives the oracle's result, and all give the same bits: the cut into
+    column ranges changes which workgroup computes a column, not how."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"small tiles, range widths, {name} r={rank}", flush=True)
+    proj = _make(name, 32, rank, torch.bfloat16, seed=140 + rank)
+    x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=141, device="cuda")
+    slots = synthetic.decode_slots(256, 32, seed=142).cuda()
+    exact, mag = _exact(proj, x, y0, slots)
+    outs = []
+    for width in (128, 512, 1024, 4096):
+        _knobs(monkeypatch, MLORA_DECODE_NT=width)
+        outs.append(_apply("mfma", proj, x, y0.clone(), slots))
+        _check(outs[-1], y0, exact, mag, slots, f"small tiles/{name}/r{rank}/ranges of {width}")
+    _knobs(monkeypatch, MLORA_DECODE_NT=None)
+    for out in outs[1:]:
+        assert torch.equal(out, outs[0])
+
+
 @pytest.mark.parametrize("sym", [0, 1])
 @pytest.mark.parametrize("wide", [5, 7])
 @pytest.mark.parametrize("kpart", [512, 1024])
