@@ -107,6 +107,23 @@ template <> struct Mma16<_Float16> {
   }
 };
 
+// After a run of MFMAs that a branch can cut short (rank blocks or k-steps left out at run time),
+// and before anything else reads the accumulators.  An MFMA's result may not be read by another
+// kind of instruction for some cycles after its issue; the compiler keeps that distance along
+// straight-line code, but where such a run is left through a branch that lands on the reading
+// code it was seen to provide for the longest way there only: the last MFMA's result was read
+// two instructions after it and came out incomplete or not, depending on where the code lay in
+// memory (rank-64 buffers with an adapter of rank 16 or less: the last k-step of a K part went
+// missing).  24 idle cycles cover the longest MFMA; the accumulators are operands so that none
+// of their reads is moved ahead of them.
+template <int N> __device__ __forceinline__ void mfma_settle(f32x4 (&acc)[N]) {
+  static_assert(N >= 1 && N <= 4, "accumulator blocks");
+  if constexpr (N == 1) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(acc[0]));
+  else if constexpr (N == 2) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(acc[0]), "+v"(acc[1]));
+  else if constexpr (N == 3) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]));
+  else asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
+}
+
 // Zero the elements of an eight-element chunk that hold ranks at or above `eff`; `first` is the
 // rank of the chunk's element 0.
 __device__ __forceinline__ void mask_ranks(Pack8& p, int first, int eff) {

@@ -305,6 +305,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   }
 
   // Sum the K-partials of the wavefronts.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
+  if constexpr (KSPW == 0) mfma_settle(acc);  // k-steps past the end of K were skipped by branches
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
   MLORA_STAMP(3);  // wavefront 0: x and A arrived, staged and multiplied

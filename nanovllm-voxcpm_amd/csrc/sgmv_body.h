@@ -245,6 +245,9 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
                 acc[rb] = Mma<T>::run(aw, xa[i], acc[rb]);
               }
             }
+            if constexpr (MASKED) {
+              if (s == NS - 1) mfma_settle(acc);  // rank blocks were skipped by branches
+            }
           }
         }
         if (active && b + 1 < nbatch) {
@@ -296,6 +299,9 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
             acc[rb] = Mma<T>::run(aw, cur[s * KS + i], acc[rb]);
           }
         }
+        if constexpr (MASKED) {
+          if (s == SPB - 1) mfma_settle(acc);  // rank blocks were skipped by branches
+        }
       }
     }
     if (!DB && ACT && b + 1 < nbatch) request_x(cur, (b + 1) * XW);
@@ -339,6 +345,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
               acc[rb] = Mma<T>::run(aw, cur[i], acc[rb]);
             }
           }
+          if constexpr (MASKED && !MORE) mfma_settle(acc);  // rank blocks were skipped by branches
         }
       };
       int b = 0;

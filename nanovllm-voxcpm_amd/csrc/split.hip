@@ -444,6 +444,7 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
         }
       }
     }
+    if constexpr (!K16 && KSTEPS > 1) mfma_settle(out);  // k-steps beyond the adapter's rank were skipped by branches
     const int c = c0 + 4 * lr;
     if (c < n1) {
 #pragma unroll

@@ -76,6 +76,46 @@ def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, 
     assert _hip.FORMS[form] >= 0
 
 
+@pytest.mark.parametrize("form", ["auto", "sgmv", "fused", "mfma", "split"])
+@pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
+def test_last_k_steps_of_every_k_part_count_for_adapters_of_every_rank(name, form):
+    """x is zero except for the last 32 columns of every sixteenth of K (the last MFMA step of every
+    K part and of every batch of one, however the kernel cuts K), so each of those steps is most of
+    the result instead of a hundredth of it.  Adapters of rank 8..64 in rank-64 buffers, with the
+    rank vector: a kernel that leaves rank blocks out takes a different path through its MFMAs for
+    each number of blocks, and the result of the last MFMA on the shortest path (one block) was once
+    read before the matrix pipeline had delivered it."""
+    from nanovllm_voxcpm_amd import _hip
+
+    tokens = 200
+    if form == "fused" and "fused" not in _hip.FORMS:
+        pytest.skip("no one-launch form in this library")
+    print(f"last k-steps {name} form={form}", flush=True)
+    ranks = [8, 12, 16, 32, 40, 64, 0, 24]
+    clean = _make(name, len(ranks), 64, torch.bfloat16, seed=810, true_ranks=ranks)
+    g = torch.Generator().manual_seed(811)
+    slots = torch.randint(-1, len(ranks), (tokens,), generator=g, dtype=torch.int32)
+    slots[:40] = 3
+    slots = slots.cuda()
+    from nanovllm_voxcpm_amd import synthetic
+
+    x, y0 = synthetic.make_activations(tokens, clean.k, sum(clean.widths), torch.bfloat16, seed=812, device="cuda")
+    keep = torch.zeros(clean.k, dtype=torch.bool, device="cuda")
+    step = clean.k // 16
+    for part in range(16):
+        keep[(part + 1) * step - 32 : (part + 1) * step] = True
+    x = x * keep
+    eff = torch.tensor(ranks, dtype=torch.int32, device="cuda")
+    exact, mag = _exact(clean, x, y0, slots)
+    backend = _backend(form)
+    for _ in range(2):
+        y = y0.clone()
+        blocks = list(y.split(clean.widths, dim=-1))
+        backend.add_lora(blocks, x, clean.a, clean.b, indices=slots, metadata=_metadata(slots), scaling=1.0,
+                         y_packed=y if len(blocks) > 1 else None, effective_rank=eff)
+        _check(y, y0, exact, mag, slots, f"last-k-steps/{name}/{form}")
+
+
 def test_layers_pass_their_rank_vector_to_the_backend():
     """A rank-64 layer holding adapters of rank 8 and 64: after the padded rows / columns of the
     rank-8 slot are overwritten with NaN behind the layer's back, its forward is still the fp64
