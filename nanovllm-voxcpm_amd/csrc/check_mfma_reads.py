@@ -6,7 +6,7 @@ left through a branch (rank blocks or k-steps that are skipped at run time) and 
 on code that reads the last result, it was seen to provide for the longest way to that code only:
 the result was read two instructions after its MFMA and came out incomplete or not depending on
 where the code lay in memory.  The kernels therefore call `mfma_settle` behind such runs; this
-script finds places where that was forgotten: an MFMA followed within a few instructions by a
+script finds places where that was forgotten: an MFMA followed within NEED wait states by a
 branch whose target reads the MFMA's destination registers after fewer than NEED wait states.
 
 usage: check_mfma_reads.py file.s [file.s ...]    (exit status 1 if anything is found)
@@ -66,20 +66,25 @@ def scan(path):
         if not t.startswith("v_mfma"):
             continue
         dst = vgprs(t.split(",")[0])
+        # walk on from the MFMA; every branch met before NEED wait states have passed is followed
         j, states = i + 1, 0
-        while j < len(lines) and states < 3:
+        while j < len(lines) and states < NEED:
             u = lines[j].strip()
             j += 1
             if not is_code(u):
                 continue
-            if not u.startswith(("s_branch", "s_cbranch")):
+            if u.startswith("s_nop"):
+                states += int(u.split()[1]) + 1
+                continue
+            if u.startswith(("s_waitcnt", "s_barrier", "s_endpgm", "v_mfma")):
                 break
-            hit = early_read(lines, labels.get(u.split()[-1], len(lines)), dst, states + 1)
-            if hit:
-                print(f"{path}:{i + 1}: {func[:70]}\n    {t}\n    -> {u.split()[-1]}: read after {hit[0]} wait states: {hit[1]}")
-                found += 1
-            if u.startswith("s_branch"):
-                break
+            if u.startswith(("s_branch", "s_cbranch")):
+                hit = early_read(lines, labels.get(u.split()[-1], len(lines)), dst, states + 1)
+                if hit:
+                    print(f"{path}:{i + 1}: {func[:70]}\n    {t}\n    -> {u.split()[-1]}: read after {hit[0]} wait states: {hit[1]}")
+                    found += 1
+                if u.startswith("s_branch"):
+                    break
             states += 1
     return found
 
