@@ -116,6 +116,33 @@ def test_last_k_steps_of_every_k_part_count_for_adapters_of_every_rank(name, for
         _check(y, y0, exact, mag, slots, f"last-k-steps/{name}/{form}")
 
 
+@pytest.mark.parametrize("form", ["auto", "mfma"])
+@pytest.mark.parametrize("rank", [16, 64])
+@pytest.mark.parametrize("k", [800, 1056])
+def test_last_k_step_of_every_wavefront_counts_when_k_is_cut_at_run_time(k, rank, form):
+    """A K for which the small-tile kernel has no instance of its own: its eight wavefronts share
+    out the 32-column steps at run time (25 steps: 3, 3, ... 4; 33 steps: 4, 4, ... 5) and skip the
+    steps past their share by branches, so the last MFMA of a wavefront may be followed by a
+    branch.  x is zero except in the last step of every wavefront's share."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"last k-step per wavefront K={k} r={rank} form={form}", flush=True)
+    shapes = {"w": (k, [256, 72])}
+    proj = synthetic.make_projection("w", 6, rank, torch.bfloat16, seed=830 + rank, device="cuda", shapes=shapes)
+    slots = synthetic.decode_slots(48, 6, seed=831).cuda()
+    x, y0 = synthetic.make_activations(48, k, sum(proj.widths), torch.bfloat16, seed=832, device="cuda")
+    steps = k // 32
+    keep = torch.zeros(k, dtype=torch.bool, device="cuda")
+    for wave in range(8):
+        last = (wave + 1) * steps // 8 - 1
+        keep[32 * last : 32 * last + 32] = True
+    x = x * keep
+    exact, mag = _exact(proj, x, y0, slots)
+    for _ in range(2):
+        got = _apply(form, proj, x, y0.clone(), slots)
+        _check(got, y0, exact, mag, slots, f"last-k-step/K{k}/r{rank}/{form}")
+
+
 def test_layers_pass_their_rank_vector_to_the_backend():
     """A rank-64 layer holding adapters of rank 8 and 64: after the padded rows / columns of the
     rank-8 slot are overwritten with NaN behind the layer's back, its forward is still the fp64
