@@ -14,6 +14,7 @@ usage: check_mfma_reads.py file.s [file.s ...]    (exit status 1 if anything is 
 import re
 import sys
 
+ANY_USE = False  # True: an early overwrite of the result counts as well as an early read
 NEED = 8  # wait states the compiler itself leaves between a 16x16x32 MFMA and a read of its result
 
 
@@ -49,7 +50,7 @@ def early_read(lines, start, dst, states):
             continue
         operands = w.split(None, 1)[1].split(",") if " " in w else []
         stores = w.startswith(("global_store", "buffer_store", "ds_write", "scratch_store"))
-        if vgprs(",".join(operands if stores else operands[1:])) & dst:
+        if vgprs(",".join(operands if stores or ANY_USE else operands[1:])) & dst:
             return states, w
         states += 1
     return None
