@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MLORA_ABI_VERSION 3
+#define MLORA_ABI_VERSION 4
 
 /* element types of x / y / A / B */
 #define MLORA_DTYPE_F32 0
@@ -46,6 +46,10 @@ extern "C" {
 #define MLORA_FORM_FUSED 6 /* the tiles of MLORA_FORM_SGMV in one launch: the workgroups of a group of tiles share
                               out its shrink, seal what they wrote to the workspace, wait for each other's seals
                               and expand a column range each; needs an initialised workspace */
+#define MLORA_FORM_SLOT 7  /* MLORA_FORM_MFMA with the grid laid over the slots instead of the tiles: the workgroup of
+                              (slot, column range) requests A[slot] and B[slot] from its own index alone, before the
+                              record of the slot's first sixteen tokens has arrived; further tiles of a slot are
+                              taken by extra workgroups of the same launch */
 
 /* error codes (negative) */
 #define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
@@ -198,6 +202,10 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
 #define MLORA_PLAN_TILES_LONG_SMALL 8 /* small tiles of segments at or above the threshold */
 #define MLORA_PLAN_TILES_LONG_BIG 9  /* big tiles of segments at or above the threshold */
 #define MLORA_PLAN_MAX_SEGMENT 10    /* longest segment */
+#define MLORA_PLAN_TILES_OVER 11     /* small tiles that are not the first tile of their slot */
+#define MLORA_PLAN_REJECTED 12       /* launches of mlora_add_lora that found this plan built for another
+                                        (num_tokens, max_slots) or not built at all and therefore left y as it
+                                        was: the one word of a plan that the apply kernels write (atomically) */
 #define MLORA_PLAN_HEADER_WORDS 16
 #define MLORA_PLAN_MAGIC_VALUE 0x4d4c5031 /* "MLP1" */
 
@@ -216,6 +224,14 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
 #define MLORA_BIG_TILE_WORDS 4
+/* Behind the row lists of the big tiles the same small tiles are listed a second time, by slot: one
+ * 128-byte record per slot id (its place follows from the slot id alone: a workgroup that serves a
+ * slot can request the slot's weights before it knows the slot's tokens) for the slot's first
+ * sixteen tokens, then one record for every further small tile of every slot (unused ones carry
+ * count 0).  Words {slot, token count, first position in sorted_idx, MLORA_PLAN_CHECK(T, L)}, then
+ * the sixteen token indices as in a small-tile record. */
+#define MLORA_PLAN_CHECK(num_tokens, max_slots) \
+  (0x4d4c5031u ^ (uint32_t)(num_tokens) ^ ((uint32_t)(max_slots) << 20))
 
 /* Arguments of the on-device metadata build: a stable counting sort of the tokens by
  * slot id.  The plan workspace (always written when non-NULL) feeds mlora_add_lora; the

@@ -78,7 +78,7 @@ namespace {
 
 // Diagnostic knobs, read from the environment once per process.
 struct ApiKnobs {
-  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, split_max_tokens, auto_fused;
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, split_max_tokens, auto_fused, slot_max_slots;
   void read() {
     generation = knob_generation();
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
@@ -101,6 +101,9 @@ struct ApiKnobs {
     // ... and while the batch has few tiles: K = 4096, rank 32 / 64, 1011 tokens: 12.0 / 17.7 us against
     // 14.8 / 23.1; 1620 tokens: 17.6 / 26.8 against 15.8 / 24.7
     split_max_tokens = env_int("MLORA_SPLIT_MAX_TOKENS", 1280);
+    // The slot-major grid launches a workgroup per (slot id, column range) whether the slot has
+    // tokens or not; with many more slot ids than adapters in the batch those requests are waste.
+    slot_max_slots = env_int("MLORA_SLOT_MAX_SLOTS", 64);
   }
 };
 const ApiKnobs& knobs() {
@@ -151,7 +154,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (a->dtype != MLORA_DTYPE_F32 && a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) {
     set_error("mlora_add_lora: unknown dtype %d", a->dtype); return MLORA_E_INVALID;
   }
-  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_FUSED) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
+  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_SLOT) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
   if (a->num_slices > MLORA_MAX_SLICES) { set_error("mlora_add_lora: %d slices exceed %d", a->num_slices, MLORA_MAX_SLICES); return MLORA_E_TOO_LARGE; }
   if (a->r > MLORA_MAX_RANK) { set_error("mlora_add_lora: rank %d exceeds %d", a->r, MLORA_MAX_RANK); return MLORA_E_TOO_LARGE; }
   if (a->num_slots > MLORA_MAX_SLOTS) { set_error("mlora_add_lora: %d slots exceed %d", a->num_slots, MLORA_MAX_SLOTS); return MLORA_E_TOO_LARGE; }
@@ -177,7 +180,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   const bool vec = vector_ok(a);
   if (form == MLORA_FORM_AUTO) {
     const int forced = knobs().force_form;
-    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_FUSED && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
+    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_SLOT && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
   }
   if (form == MLORA_FORM_AUTO) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
@@ -194,6 +197,10 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
       (knobs().no_split || !split_supported(a) || ((static_cast<long long>(a->r) * a->k < knobs().split_min_rk || a->num_tokens > knobs().split_max_tokens) && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;
+  // small tiles with the grid laid over the slots where the shape allows it and slot ids are few
+  if (form == MLORA_FORM_MFMA && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_MFMA && slot_supported(a) &&
+      a->num_slots <= knobs().slot_max_slots)
+    form = MLORA_FORM_SLOT;
   // long-segment batches in one launch, on request
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))
     form = MLORA_FORM_FUSED;
@@ -208,9 +215,17 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     case MLORA_FORM_SGMV:
     case MLORA_FORM_FUSED:
     case MLORA_FORM_SPLIT:
+    case MLORA_FORM_SLOT:
     case MLORA_FORM_MFMA: {
       if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
+      if (form == MLORA_FORM_SLOT) {
+        if (!slot_supported(a)) {
+          set_error("mlora_add_lora: the slot-major form needs one or two non-empty slices and K = 1024 (any rank) or 4096 (rank <= 16)");
+          return MLORA_E_UNSUPPORTED;
+        }
+        return launch_slot(a);
+      }
       if (form == MLORA_FORM_SPLIT) {
         if (!split_supported(a)) {
           set_error("mlora_add_lora: the split form needs K %% 512 == 0, at most 8 K parts, no empty slice and a 256-byte aligned "
@@ -323,6 +338,7 @@ extern "C" uint64_t mlora_stream_capture_id(void* stream) {
 extern "C" int mlora_trace_set(void* buf) {
 #ifdef MLORA_TRACE
   decode_trace_set(buf);
+  slot_trace_set(buf);
   split_trace_set(buf);
   fused_trace_set(buf);
   sgmv_trace_set(buf);

@@ -84,8 +84,10 @@ __global__ __launch_bounds__(kThreads) void bgmv_kernel(BgmvParams p) {
   const int32_t* rec = p.plan + p.small_off + tile * MLORA_SMALL_TILE_WORDS;  // tile < capacity: in bounds
   const int slot = rec[0], m_tile = rec[1];
   if (hdr[MLORA_PLAN_MAGIC] != MLORA_PLAN_MAGIC_VALUE || hdr[MLORA_PLAN_NUM_TOKENS] != p.T ||
-      hdr[MLORA_PLAN_MAX_SLOTS] != p.num_slots)
+      hdr[MLORA_PLAN_MAX_SLOTS] != p.num_slots) {
+    count_rejected_plan(p.plan, false);
     return;
+  }
   const int n_tiles = hdr[MLORA_PLAN_TILES_SHORT] + (p.include_long ? hdr[MLORA_PLAN_TILES_LONG_SMALL] : 0);
   if (tile >= n_tiles) return;
 

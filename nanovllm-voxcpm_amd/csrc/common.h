@@ -171,10 +171,12 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---- plan workspace layout ------------------------------------------------------------
-// int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles | big-tile rows
+// int32 words:  header | sorted_idx[T] | counts[L+1] | offsets[L+2] | small tiles | big tiles | big-tile rows |
+//               records by slot | records of the further small tiles
 // Small tiles are 32-word records (128-byte aligned), big tiles four words, their row lists 64 words; see mlora.h.
 struct PlanLayout {
-  int sorted_off, counts_off, offsets_off, small_off, big_off, bigrows_off, cap_small, cap_big, total_words;
+  int sorted_off, counts_off, offsets_off, small_off, big_off, bigrows_off, cap_small, cap_big;
+  int slotrec_off, cap_slotrec, over_off, cap_over, total_words;
 };
 
 __host__ __device__ inline int round_up4(int v) { return (v + 3) & ~3; }
@@ -192,8 +194,23 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
   p.cap_big = (T / MLORA_TILE_BIG + segs + 31) & ~31;  // groups of up to four tiles, eight groups abreast
   p.bigrows_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;  // (a multiple of 32 words again)
-  p.total_words = p.bigrows_off + MLORA_TILE_BIG * p.cap_big;
+  // the small tiles once more, by slot: one record per slot id, then one per further tile (a
+  // further tile has sixteen tokens of its slot in front of it, so T / 16 bounds their number)
+  p.slotrec_off = p.bigrows_off + MLORA_TILE_BIG * p.cap_big;
+  p.cap_slotrec = (L + 7) & ~7;
+  p.over_off = p.slotrec_off + MLORA_SMALL_TILE_WORDS * p.cap_slotrec;
+  p.cap_over = (T / MLORA_TILE_SMALL + 7) & ~7;
+  p.total_words = p.over_off + MLORA_SMALL_TILE_WORDS * p.cap_over;
   return p;
+}
+
+// A launch that finds its plan built for another batch shape (or not built at all) leaves y as it
+// was; its first workgroup counts the launch in the plan's header (MLORA_PLAN_REJECTED), the one
+// word of a plan that the apply kernels write.  Called on the way out only: nothing of it stands
+// in front of a working workgroup's loads.
+__device__ __forceinline__ void count_rejected_plan(const int32_t* plan, bool header_ok) {
+  if (!header_ok && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+    atomicAdd(const_cast<int32_t*>(plan) + MLORA_PLAN_REJECTED, 1);
 }
 
 // ---- workspace head (see MLORA_WORKSPACE_HEAD_BYTES in mlora.h) -------------------------------

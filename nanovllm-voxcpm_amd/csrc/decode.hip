@@ -118,7 +118,11 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
                      int(slot < num_slots) & int(sp.n0 < sp.n1) & int(sp.a != nullptr) & int(sp.b != nullptr) &
                      int(sp.n > 0) & int(sp.y_col >= 0) & int(__builtin_amdgcn_readfirstlane(row) >= 0) &
                      int(__builtin_amdgcn_readfirstlane(rows4[0]) >= 0);
-  if (!usable) return;
+  if (!usable) {
+    count_rejected_plan(plan, hdr[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE && hdr[MLORA_PLAN_NUM_TOKENS] == T_ &&
+                                  hdr[MLORA_PLAN_MAX_SLOTS] == num_slots);
+    return;
+  }
   MLORA_STAMP(1);  // tile record and plan header are here
 
   // rank of the adapter in this slot (requested together with the record, see rank_prefetch)

@@ -159,6 +159,8 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
     }
   };
   if (!usable) {
+    count_rejected_plan(plan, hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE && hdr0[MLORA_PLAN_NUM_TOKENS] == T_ &&
+                                  hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots);
     count_done();
     return;
   }

@@ -24,6 +24,11 @@ int launch_bgmv(const MloraAddArgs* a, bool include_long);
 bool decode_supported(const MloraAddArgs* a);  // x and y below 2 GiB each
 int launch_decode(const MloraAddArgs* a, bool include_long);
 
+// slot.hip: the same small tiles, the grid laid over the slots: weights are requested from the
+// workgroup index alone, before the slot's record has arrived.
+bool slot_supported(const MloraAddArgs* a);
+int launch_slot(const MloraAddArgs* a);
+
 // split.hip: the same small tiles, producers and consumers of the intermediate in one launch.
 // trusted_workspace: the head of the workspace is known to be in its initial or a left-behind
 // state without carrying the signature (the library's own zero-initialised array).
@@ -45,6 +50,7 @@ int launch_fused(const MloraAddArgs* a, bool trusted_workspace);
 
 // in-kernel timeline of trace builds (no-ops otherwise)
 void decode_trace_set(void* buf);
+void slot_trace_set(void* buf);
 void split_trace_set(void* buf);
 void fused_trace_set(void* buf);
 void sgmv_trace_set(void* buf);

@@ -58,6 +58,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   int* ts_short = cidx + NB + 1;       // [NB + 1]: first small tile of a short segment
   int* ts_long = ts_short + NB + 1;    // [NB + 1]: first small tile of a long segment
   int* ts_big = ts_long + NB + 1;      // [NB + 1]: first big tile of a long segment
+  int* ts_over = ts_big + NB + 1;      // [NB + 1]: first of the small tiles behind a slot's first one
   __shared__ int s_bad, s_max;
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   // Wave 0: exclusive scans over the buckets.
   const int b0 = p.no_lora_bucket ? 0 : 1;  // first bucket of the compact arrays
   if (wave == 0) {
-    int run0 = 0, run1 = 0, run2 = 0, run3 = 0, run4 = 0, mx = 0;
+    int run0 = 0, run1 = 0, run2 = 0, run3 = 0, run4 = 0, run5 = 0, mx = 0;
     for (int base = 0; base < NB; base += kWave) {
       int b = base + lane;
       int c_all = b < NB ? total[b] : 0;
@@ -134,27 +135,30 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       int v2 = is_short ? nsmall : 0;
       int v3 = is_short ? 0 : nsmall;
       int v4 = is_short ? 0 : (c + MLORA_TILE_BIG - 1) / MLORA_TILE_BIG;
+      int v5 = nsmall > 1 ? nsmall - 1 : 0;
       int i0 = wave_incl_scan(v0, lane), i1 = wave_incl_scan(v1, lane), i2 = wave_incl_scan(v2, lane);
-      int i3 = wave_incl_scan(v3, lane), i4 = wave_incl_scan(v4, lane);
+      int i3 = wave_incl_scan(v3, lane), i4 = wave_incl_scan(v4, lane), i5 = wave_incl_scan(v5, lane);
       if (b < NB) {
         off[b] = run0 + i0 - v0;
         cidx[b] = run1 + i1 - v1;
         ts_short[b] = run2 + i2 - v2;
         ts_long[b] = run3 + i3 - v3;
         ts_big[b] = run4 + i4 - v4;
+        ts_over[b] = run5 + i5 - v5;
       }
       run0 += __shfl(i0, kWave - 1, kWave);
       run1 += __shfl(i1, kWave - 1, kWave);
       run2 += __shfl(i2, kWave - 1, kWave);
       run3 += __shfl(i3, kWave - 1, kWave);
       run4 += __shfl(i4, kWave - 1, kWave);
+      run5 += __shfl(i5, kWave - 1, kWave);
       int m = c;
 #pragma unroll
       for (int o = 32; o >= 1; o >>= 1) { int n = __shfl_xor(m, o, kWave); m = n > m ? n : m; }
       mx = m > mx ? m : mx;
     }
     if (lane == 0) {
-      off[NB] = run0; cidx[NB] = run1; ts_short[NB] = run2; ts_long[NB] = run3; ts_big[NB] = run4;
+      off[NB] = run0; cidx[NB] = run1; ts_short[NB] = run2; ts_long[NB] = run3; ts_big[NB] = run4; ts_over[NB] = run5;
       s_max = mx;
     }
   }
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   const bool reset_only = p.no_lora_bucket && n_lora == 0;
   const int n_neg = (p.no_lora_bucket && !reset_only) ? total[0] : 0;  // tokens sorted ahead of every slot
   const int n_compact = reset_only ? 0 : cidx[NB];
-  const int n_short = ts_short[NB], n_long = ts_long[NB], n_big = ts_big[NB];
+  const int n_short = ts_short[NB], n_long = ts_long[NB], n_big = ts_big[NB], n_over = ts_over[NB];
   const PlanLayout lay = plan_layout(T, L);
 
   if (tid == 0) {
@@ -183,7 +187,8 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       h[MLORA_PLAN_TILES_LONG_SMALL] = n_long;
       h[MLORA_PLAN_TILES_LONG_BIG] = n_big;
       h[MLORA_PLAN_MAX_SEGMENT] = s_max;
-      for (int i = MLORA_PLAN_MAX_SEGMENT + 1; i < MLORA_PLAN_HEADER_WORDS; ++i) h[i] = 0;
+      h[MLORA_PLAN_TILES_OVER] = n_over;
+      for (int i = MLORA_PLAN_TILES_OVER + 1; i < MLORA_PLAN_HEADER_WORDS; ++i) h[i] = 0;  // (MLORA_PLAN_REJECTED among them)
     }
     if (p.scalars) {
       p.scalars[0] = n_compact;
@@ -245,6 +250,27 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
     // row lists of the big tiles: cleared, the scatter below enters the tokens
     i32x4* rows = reinterpret_cast<i32x4*>(p.plan + lay.bigrows_off);
     for (int q = tid; q < n_big * (MLORA_TILE_BIG / 4); q += kMetaThreads) rows[q] = i32x4{0, 0, 0, 0};
+    // the small tiles once more, by slot: the record of every slot id (count 0 for a slot without
+    // tokens and for the ids that round the list up to a multiple of eight), then the further
+    // tiles of every slot, then count 0 up to the capacity
+    const int check = static_cast<int>(MLORA_PLAN_CHECK(T, L));
+    i32x4* byslot = reinterpret_cast<i32x4*>(p.plan + lay.slotrec_off);
+    for (int q = tid; q < lay.cap_slotrec + lay.cap_over; q += kMetaThreads) {
+      i32x4 head = i32x4{-1, 0, 0, check};
+      if (q < L) {
+        const int c = total[q + 1];
+        head = i32x4{q, c < MLORA_TILE_SMALL ? c : MLORA_TILE_SMALL, off[q + 1], check};
+      } else if (q >= lay.cap_slotrec && q - lay.cap_slotrec < n_over) {
+        const int qq = q - lay.cap_slotrec;
+        const int b = find_bucket(ts_over, NB, qq);
+        const int j = qq - ts_over[b] + 1, left = total[b] - j * MLORA_TILE_SMALL;
+        head = i32x4{b - 1, left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL, off[b] + j * MLORA_TILE_SMALL, check};
+      }
+      i32x4* rec = byslot + q * (MLORA_SMALL_TILE_WORDS / 4);
+      rec[0] = head;
+#pragma unroll
+      for (int w = 1; w < MLORA_SMALL_TILE_WORDS / 4; ++w) rec[w] = i32x4{0, 0, 0, 0};
+    }
   }
   __syncthreads();
 
@@ -278,10 +304,15 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
           // the token's own entry, and every entry past the tile's count that repeats it: a tile of
           // n < 16 tokens lists them cyclically, so that a kernel which fetches all sixteen rows
           // touches no memory beyond the rows of the tile itself
-          const int left = c - (r / MLORA_TILE_SMALL) * MLORA_TILE_SMALL;
+          const int tile = r / MLORA_TILE_SMALL;
+          const int left = c - tile * MLORA_TILE_SMALL;
           const int n = left < MLORA_TILE_SMALL ? left : MLORA_TILE_SMALL;
-          for (int pos = r % MLORA_TILE_SMALL; pos < MLORA_TILE_SMALL; pos += n)
+          // (the same sixteen entries in the tile's record of the list by slot)
+          const int q2 = tile == 0 ? key - 1 : lay.cap_slotrec + ts_over[key] + tile - 1;
+          for (int pos = r % MLORA_TILE_SMALL; pos < MLORA_TILE_SMALL; pos += n) {
             p.plan[lay.small_off + q * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + pos] = t;
+            p.plan[lay.slotrec_off + q2 * MLORA_SMALL_TILE_WORDS + MLORA_SMALL_TILE_ROWS + pos] = t;
+          }
           // its entry in the row list of the segment's 64-token tile (entries past a tile's count
           // stay 0, a valid row: only the last tile of a segment has any, and repeating its tokens
           // there as in the small records is a loop of up to 64 stores in one lane)
@@ -342,7 +373,7 @@ extern "C" int mlora_meta_build(const MloraMetaArgs* a) {
   p.padded_tts = a->padded_token_to_slot; p.padded_len = a->padded_len;
   p.scalars = a->scalars;
   const int NB = p.L + 1;
-  const size_t lds = sizeof(int) * (static_cast<size_t>(kMetaWaves + 1) * NB + 5 * (NB + 1));
+  const size_t lds = sizeof(int) * (static_cast<size_t>(kMetaWaves + 1) * NB + 6 * (NB + 1));
   hipLaunchKernelGGL(meta_kernel, dim3(1), dim3(kMetaThreads), lds, static_cast<hipStream_t>(a->stream), p);
   return check_launch("mlora_meta_build");
 }

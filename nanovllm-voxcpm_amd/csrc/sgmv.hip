@@ -52,7 +52,10 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   MLORA_STAMP(0);  // first instruction
   const int row = tile_row(plan, bigrows_off, small_off, big_cap, tile, (threadIdx.x / kWave) * 16 + (threadIdx.x & 15));
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
-  if (!tr.ok) return;
+  if (!tr.ok) {
+    count_rejected_plan(plan, tr.plan_ok);
+    return;
+  }
   MLORA_STAMP(1);  // tile record here
   // rank of the adapter in this slot (a second, dependent fetch, only with the vector given)
   int eff = R;
@@ -140,7 +143,11 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   }
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0) & int(sp.n0 < sp.n1);
-  if (!usable) return;
+  if (!usable) {
+    count_rejected_plan(plan, hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE && hdr0[MLORA_PLAN_NUM_TOKENS] == T_ &&
+                                  hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots);
+    return;
+  }
   MLORA_STAMP(9);  // expand: tile records here
 
   bool masked = false;

@@ -35,6 +35,7 @@ struct ExpandSplits {
 // sixteen tokens, one small-tile record each), so that one pair of launches covers the batch.
 struct TileRef {
   int slot, start, m, ok;
+  int plan_ok;  // the plan's header is that of this call's batch shape
 };
 
 __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, int big_off, int small_off, int big_cap, int tile,
@@ -57,6 +58,8 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
   t.ok = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
          int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(index < limit) & int(t.m > 0) & int(t.slot >= 0) &
          int(t.slot < num_slots);
+  t.plan_ok = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
+              int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots);
   return t;
 }
 

@@ -1,0 +1,527 @@
+// The small-tile fused apply of decode.hip (one workgroup per (<= 16 tokens of one slot, column
+// range), both products on the matrix cores; same arithmetic, same order, same bits) with the grid
+// laid over the SLOTS instead of over the tiles.  Computes what the reference computes with a
+// shrink launch, a temporary [slices, T, r] tensor and one or two expand launches
+// (nanovllm_voxcpm/lora.py:291-381, lora_ops/triton_ops/lora_shrink_op.py:16-173,
+// lora_expand_op.py:11-91).
+//
+// Why a second grid.  A decode launch lives for three to five trips to memory, and in the
+// tile-major kernel the first of them fetches nothing but the 128-byte tile record: which slot a
+// workgroup serves is written there, so not one operand can be requested before it has arrived.
+// More than half of a decode launch's bytes are A[slot] and B[slot], and their addresses need the
+// slot id only.  Here the slot id IS the workgroup index: workgroup (x, range, z) serves slot
+// 8 z + x, so it requests the slot's record (its first sixteen tokens) and right behind it, without
+// waiting, every A and B line it will need; the record is waited for while the weights are on
+// their way, and only the x and y rows (whose addresses are token indices) hang on it.  For that
+// to be true the weight pointers must not need a fetch either: they are leading kernel arguments,
+// which arrive preloaded in scalar registers with the wavefront (14 dwords: the record list, two
+// slices' A and B, their widths, and a packed word).  A slot without tokens costs its workgroups
+// the weight lines they requested in vain; they leave as soon as the record says so.
+//
+// Tiles behind a slot's first sixteen tokens are taken by further workgroups of the same launch
+// (z beyond the slot layers), which learn their slot from their record like the tile-major
+// kernel: a batch with every token on one adapter spreads over as many workgroups as before.
+#include "common.h"
+#include "launch.h"
+
+namespace mlora {
+
+namespace {
+
+constexpr int kNW = 8;  // wavefronts per workgroup
+
+MLORA_TRACE_DECL
+
+// What a workgroup needs to know of its column range.
+struct Range {
+  const void* a;
+  const void* b;
+  int n, y_col, n0, n1;
+};
+
+// One tile.  EARLY: the slot is known from the workgroup index (slot_early) and the weights are
+// requested before the record has arrived; otherwise the record names the slot.
+// The operand path is the staged one of decode.hip: x rows and A rows of a wavefront's K range are
+// fetched row-contiguously (sixteen lanes per 256 bytes of a row), turned into MFMA operand layout
+// through a private LDS block per wavefront, and the expand runs with the tokens as MFMA rows.
+template <typename T, int R, int KSPW, bool MASKED, int SA, bool EARLY>
+__device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const int slot_early, const int early_ok, const Range sp,
+                                          const int y_col0, const int y_col1, const bool second, const void* __restrict__ xv, void* __restrict__ yv_, const int64_t xs, const int64_t ys,
+                                          const int num_slots, const float scaling, const int32_t* __restrict__ eff_rank,
+                                          const uint32_t check, int32_t* __restrict__ plan_hdr, float* __restrict__ s_red,
+                                          T* __restrict__ s_hi, T* __restrict__ s_lo, i32x4* __restrict__ s_stage) {
+  constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
+  constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
+  constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
+  constexpr int NT = kNW * kWave;
+  constexpr int ROUNDS = KSPW / 4;       // groups of four k-steps per wavefront
+  constexpr int K = 32 * kNW * KSPW;
+  constexpr int kStageRow = 17;          // 16 chunks of 16 bytes + one of padding
+  constexpr int SB = RB < 2 ? RB : 2;    // 16-rank blocks of A staged together
+  constexpr bool K16 = R == 16;          // expand on the 16x16x16 MFMA: 64-bit operand pieces
+  static_assert(KSPW >= 4 && KSPW % 4 == 0, "the k-steps of a wavefront are taken four at a time");
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int lr = lane & 15, lg = lane >> 4;
+
+  // ---- requests that depend on nothing but the workgroup index --------------------------------
+  // The record comes through the scalar cache: one request per wavefront that does not queue with
+  // the vector requests behind it, and arrives in about half the time of a vector load.
+  typedef int i32x16a __attribute__((ext_vector_type(16), aligned(16)));
+  const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);                                        // slot, count, start, check
+  const i32x16a rows16 = *reinterpret_cast<const i32x16a*>(rec + MLORA_SMALL_TILE_ROWS);          // the sixteen token rows
+  int eff_early = R;
+  if constexpr (MASKED && EARLY) eff_early = eff_rank[slot_early];
+  const RankPrefetch ranks = rank_prefetch((MASKED && !EARLY) ? eff_rank : nullptr, num_slots, lane);
+  if constexpr (EARLY) __builtin_amdgcn_sched_barrier(0);  // the record's requests go out first
+
+  const int ks0 = wave * KSPW;
+  i32x4 ast[RB][4 * ROUNDS];
+  Pack8 bop[SA][4][KSTEPS];
+  // every A line of this wavefront's K range and the B rows of its spans
+  auto request_weights = [&](const int slot, const int rb_n) {
+    const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int64_t koff = static_cast<int64_t>(ks0 + 4 * r) * 32 + (lane & 15) * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const int rr = rb * 16 + 4 * lg + i;
+          if (!MASKED || EARLY || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          else ast[rb][4 * r + i] = i32x4{0, 0, 0, 0};
+        }
+      }
+    }
+    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
+#pragma unroll
+    for (int s = 0; s < SA; ++s) {
+      const int c0 = sp.n0 + (wave + s * kNW) * 64;
+      // requested whether the span exists or not (addresses clamped into the range)
+      if constexpr (K16) {
+        // a span's 64 B rows of 32 bytes are 2 KB of contiguous memory: fetched as such
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          int n = c0 + 32 * h + (lane >> 1);
+          n = n < sp.n1 ? n : sp.n1 - 1;
+          bop[s][h][0].raw = load128(B + static_cast<int64_t>(n) * R + (lane & 1) * 8);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          int n = c0 + 4 * lr + j;
+          n = n < sp.n1 ? n : sp.n1 - 1;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int kc = (lg + 4 * ks) & (R / 8 - 1);
+            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          }
+        }
+      }
+    }
+  };
+  // The requests made in vain by a workgroup that turns out to have no work: waited for, and named
+  // as used on that path too, so that the compiler cannot move them behind the test on the record
+  // (left to itself it sinks every load into the only path that uses it).
+  auto settle_requests = [&]() {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int j = 0; j < 4 * ROUNDS; ++j) asm volatile("" ::"v"(ast[rb][j]));
+#pragma unroll
+    for (int s = 0; s < SA; ++s)
+#pragma unroll
+      for (int j = 0; j < (K16 ? 2 : 4); ++j)
+#pragma unroll
+        for (int ks = 0; ks < (K16 ? 1 : KSTEPS); ++ks) asm volatile("" ::"v"(bop[s][j][ks].raw));
+  };
+  if constexpr (EARLY) request_weights(slot_early, RB);
+  // (everything above is requested before anything below is scheduled)
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the record is here (the weights, when requested early, are still on their way) ---------
+  const int slot = EARLY ? slot_early : rec0[0];
+  const int m = rec0[1];
+  const int matches = int(static_cast<uint32_t>(rec0[3]) == check);
+  // (every word of the record takes part in the test: a word that nothing reads is a register the
+  // compiler hands out again while the request is still on its way, and the write to it then
+  // waits for the record in the middle of the requests for the weights)
+  const int usable = matches & early_ok & int(m > 0) & int(slot >= 0) & int(slot < num_slots) & int(sp.n0 < sp.n1) &
+                     int(rows16[0] >= 0) & int(rec0[2] >= 0) & int(!EARLY || rec0[0] == slot_early);
+  if (!usable) {
+    // a plan that was built for another batch shape (or never built): count the launch that found
+    // it so, once (the first workgroup's record exists in every plan)
+    if (!matches && EARLY && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0 && plan_hdr)
+      atomicAdd(plan_hdr + MLORA_PLAN_REJECTED, 1);
+    if constexpr (EARLY) settle_requests();
+    return;
+  }
+  MLORA_STAMP(1);
+  // tokens 4*lg .. 4*lg+3 of this lane group
+  i32x4 rows4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) rows4[i] = lg == 0 ? rows16[i] : lg == 1 ? rows16[4 + i] : lg == 2 ? rows16[8 + i] : rows16[12 + i];
+  // (the column offset of the slice inside y comes with the arguments that are not preloaded:
+  // selected here, behind the wait for the record, it holds nothing up)
+  const int y_col = second ? y_col1 : y_col0;
+
+  int eff = R;
+  if constexpr (MASKED) {
+    if constexpr (EARLY) {
+      const int e = __builtin_amdgcn_readfirstlane(eff_early);
+      eff = e < 0 ? 0 : e > R ? R : e;
+    } else {
+      eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
+    }
+    if (eff == 0) {
+      if constexpr (EARLY) settle_requests();
+      return;
+    }
+  }
+  const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
+  if constexpr (!EARLY) request_weights(slot, rb_n);
+
+  // ---- the rows the record names --------------------------------------------------------------
+  i32x4 xst[4 * ROUNDS];
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int64_t koff = static_cast<int64_t>(ks0 + 4 * r) * 32 + (lane & 15) * 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xst[4 * r + i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
+  }
+  uint2 yq[SA][4];  // four columns of four tokens per lane and span
+  T* const ycols = static_cast<T*>(yv_) + y_col;
+  auto request_y = [&](int c0, uint2(&yy)[4]) {
+    const int c = c0 + 4 * lr < sp.n1 ? c0 + 4 * lr : sp.n1 - 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) yy[i] = *reinterpret_cast<const uint2*>(ycols + static_cast<int64_t>(rows4[i]) * ys + c);
+  };
+#pragma unroll
+  for (int s = 0; s < SA; ++s) request_y(sp.n0 + (wave + s * kNW) * 64, yq[s]);
+  MLORA_STAMP(2);  // every load is issued
+
+  // ---- shrink: H[token, rank] partial over this wavefront's K range ----------------------------
+  f32x4 acc[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  Pack8 xa[4], aw[RB][4];
+  i32x4* stage = s_stage + wave * (1 + SB) * 16 * kStageRow;
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[4 * r + i];
+#pragma unroll
+    for (int p = 0; p < RB / SB; ++p) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int sb = 0; sb < SB; ++sb) {
+          i32x4 v = ast[p * SB + sb][4 * r + i];
+          // rank blocks the adapter does not have were requested before its rank was known: they
+          // never reach a multiplier
+          if (MASKED && EARLY && RB > 1 && p * SB + sb >= rb_n) v = i32x4{0, 0, 0, 0};
+          stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = v;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+#pragma unroll
+        for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
+      }
+      __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass or round (and later by the expand)
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+    }
+  }
+
+  // Sum the K-partials of the wavefronts.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
+  MLORA_STAMP(3);
+  __syncthreads();
+  MLORA_STAMP(4);
+  for (int e = tid; e < RB * 256; e += NT) {
+    const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+    const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+    if (r < R) {
+      const float v = (!MASKED || r < eff) ? sum * scaling : 0.f;  // ranks the adapter does not have contribute nothing
+      const T hi = from_f32<T>(v);
+      s_hi[tok * HSTRIDE + r] = hi;
+      s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+    }
+  }
+  __syncthreads();
+  MLORA_STAMP(5);  // the intermediate is in LDS
+
+  // ---- expand: tokens as MFMA rows, lane holds out[token 4 * lg + i][column c0 + 4 * lr + j] ----
+  Pack8 hop[KSTEPS], hlo[KSTEPS];
+  uint2 hop16 = {0, 0}, hlo16 = {0, 0};
+  if constexpr (K16) {
+    hop16 = *reinterpret_cast<const uint2*>(&s_hi[lr * HSTRIDE + 4 * lg]);
+    hlo16 = *reinterpret_cast<const uint2*>(&s_lo[lr * HSTRIDE + 4 * lg]);
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const int kc = lg + 4 * ks;
+      if (kc * 8 < R) {
+        hop[ks].raw = load128(&s_hi[lr * HSTRIDE + kc * 8]);
+        hlo[ks].raw = load128(&s_lo[lr * HSTRIDE + kc * 8]);
+      } else {
+        hop[ks].raw = i32x4{0, 0, 0, 0};
+        hlo[ks].raw = i32x4{0, 0, 0, 0};
+      }
+    }
+  }
+  auto finish_span = [&](int c0, Pack8(&bo)[4][KSTEPS], uint2(&yy)[4]) {
+    f32x4 out[4];
+    uint2 pieces[4];
+    if constexpr (K16) {
+      if (MASKED && eff < R) {
+        mask_ranks(bo[0][0], (lane & 1) * 8, eff);
+        mask_ranks(bo[1][0], (lane & 1) * 8, eff);
+      }
+      // B rows -> operand pieces through the wavefront's LDS block: four rows (128 bytes) per
+      // group, groups 144 bytes apart.  MFMA j of lane (lr, lg) takes ranks 4*lg .. 4*lg+3 of
+      // column c0 + 4*lr + j.
+      char* blk = reinterpret_cast<char*>(stage);
+      *reinterpret_cast<i32x4*>(blk + (lane >> 3) * 144 + (lane & 7) * 16) = bo[0][0].raw;
+      *reinterpret_cast<i32x4*>(blk + ((lane >> 3) + 8) * 144 + (lane & 7) * 16) = bo[1][0].raw;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pieces[j] = *reinterpret_cast<const uint2*>(blk + lr * 144 + j * 32 + lg * 8);
+      __builtin_amdgcn_wave_barrier();
+    } else if (MASKED && eff < R) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) mask_ranks(bo[j][ks], ((lg + 4 * ks) & (R / 8 - 1)) * 8, eff);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      out[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if constexpr (K16) {
+        const uint2 piece = pieces[j];
+        out[j] = Mma16<T>::run(hlo16, piece, out[j]);
+        out[j] = Mma16<T>::run(hop16, piece, out[j]);
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          out[j] = Mma<T>::run(hlo[ks], bo[j][ks], out[j]);
+          out[j] = Mma<T>::run(hop[ks], bo[j][ks], out[j]);
+        }
+      }
+    }
+    const int c = c0 + 4 * lr;
+    // (the y values are taken as they are only here: unpacked where they were requested, the
+    // wavefront would wait for their arrival before the shrink)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(yy[i].x), "+v"(yy[i].y));
+    if (c < sp.n1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (4 * lg + i < m) {
+          union { uint2 raw; T e[4]; } v;
+          v.raw = yy[i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v.e[j] = from_f32<T>(to_f32(v.e[j]) + out[j][i]);
+          *reinterpret_cast<uint2*>(ycols + static_cast<int64_t>(rows4[i]) * ys + c) = v.raw;
+        }
+      }
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < SA; ++s) {
+    const int c0 = sp.n0 + (wave + s * kNW) * 64;
+    if (c0 < sp.n1) finish_span(c0, bop[s], yq[s]);
+  }
+  MLORA_STAMP(6);
+#ifdef MLORA_TRACE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  MLORA_STAMP(7);
+  __syncthreads();
+  MLORA_STAMP(8);
+#endif
+}
+
+// Leading arguments up to `packed` (13 dwords) arrive preloaded in scalar registers: everything the
+// early requests need.  packed = columns per range / 64 | ranges of slice 0 << 8 | slots << 16.
+// A launch of one slice passes n1 = 0 (blockIdx.y never reaches a second slice).
+template <typename T, int R, int KSPW, bool MASKED, int SA>
+__global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restrict__ recs, const void* __restrict__ a0,
+                                                          const void* __restrict__ b0, const void* __restrict__ a1,
+                                                          const void* __restrict__ b1, int n0, int n1, uint32_t packed,
+                                                          const void* __restrict__ xv, void* __restrict__ yv_, int64_t xs, int64_t ys,
+                                                          int y_col0, int y_col1, uint32_t check, float scaling,
+                                                          const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr) {
+  constexpr int RB = (R + 15) / 16;
+  constexpr int HSTRIDE = R + 8;
+  constexpr int kStageRow = 17;
+  constexpr int SB = RB < 2 ? RB : 2;
+  __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
+  __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) i32x4 s_stage[kNW * (1 + SB) * 16 * kStageRow];
+  MLORA_STAMP(0);
+
+  const int nt = static_cast<int>(packed & 255u) * 64, ranges0 = static_cast<int>((packed >> 8) & 255u);
+  const int num_slots = static_cast<int>(packed >> 16);
+  const int ri = blockIdx.y;
+  const bool second = ri >= ranges0;
+  Range sp;
+  sp.a = second ? a1 : a0;
+  sp.b = second ? b1 : b0;
+  sp.n = second ? n1 : n0;
+  sp.y_col = 0;  // (selected inside, late)
+  sp.n0 = (second ? ri - ranges0 : ri) * nt;
+  sp.n1 = sp.n0 + nt < sp.n ? sp.n0 + nt : sp.n;
+
+  // grid (8, column ranges, slot layers + layers of further tiles): blockIdx.x is the XCD, so a
+  // slot's column ranges share an L2
+  const int zslots = (num_slots + 7) >> 3;
+  if (static_cast<int>(blockIdx.z) < zslots) {
+    const int s = blockIdx.z * 8 + blockIdx.x;  // its record exists: the list is rounded up to eight
+    const int slot = s < num_slots ? s : num_slots - 1;
+    slot_tile<T, R, KSPW, MASKED, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
+                                            scaling, eff_rank, check, plan_hdr, s_red, s_hi, s_lo, s_stage);
+  } else {
+    const int q = zslots * 8 + (blockIdx.z - zslots) * 8 + blockIdx.x;
+    slot_tile<T, R, KSPW, MASKED, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots, scaling,
+                                             eff_rank, check, plan_hdr, s_red, s_hi, s_lo, s_stage);
+  }
+}
+
+struct Launch {
+  const MloraAddArgs* a;
+  dim3 grid;
+  uint32_t packed;
+  int widest;
+};
+
+template <typename T, int R, int KSPW, bool MASKED, int SA>
+void launch_spans(const Launch& l) {
+  const MloraAddArgs* a = l.a;
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+  const MloraSlice& s0 = a->slices[0];
+  const MloraSlice s1 = a->num_slices > 1 ? a->slices[1] : MloraSlice{nullptr, nullptr, 0, 0};
+  hipLaunchKernelGGL((slot_kernel<T, R, KSPW, MASKED, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+                     a->plan + lay.slotrec_off, s0.a, s0.b, s1.a, s1.b, s0.n, s1.n, l.packed, a->x, a->y, a->x_stride, a->y_stride,
+                     s0.y_col, s1.y_col, static_cast<uint32_t>(MLORA_PLAN_CHECK(a->num_tokens, a->num_slots)), a->scaling,
+                     a->effective_rank, const_cast<int32_t*>(a->plan));
+}
+
+template <typename T, int R, int KSPW>
+void launch_one(const Launch& l) {
+  if (l.a->effective_rank) {
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, true, 1>(l);
+    else launch_spans<T, R, KSPW, true, 2>(l);
+  } else {
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, false, 1>(l);
+    else launch_spans<T, R, KSPW, false, 2>(l);
+  }
+}
+
+template <typename T>
+bool launch_rank(const Launch& l, int r, int kspw) {
+  if (kspw == 4) {
+    switch (r) {
+      case 8: launch_one<T, 8, 4>(l); return true;
+      case 16: launch_one<T, 16, 4>(l); return true;
+      case 32: launch_one<T, 32, 4>(l); return true;
+      case 64: launch_one<T, 64, 4>(l); return true;
+    }
+  } else if (kspw == 16) {
+    switch (r) {
+      case 8: launch_one<T, 8, 16>(l); return true;
+      case 16: launch_one<T, 16, 16>(l); return true;
+    }
+  }
+  return false;
+}
+
+int kspw_of(const MloraAddArgs* a) { return a->k % (32 * kNW) == 0 ? a->k / (32 * kNW) : 0; }
+
+}  // namespace
+
+// K = 1024 at every rank, K = 4096 up to rank 16 (what fits the register file as one batch of
+// loads), one or two slices (what fits the preloaded arguments), 16-bit elements.
+bool slot_supported(const MloraAddArgs* a) {
+  if (a->dtype != MLORA_DTYPE_BF16 && a->dtype != MLORA_DTYPE_F16) return false;
+  if (a->num_slices < 1 || a->num_slices > 2 || !a->plan) return false;
+  long long cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) {
+    if (a->slices[i].n <= 0) return false;
+    cols += a->slices[i].n;
+  }
+  if (cols > 200 * 1024) return false;  // at most 255 column ranges of up to 1024 columns
+  const int kspw = kspw_of(a);
+  if (kspw == 4) return a->r == 8 || a->r == 16 || a->r == 32 || a->r == 64;
+  if (kspw == 16) return a->r == 8 || a->r == 16;
+  return false;
+}
+
+void slot_trace_set(void* buf) {
+#ifdef MLORA_TRACE
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(trace_buf), &buf, sizeof(buf));
+#else
+  (void)buf;
+#endif
+}
+
+// Columns per range: as in the tile-major launch, sized for 150-250 workgroups; at most 1024 (two
+// 64-column spans per wavefront, all loads in registers).
+int range_columns(const MloraAddArgs* a) {
+  long long cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+  const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
+  const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
+  const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
+  int nt = static_cast<int>(cols * tiles / 160);
+  if (nt > 1024) nt = 1024;
+  if (nt < 128) nt = 128;
+  nt = (nt + 63) & ~63;
+  while (nt < 1024) {
+    int total = 0;
+    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
+    if (total <= 32) break;
+    nt *= 2;
+  }
+  return nt > 1024 ? 1024 : nt;
+}
+
+int launch_slot(const MloraAddArgs* a) {
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+  const int nt = range_columns(a);
+  const int ranges0 = (a->slices[0].n + nt - 1) / nt;
+  const int total = ranges0 + (a->num_slices > 1 ? (a->slices[1].n + nt - 1) / nt : 0);
+  if (total > 255) {
+    set_error("mlora_add_lora(slot-major): %d column ranges exceed 255", total);
+    return MLORA_E_UNSUPPORTED;
+  }
+  Launch l;
+  l.a = a;
+  l.packed = static_cast<uint32_t>(nt / 64) | (static_cast<uint32_t>(ranges0) << 8) | (static_cast<uint32_t>(a->num_slots) << 16);
+  l.widest = 0;
+  for (int i = 0; i < a->num_slices; ++i) {
+    const int w = a->slices[i].n < nt ? a->slices[i].n : nt;
+    if (w > l.widest) l.widest = w;
+  }
+  l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>((lay.cap_slotrec + lay.cap_over) / 8));
+  const int kspw = kspw_of(a);
+  const bool ok = a->dtype == MLORA_DTYPE_BF16 ? launch_rank<__bf16>(l, a->r, kspw) : launch_rank<_Float16>(l, a->r, kspw);
+  if (!ok) {
+    set_error("mlora_add_lora(slot-major): unsupported rank %d / K %d", a->r, a->k);
+    return MLORA_E_UNSUPPORTED;
+  }
+  return check_launch("mlora_add_lora(small tiles, one workgroup per slot and column range)");
+}
+
+}  // namespace mlora

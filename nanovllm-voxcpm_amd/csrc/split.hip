@@ -136,6 +136,8 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
     }
   };
   if (!usable) {
+    count_rejected_plan(plan, hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE && hdr0[MLORA_PLAN_NUM_TOKENS] == T_ &&
+                                  hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots);
     count_done();
     return;
   }

@@ -22,9 +22,9 @@ MAX_SLOTS = 1024
 MAX_RANK = 256
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
-FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT, FORM_FUSED = 0, 1, 2, 3, 4, 5, 6
+FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT, FORM_FUSED, FORM_SLOT = 0, 1, 2, 3, 4, 5, 6, 7
 FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA, "split": FORM_SPLIT,
-         "fused": FORM_FUSED}
+         "fused": FORM_FUSED, "slot": FORM_SLOT}
 
 PLAN_HEADER_WORDS = 16
 (
@@ -39,7 +39,9 @@ PLAN_HEADER_WORDS = 16
     PLAN_TILES_LONG_SMALL,
     PLAN_TILES_LONG_BIG,
     PLAN_MAX_SEGMENT,
-) = range(11)
+    PLAN_TILES_OVER,
+    PLAN_REJECTED,
+) = range(13)
 PLAN_MAGIC_VALUE = 0x4D4C5031
 SEGMENT_THRESHOLD, TILE_SMALL, TILE_BIG = 16, 16, 64
 SMALL_TILE_WORDS, SMALL_TILE_ROWS, BIG_TILE_WORDS = 32, 4, 4

@@ -133,6 +133,11 @@ class _LoRALayerBase(nn.Module):
         if context.token_to_slot is None:
             return None
         meta = context._cached_metadata
+        # (a field assigned on the installed context without installing it again, as the
+        # reference's mutable dataclass allows, makes the cached view stale: compared by identity)
+        if meta is not None and (meta.token_to_slot is not context.token_to_slot or meta.no_lora_flag != context.no_lora_flag):
+            context._segment_plans.clear()
+            meta = None
         if meta is None:
             meta = LoRAMetadata(
                 token_to_slot=context.token_to_slot,

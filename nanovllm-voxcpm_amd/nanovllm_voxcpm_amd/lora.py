@@ -143,8 +143,9 @@ class HipLoRABackend:
         * a metadata object made from a ``LoRAContext`` carries the context's own plan table
           (``_mlora_context_plans``).  The plan is then a derived array of the context, like the
           sorted indices and counts the reference keeps there: it lives until the context is
-          installed again, and whoever refreshes the context's buffers in place
-          (``graph_meta.copy_lora_domain_to_graph_vars``) drops it;
+          installed again, is keyed by the slot vector's in-place version where the tensor has
+          one, and whoever refreshes the context's buffers in a way the version does not see
+          (``graph_meta.copy_lora_domain_to_graph_vars``, inference tensors) drops it;
         * any other metadata object gets a table keyed by the slot vector's address, length and
           in-place version.  Inference tensors have no version counter, so an in-place rewrite
           could not be noticed: for them nothing is kept and every call builds its plan.
@@ -158,13 +159,17 @@ class HipLoRABackend:
             return build_segment_plan(tts, max_slots)  # converted / foreign vector: do not cache
         if capture is None:
             capture = _hip.stream_capture_id(tts.device)
+        try:
+            version = own._version
+        except RuntimeError:  # inference tensors carry no version counter
+            version = None
         cache = getattr(metadata, _CONTEXT_PLANS_ATTR, None)
         if cache is not None:
-            key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, capture)
+            # the version (where the tensor has one) catches an in-place rewrite that nobody
+            # announced; writes that bypass the counter are announced by whoever makes them
+            key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, capture)
         else:
-            try:
-                version = own._version
-            except RuntimeError:  # inference tensors carry no version counter
+            if version is None:
                 return build_segment_plan(tts, max_slots)
             key = (tts.data_ptr(), tts.numel(), max_slots, tts.device, version, capture)
             cache = getattr(metadata, _PLAN_ATTR, None)

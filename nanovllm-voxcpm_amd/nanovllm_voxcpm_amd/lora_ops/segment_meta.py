@@ -37,6 +37,13 @@ class SegmentPlan:
         """Header words copied to the host (synchronises; diagnostics and tests only)."""
         return self.workspace[: _hip.PLAN_HEADER_WORDS].tolist()
 
+    def rejected_launches(self) -> int:
+        """How many launches found this plan built for another batch shape (or not built at all)
+        and therefore left y untouched.  The C-ABI returns 0 for such a launch - only the device
+        sees the mismatch - so a native caller that reuses plans checks this word; the Python
+        boundary builds its plans itself and never gets there.  Synchronises."""
+        return int(self.workspace[_hip.PLAN_REJECTED].item())
+
 
 def build_segment_plan(token_to_slot: torch.Tensor, max_slots: int) -> SegmentPlan:
     """Group the tokens by slot on the device; no host synchronisation."""

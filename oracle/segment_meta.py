@@ -121,3 +121,22 @@ def plan_tiles(token_to_slot: list[int], max_slots: int, threshold: int = 16, sm
             for j in range(0, c, big):
                 long_big.append((slot, off + j, min(big, c - j)))
     return short_small, long_small, long_big
+
+
+def plan_tiles_by_slot(token_to_slot: list[int], max_slots: int, small: int = 16):
+    """The same small tiles listed by slot: ``first[s]`` = (count, first position in sorted_idx) of
+    the first tile of slot id ``s`` for every s in [0, max_slots) (count 0 and the slot's position
+    in the running totals for a slot without tokens), and ``further`` = (slot, first position,
+    count) of every tile behind a slot's first one, slots ascending.  Slot ids >= max_slots count
+    as -1.  (No reference counterpart, like plan_tiles.)"""
+    cleaned = [s if 0 <= s < max_slots else -1 for s in token_to_slot]
+    _, active, counts, offsets = engine_layout(cleaned)
+    per_slot = dict(zip(active, zip(counts, offsets)))
+    first, further, run = [], [], 0
+    for s in range(max_slots):
+        c, off = per_slot.get(s, (0, run))
+        first.append((min(c, small), off))
+        for j in range(small, c, small):
+            further.append((s, off + j, min(small, c - j)))
+        run = off + c
+    return first, further

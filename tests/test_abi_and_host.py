@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     assert declared and set(declared) == set(_hip.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mlora_abi_version() == int(re.search(r"#define MLORA_ABI_VERSION (\d+)", HEADER.read_text()).group(1)) == 3
+    assert lib.mlora_abi_version() == int(re.search(r"#define MLORA_ABI_VERSION (\d+)", HEADER.read_text()).group(1)) == 4
     assert "gfx950" in _hip.build_info()
 
 
@@ -64,7 +64,9 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
     text = HEADER.read_text()
     for macro, value in (("MLORA_MAX_SLICES", 8), ("MLORA_MAX_SLOTS", _hip.MAX_SLOTS), ("MLORA_MAX_RANK", _hip.MAX_RANK),
                          ("MLORA_TILE_SMALL", 16), ("MLORA_SMALL_TILE_WORDS", _hip.SMALL_TILE_WORDS), ("MLORA_BIG_TILE_WORDS", _hip.BIG_TILE_WORDS), ("MLORA_TILE_BIG", 64), ("MLORA_SEGMENT_THRESHOLD", 16),
-                         ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS), ("MLORA_FORM_SPLIT", _hip.FORM_SPLIT)):
+                         ("MLORA_PLAN_HEADER_WORDS", _hip.PLAN_HEADER_WORDS), ("MLORA_FORM_SPLIT", _hip.FORM_SPLIT),
+                         ("MLORA_FORM_SLOT", _hip.FORM_SLOT), ("MLORA_PLAN_TILES_OVER", _hip.PLAN_TILES_OVER),
+                         ("MLORA_PLAN_REJECTED", _hip.PLAN_REJECTED), ("MLORA_PLAN_MAX_SEGMENT", _hip.PLAN_MAX_SEGMENT)):
         assert re.search(rf"#define {macro} {value}\b", text), macro
     assert re.search(r"#define MLORA_WORKSPACE_HEAD_BYTES \(16384 \+ \(4 << 20\) \+ \(64 << 10\)\)", text) and _hip.WORKSPACE_HEAD_BYTES == 16384 + (4 << 20) + (64 << 10)
     assert re.search(r"#define MLORA_STATIC_SCRATCH_BYTES \(16u << 20\)", text) and _hip.STATIC_SCRATCH_BYTES == 16 << 20
@@ -120,6 +122,16 @@ def test_arguments_are_rejected_before_any_launch():
     assert lib.mlora_add_workspace_bytes(256, 3, 16, 2) == _hip.WORKSPACE_HEAD_BYTES + 4 * 256 * 3 * 16 * 4
     assert lib.mlora_plan_workspace_bytes(256, 32) == 4 * _hip.plan_workspace_words(256, 32) > 0
     assert lib.mlora_plan_workspace_bytes(-1, 2) == 0
+    # the plan's layout as documented: header, sorted indices, dense counts and offsets, small tiles, big
+    # tiles and their row lists, then a 128-byte record per slot id and per further tile
+    def words(t, l):
+        r4 = lambda v: (v + 3) & ~3  # noqa: E731
+        small_off = (16 + r4(t) + r4(l + 1) + r4(l + 2) + 31) & ~31
+        cap_small = ((t + 15) // 16 + min(l, t) + 7) & ~7
+        cap_big = (t // 64 + min(l, t) + 31) & ~31
+        return small_off + 32 * cap_small + (4 + 64) * cap_big + 32 * ((l + 7) & ~7) + 32 * ((t // 16 + 7) & ~7)
+    for t, l in ((256, 32), (1, 1), (8192, 128), (20000, 1024), (15, 600)):
+        assert lib.mlora_plan_workspace_bytes(t, l) == 4 * words(t, l), (t, l)
 
 
 def test_no_gpu_means_unavailable_and_loud():

@@ -145,6 +145,40 @@ def test_config2_decode_bf16(name, form):
     _check(got, y0, exact, mag, slots, f"config2/{name}/{form}")
 
 
+def _slot_form_batches(T, L, seed):
+    """Slot vectors that exercise the slot-major grid: uniform decode ids; ids with rows without
+    adapter and slot ids nobody uses; every token on one adapter (all tiles but the first are
+    further tiles); a batch in which only the last slot id is used."""
+    g = torch.Generator().manual_seed(seed)
+    uniform = torch.randint(0, L, (T,), generator=g, dtype=torch.int32)
+    sparse = torch.randint(-1, max(1, L // 2), (T,), generator=g, dtype=torch.int32)
+    one = torch.full((T,), L - 1 if L > 1 else 0, dtype=torch.int32)
+    one[::5] = -1
+    skew = uniform.clone()
+    skew[: (2 * T) // 3] = min(2, L - 1)
+    return {"uniform": uniform, "sparse": sparse, "one adapter": one, "skewed": skew}
+
+
+@pytest.mark.parametrize("name,rank,T,L", [("o", 16, 256, 32), ("gate_up", 16, 256, 32), ("down", 16, 256, 32), ("o", 32, 64, 32),
+                                           ("gate_up", 64, 100, 5), ("o", 8, 37, 13), ("down", 8, 300, 9), ("gate_up", 32, 19, 64)])
+def test_slot_major_grid_gives_the_bits_of_the_tile_major_grid(name, rank, T, L):
+    """The slot-major form requests a slot's weights before its record has arrived; what it computes
+    is the small-tile form's arithmetic in the same order, so its results are the oracle's and,
+    bit for bit, those of the tile-major grid - for slots without tokens, slot ids that are not a
+    multiple of eight, rows without adapter and slots with several tiles alike."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    proj = _make(name, L, rank, torch.bfloat16, seed=170 + rank)
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=171, device="cuda")
+    for tag, slots in _slot_form_batches(T, L, 172 + T).items():
+        print(f"slot-major {name} r={rank} T={T} L={L} {tag}", flush=True)
+        slots = slots.cuda()
+        got = _apply("slot", proj, x, y0.clone(), slots)
+        exact, mag = _exact(proj, x, y0, slots)
+        _check(got, y0, exact, mag, slots, f"slot-major/{name}/r{rank}/{tag}")
+        assert torch.equal(got, _apply("mfma", proj, x, y0.clone(), slots)), tag
+
+
 @pytest.mark.parametrize("rank", [16, 64])
 @pytest.mark.parametrize("name", ["gate_up", "o"])
 def test_small_tile_form_is_the_same_for_every_column_range_width(name, rank, monkeypatch):
@@ -887,7 +921,37 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
     cap_big = (T // 64 + min(L, T) + 31) & ~31
     bigrows_off = big_off + 4 * cap_big
-    assert len(ws) == bigrows_off + 64 * cap_big
+    slotrec_off = bigrows_off + 64 * cap_big
+    cap_slotrec = (L + 7) & ~7
+    over_off = slotrec_off + 32 * cap_slotrec
+    cap_over = (T // 16 + 7) & ~7
+    assert len(ws) == over_off + 32 * cap_over
+    # the small tiles once more, by slot: a record per slot id, then the further tiles of every slot
+    first, further = meta_oracle.plan_tiles_by_slot(slots_l, L)
+    check = (0x4D4C5031 ^ T ^ (L << 20)) & 0xFFFFFFFF
+    check = check - (1 << 32) if check >= 1 << 31 else check  # as the int32 word reads
+    assert hdr[_hip.PLAN_TILES_OVER] == len(further) and hdr[_hip.PLAN_REJECTED] == 0
+    assert len(further) <= T // 16
+
+    def record(at):
+        return ws[at : at + 32]
+
+    for slot, (count, start) in enumerate(first):
+        rec = record(slotrec_off + 32 * slot)
+        assert rec[:4] == [slot, count, start, check]
+        own = s[start : start + count]
+        assert rec[4:20] == ([own[j % count] for j in range(16)] if count else [0] * 16) and rec[20:] == [0] * 12
+    for slot in range(L, cap_slotrec):
+        assert record(slotrec_off + 32 * slot) == [-1, 0, 0, check] + [0] * 28
+    for q, (slot, start, count) in enumerate(further):
+        rec = record(over_off + 32 * q)
+        assert rec[:4] == [slot, count, start, check]
+        own = s[start : start + count]
+        assert rec[4:20] == [own[j % count] for j in range(16)] and rec[20:] == [0] * 12
+    for q in range(len(further), cap_over):
+        assert record(over_off + 32 * q) == [-1, 0, 0, check] + [0] * 28
+    # both lists hold the same tiles
+    assert sorted([(sl, st, c) for sl, (c, st) in enumerate(first) if c] + further) == sorted(short + long_small)
     assert ws[sorted_off : sorted_off + len(s)] == s
     dense = [0] * (L + 1)
     for slot, n in zip(a, c):

@@ -29,7 +29,7 @@ def _poisoned(proj, ranks):
     return a, b
 
 
-@pytest.mark.parametrize("form", ["auto", "split", "mfma", "sgmv", "token"])
+@pytest.mark.parametrize("form", ["auto", "split", "mfma", "slot", "sgmv", "token"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 @pytest.mark.parametrize("tokens", [200, 3000])
 def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, form):
@@ -42,6 +42,8 @@ def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, 
 
     if form == "split" and tokens > 256:
         pytest.skip("the split form takes decode-sized batches only (its exchange area holds ~128 rank-64 partial tiles)")
+    if form == "slot" and name in ("qkv", "down"):
+        pytest.skip("the slot-major form takes one or two slices, and K = 4096 up to rank 16 only")
     print(f"rank masking {name} T={tokens} form={form}", flush=True)
     ranks = [8, 12, 16, 32, 40, 64, 0, 24]
     clean = _make(name, len(ranks), 64, torch.bfloat16, seed=800, true_ranks=ranks)
@@ -260,6 +262,87 @@ def test_context_plans_follow_an_in_place_refresh_of_graph_buffers():
             if s >= 0:
                 want[t] = x[t].double().cpu() @ a[s].T @ b[s].T
         assert torch.allclose(y.double().cpu(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("form", ["mfma", "slot", "split", "sgmv", "fused", "bgmv"])
+def test_a_plan_of_another_batch_shape_is_counted_not_followed(form):
+    """Through the C-ABI a plan built for another (num_tokens, max_slots) is only recognised on the
+    device: the call returns 0, y keeps its bits, and the launch is counted in the header of the
+    plan that was passed (MLORA_PLAN_REJECTED), where a native caller can see it.  The matching
+    plan, passed next, is followed and not counted."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
+    from nanovllm_voxcpm_amd.lora_ops import build_segment_plan
+
+    T, L = 200, 8
+    proj = _make("o", L, 16, torch.bfloat16, seed=870)
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=871, device="cuda")
+    g = torch.Generator().manual_seed(872)
+    slots = torch.randint(0, L, (T,), generator=g, dtype=torch.int32).cuda()
+    longer = torch.randint(0, L, (2 * T,), generator=g, dtype=torch.int32).cuda()
+    stale = build_segment_plan(longer, L)        # built for 400 tokens: larger than any offset a call for 200 reads
+    other_slots = build_segment_plan(torch.cat([slots, slots]), L + 8)
+    good = build_segment_plan(slots, L)
+    scratch = torch.empty(_hip.add_workspace_bytes(T, 1, 16, torch.bfloat16), dtype=torch.uint8, device="cuda")
+    _hip.workspace_init(scratch)
+    print(f"stale plan, form {form}", flush=True)
+    for plan in (stale, other_slots):
+        y = y0.clone()
+        _hip.add_lora(y, x, proj.a, proj.b, [0], slots, plan.workspace, 1.0, _hip.FORMS[form], scratch)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y0), "a plan of another batch shape was followed"
+        assert plan.rejected_launches() >= 1
+    y = y0.clone()
+    _hip.add_lora(y, x, proj.a, proj.b, [0], slots, good.workspace, 1.0, _hip.FORMS[form], scratch)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(y, y0, exact, mag, slots, f"matching plan/{form}")
+    assert good.rejected_launches() == 0
+
+
+def test_context_plans_follow_a_versioned_slot_vector_rewritten_in_place():
+    """A context that lives across steps and whose slot vector is rewritten with ``copy_`` outside
+    inference mode (nobody announces the write): the tensor's version counter is part of the key of
+    the context's plan table, so the next forward builds a new plan and follows the new slot ids.
+    A new vector put on the same context without installing it again is followed too."""
+    from nanovllm_voxcpm_amd.layers.lora import LoRALinear
+    from nanovllm_voxcpm_amd.utils.context import LoRAContext, reset_lora_context, set_lora_context
+
+    g = torch.Generator().manual_seed(835)
+    T, L = 48, 4
+    layer = LoRALinear(256, 128, bias=False, max_loras=L, max_lora_rank=16).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.zero_()
+        for s in range(L):
+            layer.set_slot_lora(s, (torch.randn(16, 256, generator=g) * 0.1).cuda(), (torch.randn(128, 16, generator=g) * 0.1).cuda(), 16, 1.0)
+    x = torch.randn(T, 256, generator=g).to(torch.bfloat16).cuda()
+    a, b = layer.lora_A.detach().double().cpu(), layer.lora_B.detach().double().cpu()
+
+    def want_for(ids):
+        want = torch.zeros(T, 128, dtype=torch.float64)
+        for t, s in enumerate(ids.tolist()):
+            if s >= 0:
+                want[t] = x[t].double().cpu() @ a[s].T @ b[s].T
+        return want
+
+    first = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32)
+    second = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32)
+    third = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32)
+    assert not torch.equal(first, second) and not torch.equal(second, third)
+    slots = first.cuda()
+    ctx = LoRAContext(token_to_slot=slots, no_lora_flag=False)
+    set_lora_context(ctx)
+    try:
+        with torch.no_grad():
+            y1 = layer(x)
+            slots.copy_(second.cuda())  # same tensor, same context, new contents, no announcement
+            y2 = layer(x)
+            y2_again = layer(x)
+            ctx.token_to_slot = third.cuda()  # a new vector on the same, still installed context
+            y3 = layer(x)
+    finally:
+        reset_lora_context()
+    assert torch.equal(y2, y2_again)
+    for got, ids in ((y1, first), (y2, second), (y3, third)):
+        assert torch.allclose(got.double().cpu(), want_for(ids), rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("name,tokens,rank", [("down", 200, 16), ("gate_up", 2000, 64)])

@@ -250,3 +250,13 @@ def test_layouts_agree_with_brute_force_sort(seed):
     assert sorted(p for (_, st, n) in long_big for p in range(st, st + n)) == sorted(
         p for (_, st, n) in long_small for p in range(st, st + n)
     )
+    # the list by slot holds exactly the small tiles, every position once, a slot's first tile
+    # under its own id and slots without tokens with count 0 at their place in the running totals
+    first, further = meta_oracle.plan_tiles_by_slot(slots, L)
+    assert len(first) == L and all(0 <= cnt <= 16 for cnt, _ in first)
+    assert sorted([(sl, st, cnt) for sl, (cnt, st) in enumerate(first) if cnt] + further) == sorted(short + long_small)
+    for sl, (cnt, st) in enumerate(first):
+        assert st == sum(1 for v in slots if 0 <= v < sl)
+        assert cnt == min(16, slots.count(sl))
+        assert all(slots[s[p]] == sl for p in range(st, st + cnt))
+    assert all(slots[s[p]] == sl for (sl, st, cnt) in further for p in range(st, st + cnt))
