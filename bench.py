@@ -116,7 +116,7 @@ def make_step(layers, slots, form: str, only: str | None = None, eff=None):
     status = backend.availability()
     if not status.available:
         raise RuntimeError(f"HIP LoRA backend unavailable: {status.reason}")
-    names = [only] if only else list(ORDER)
+    names = list(only) if isinstance(only, (tuple, list)) else [only] if only else list(ORDER)
     calls = []
     for entry in layers:
         for name in names:
@@ -213,14 +213,23 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
         one_med, _ = timed(one_layer, budget_s * 0.3)
     finally:
         torch.set_num_threads(threads)
-    model = ""
+    # the model string as the host reports it (a virtual machine may report the family name only:
+    # family / model / stepping numbers are appended, they identify the part)
+    model, ids = "", {}
     try:
         for line in Path("/proc/cpuinfo").read_text().splitlines():
-            if line.startswith("model name"):
-                model = line.split(":", 1)[1].strip()
-                break
+            if not line.strip():
+                break  # first processor only
+            key, _, val = line.partition(":")
+            key = key.strip()
+            if key == "model name":
+                model = val.strip()
+            elif key in ("cpu family", "model", "stepping"):
+                ids[key] = val.strip()
     except OSError:
         pass
+    if ids:
+        model = f"{model} (family {ids.get('cpu family', '?')} model {ids.get('model', '?')} stepping {ids.get('stepping', '?')})".strip()
     return {
         "value": round(layer_bytes / med / 1e9, 4),
         "unit": "GB/s",
@@ -421,7 +430,7 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
     if eff is not None:  # adapters of lower rank in rank-`rank` buffers, and the kernels are told
         rank_sum = int(eff[used_ids.long()].sum())
         token_rank_sum = int(eff[slots[slots >= 0].long()].sum())
-    names = [only] if only else list(ORDER)
+    names = list(only) if isinstance(only, (tuple, list)) else [only] if only else list(ORDER)
     shapes = {n: layers[0][n][0] for n in names}
     per_proj = {n: algorithmic_bytes(p.k, p.widths, t_lora, used, rank, num_tokens, rank_sum) for n, p in shapes.items()}
     per_proj_flops = {n: algorithmic_flops(p.k, p.widths, t_lora, rank, token_rank_sum) for n, p in shapes.items()}
@@ -443,8 +452,8 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
 
     # per-projection time: the same step restricted to one projection (24 launches)
     per_proj_us = {}
-    if per_projection and not only and not eager:
-        for n in ORDER:
+    if per_projection and not isinstance(only, str) and not eager:
+        for n in names:
             sub, cnt = make_step(layers, slots, form, n, eff)
             g = capture(sub)
             for _ in range(2):
@@ -707,13 +716,21 @@ def main() -> None:
         extra = {}
         for name in ("prefill", "mixed"):
             r, (wl_layers, wl_slots, _, _) = measure_workload(name, device, "auto", 5, 2, per_projection=True)
-            extra[name] = {k: r[k] for k in ("config", "us_per_step", "value", "pct_of_hbm_peak", "tflops", "pct_of_mfma_bf16_peak",
-                                             "algorithmic_bytes_per_step", "us_per_call_by_projection", "roofline")}
+            extra[name] = {k: r[k] for k in ("config", "us_per_step", "us_per_step_eager", "value", "pct_of_hbm_peak", "tflops",
+                                             "pct_of_mfma_bf16_peak", "algorithmic_bytes_per_step", "us_per_call_by_projection", "roofline")}
             extra[name]["unit"] = "GB/s"
             if name == "prefill":
                 extra[name]["latency"] = measure_long_form_latency(wl_layers, wl_slots)
             del wl_layers, wl_slots
             torch.cuda.empty_cache()
+        # the reference's own default LoRA shape (max_lora_rank 32, targets q / k / v / o only:
+        # nanovllm_voxcpm/models/voxcpm/config.py:87-90) on the same decode batch
+        r, _ = measure_workload("decode", device, "auto", 50, 10, only=("qkv", "o"), rank=32)
+        extra["reference_default"] = {k: r[k] for k in ("config", "us_per_step", "us_per_step_eager", "value", "pct_of_hbm_peak",
+                                                        "algorithmic_bytes_per_step", "calls_per_step", "us_per_call_by_projection",
+                                                        "gbs_by_projection")}
+        extra["reference_default"]["unit"] = "GB/s"
+        torch.cuda.empty_cache()
         extra["backbone"] = measure_backbone(10, 3)
         extra["unfused_ops"] = measure_unfused(layers, slots)
         torch.cuda.empty_cache()

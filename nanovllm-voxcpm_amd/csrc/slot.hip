@@ -65,11 +65,10 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   const int lr = lane & 15, lg = lane >> 4;
 
   // ---- requests that depend on nothing but the workgroup index --------------------------------
-  // The record comes through the scalar cache: one request per wavefront that does not queue with
-  // the vector requests behind it, and arrives in about half the time of a vector load.
-  typedef int i32x16a __attribute__((ext_vector_type(16), aligned(16)));
-  const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);                                        // slot, count, start, check
-  const i32x16a rows16 = *reinterpret_cast<const i32x16a*>(rec + MLORA_SMALL_TILE_ROWS);          // the sixteen token rows
+  // (the token rows as a vector load, four per lane group: all sixteen through the scalar cache
+  // into scalar registers measured slower, 556 -> 598 us per decode step in the tile-major kernel)
+  const i32x4 rows4 = *reinterpret_cast<const i32x4*>(rec + MLORA_SMALL_TILE_ROWS + 4 * lg);  // tokens 4*lg .. 4*lg+3
+  const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);                                     // slot, count, start, check
   int eff_early = R;
   if constexpr (MASKED && EARLY) eff_early = eff_rank[slot_early];
   const RankPrefetch ranks = rank_prefetch((MASKED && !EARLY) ? eff_rank : nullptr, num_slots, lane);
@@ -148,7 +147,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   // compiler hands out again while the request is still on its way, and the write to it then
   // waits for the record in the middle of the requests for the weights)
   const int usable = matches & early_ok & int(m > 0) & int(slot >= 0) & int(slot < num_slots) & int(sp.n0 < sp.n1) &
-                     int(rows16[0] >= 0) & int(rec0[2] >= 0) & int(!EARLY || rec0[0] == slot_early);
+                     int(__builtin_amdgcn_readfirstlane(rows4[0]) >= 0) & int(rec0[2] >= 0) & int(!EARLY || rec0[0] == slot_early);
   if (!usable) {
     // a plan that was built for another batch shape (or never built): count the launch that found
     // it so, once (the first workgroup's record exists in every plan)
@@ -158,10 +157,6 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
     return;
   }
   MLORA_STAMP(1);
-  // tokens 4*lg .. 4*lg+3 of this lane group
-  i32x4 rows4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) rows4[i] = lg == 0 ? rows16[i] : lg == 1 ? rows16[4 + i] : lg == 2 ? rows16[8 + i] : rows16[12 + i];
   // (the column offset of the slice inside y comes with the arguments that are not preloaded:
   // selected here, behind the wait for the record, it holds nothing up)
   const int y_col = second ? y_col1 : y_col0;

@@ -403,6 +403,13 @@ def add_lora(
             _check(lib.mlora_add_lora(C.byref(args)), "mlora_add_lora")
 
 
+def call_add_lora(args: MloraAddArgs) -> None:
+    """Enqueue the fused apply described by an argument block the caller filled and checked."""
+    rc = load().mlora_add_lora(C.byref(args))
+    if rc != 0:
+        _check(rc, "mlora_add_lora")
+
+
 def shrink(
     x: torch.Tensor, a_slices: list[torch.Tensor], out: torch.Tensor, token_to_slot: torch.Tensor, scaling: float
 ) -> None:

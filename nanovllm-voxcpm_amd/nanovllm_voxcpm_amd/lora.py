@@ -14,6 +14,8 @@ There is no host fallback: without a GPU or without the built library the probed
 from __future__ import annotations
 
 import os
+import struct
+import threading
 from dataclasses import dataclass
 from typing import Protocol
 
@@ -97,6 +99,27 @@ _PLAN_ATTR = "_mlora_segment_plans"
 _CONTEXT_PLANS_ATTR = "_mlora_context_plans"  # plan table of the LoRAContext a metadata object was made from
 
 
+# The per-step fields of MloraAddArgs as they lie in memory: stream, x, y, x_stride, y_stride,
+# token_to_slot, plan (eight bytes each, from offset 0) and num_tokens; scaling; workspace,
+# workspace_bytes, effective_rank.
+_STEP_HEAD = struct.Struct("=QQQqqQQi")
+_STEP_SCALE = struct.Struct("=f")
+_STEP_TAIL = struct.Struct("=QqQ")
+_OFF_SCALING = _hip.MloraAddArgs.scaling.offset
+_OFF_WORKSPACE = _hip.MloraAddArgs.workspace.offset
+assert _hip.MloraAddArgs.stream.offset == 0 and _hip.MloraAddArgs.num_tokens.offset == 56 and _STEP_HEAD.size == 60
+assert _hip.MloraAddArgs.effective_rank.offset == _OFF_WORKSPACE + 16
+
+
+class _CallSite:
+    """What a call of ``add_lora`` derives from its weight tensors alone, kept per set of weight
+    buffers (a LoRA linear calls with the same buffers on every step): the filled argument block
+    of the C entry point with everything but the per-step fields, and the outcome of the checks
+    that concern the weights.  One per thread and set of buffers (addresses, shapes, element type)."""
+
+    __slots__ = ("args", "view", "k", "rank", "num_slots", "dtype", "device", "widths", "weights_vectorisable", "num_slices")
+
+
 class HipLoRABackend:
     """``LoRABackend`` whose arithmetic runs in the hand-written gfx950 kernels."""
 
@@ -110,6 +133,7 @@ class HipLoRABackend:
         self._scratch: dict = {}
         self._spares: dict = {}          # device -> initialised buffer kept for the next graph capture
         self._graph_scratch: list = []   # buffers captured graphs refer to
+        self._sites = threading.local()  # per thread: weight buffers -> _CallSite
 
     # -- capability ---------------------------------------------------------------------
     def availability(self) -> LoRAAvailability:
@@ -245,6 +269,117 @@ class HipLoRABackend:
                 return False
         return True
 
+    # -- the usual call, with what the weights determine kept per set of buffers -----------------
+    def _site_for(self, a_list, b_list, widths) -> "_CallSite | None":
+        """The call site of these weight buffers, made on first use; None when the call is not of
+        the usual kind (slices of different rank or K, an empty slice, too many slices), which the
+        general path below then handles."""
+        key = []
+        for t in a_list:
+            key.append(t.data_ptr())
+            key.append(t.shape)
+        for t in b_list:
+            key.append(t.data_ptr())
+            key.append(t.shape)
+        a0 = a_list[0]
+        key.append(a0.dtype)
+        key = tuple(key)
+        table = getattr(self._sites, "table", None)
+        if table is None:
+            table = self._sites.table = {}
+        site = table.get(key)
+        if site is not None:
+            return site if site.widths == widths else None
+        if len(a_list) > _hip.MAX_SLICES or a0.dim() != 3 or any(w == 0 for w in widths):
+            return None
+        rank, k, slots = a0.size(-2), a0.size(-1), a0.size(0)
+        dev, dt = a0.device, a0.dtype
+        for a, b, w in zip(a_list, b_list, widths):
+            if a.dim() != 3 or b.dim() != 3 or a.size(-2) != rank or a.size(-1) != k or a.size(0) != slots or b.size(0) != slots:
+                return None
+            if b.size(-1) != rank or b.size(1) != w or a.device != dev or b.device != dev or a.dtype != dt or b.dtype != dt:
+                return None
+        if not a0.is_cuda or dt not in _hip._DTYPES:
+            return None
+        site = _CallSite()
+        args = site.args = _hip.MloraAddArgs()
+        args.k, args.r, args.num_slots, args.num_slices, args.dtype = k, rank, slots, len(a_list), _hip.dtype_code(dt)
+        args.form = _hip.FORMS[self.form]
+        col, ok = 0, dt in (torch.float16, torch.bfloat16) and rank in _VECTOR_RANKS and k % 8 == 0
+        for i, (a, b, w) in enumerate(zip(a_list, b_list, widths)):
+            sl = args.slices[i]
+            sl.a, sl.b, sl.n, sl.y_col = a.data_ptr(), b.data_ptr(), w, col
+            ok = ok and w % 8 == 0 and col % 8 == 0 and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0
+            col += w
+        # (no reference to the tensors is kept: the key is their addresses, shapes and element type,
+        # so whatever answers to the key later lies where the block says)
+        site.view = memoryview(args).cast("B")
+        site.k, site.rank, site.num_slots, site.dtype, site.device, site.widths = k, rank, slots, dt, dev, widths
+        site.weights_vectorisable, site.num_slices = ok, len(a_list)
+        if len(table) >= 512:
+            table.clear()
+        table[key] = site
+        return site
+
+    def _add_lora_at_site(self, outputs, target, x, a_list, b_list, indices, metadata, scaling, effective_rank) -> bool:
+        """The usual call - every slice non-empty, all of one rank and K, unit column strides - with
+        the argument block of its weight buffers reused from the last step: only what changes per
+        step (activations, slot vector, plan, scratch, stream) is entered.  Returns False, having
+        done nothing, for anything else and for everything that has to raise: the general path
+        then runs, with its checks and their messages."""
+        if x.dim() != 2 or x.stride(1) != 1 or target.dim() != 2 or target.stride(1) != 1:
+            return False
+        widths = tuple([y.size(-1) for y in outputs])
+        site = self._site_for(a_list, b_list, widths)
+        if site is None:
+            return False
+        rows = x.size(0)
+        source = metadata.token_to_slot if metadata.token_to_slot is not None else indices
+        if (x.size(1) != site.k or x.dtype != site.dtype or target.dtype != site.dtype or x.device != site.device or
+                target.device != site.device or source.device != site.device or source.numel() < rows or target.size(0) < rows or
+                source.dtype != torch.int32 or not source.is_contiguous() or source.dim() != 1):
+            return False
+        x_ptr, y_ptr, xs, ys = x.data_ptr(), target.data_ptr(), x.stride(0), target.stride(0)
+        args = site.args
+        eff_ptr = 0
+        if effective_rank is not None:
+            if (effective_rank.dtype != torch.int32 or not effective_rank.is_contiguous() or effective_rank.numel() < site.num_slots or
+                    effective_rank.device != site.device):
+                return False
+            eff_ptr = effective_rank.data_ptr()
+        dev = site.device
+        if dev.index is not None and dev.index != torch.cuda.current_device():
+            return False  # another GPU of this process: the general path makes it current
+        stream = _hip.current_stream_handle(dev)
+        plan_ptr = ws_ptr = ws_bytes = 0
+        if site.weights_vectorisable and args.form != _hip.FORM_TOKEN and not (xs % 8 or ys % 8 or x_ptr % 16 or y_ptr % 16):
+            capture = _hip.stream_capture_id(dev, stream)
+            # every LoRA linear of a step calls with the same metadata object, slot vector, stream
+            # and capture: what the last call of this thread looked up serves the next one
+            try:
+                version = source._version
+            except RuntimeError:  # inference tensors carry no version counter: nothing is remembered for them
+                version = None
+            memo = getattr(self._sites, "step", None)
+            if (memo is not None and version is not None and memo[0] is metadata and memo[1] is source and memo[2] == version and
+                    memo[3] == capture and memo[4] == stream and memo[5] == site.num_slots and memo[6] == rows):
+                plan_ptr = memo[7]
+            else:
+                tts = source if source.numel() == rows else source[:rows]
+                plan = self._plan_for(metadata, tts, site.num_slots, capture)
+                plan_ptr = plan.workspace.data_ptr()
+                # (the plan object is part of the memo: its workspace stays allocated while it is remembered)
+                self._sites.step = (metadata, source, version, capture, stream, site.num_slots, rows, plan_ptr, plan)
+            scratch = self._scratch_for(x, site.num_slices, site.rank, stream, capture)
+            ws_ptr, ws_bytes = scratch.data_ptr(), scratch.numel()
+        # the per-step fields, written in three strokes (they lie together in the block; one attribute
+        # assignment per field costs several times as much)
+        _STEP_HEAD.pack_into(site.view, 0, stream or 0, x_ptr, y_ptr, xs, ys, source.data_ptr(), plan_ptr, rows)
+        _STEP_SCALE.pack_into(site.view, _OFF_SCALING, scaling)
+        _STEP_TAIL.pack_into(site.view, _OFF_WORKSPACE, ws_ptr, ws_bytes, eff_ptr)
+        _hip.call_add_lora(args)
+        return True
+
     # -- the fused apply -------------------------------------------------------------------
     def add_lora(
         self,
@@ -278,10 +413,12 @@ class HipLoRABackend:
             raise ValueError("add_lora expects aligned y/lora_a/lora_b slice lists")
         if metadata is None:
             raise RuntimeError("LoRA metadata must be prepared by the model runner before backend execution")
-        if any(not a.is_contiguous() for a in lora_a_slices):
-            raise ValueError("add_lora expects contiguous lora_a slices")
-        if any(not b.is_contiguous() for b in lora_b_slices):
-            raise ValueError("add_lora expects contiguous lora_b slices")
+        for a in lora_a_slices:
+            if not a.is_contiguous():
+                raise ValueError("add_lora expects contiguous lora_a slices")
+        for b in lora_b_slices:
+            if not b.is_contiguous():
+                raise ValueError("add_lora expects contiguous lora_b slices")
 
         outputs = list(y_slices)
         if y_packed is not None:
@@ -296,6 +433,9 @@ class HipLoRABackend:
             outputs = list(target.split(widths, dim=-1))
 
         if metadata.no_lora_flag or x.size(0) == 0:
+            return outputs
+
+        if self._add_lora_at_site(outputs, target, x, lora_a_slices, lora_b_slices, indices, metadata, scaling, effective_rank):
             return outputs
 
         cols, col = [], 0
