@@ -246,74 +246,6 @@ def cpu_baseline(layers, slots, rank: int, budget_s: float = 20.0) -> dict:
     }
 
 
-STAMPS = {
-    "decode_kernel": ["entry", "record here", "loads issued", "wave 0 shrink done", "partials in LDS", "intermediate in LDS",
-                      "wave 0 first spans stored", "wave 0 stores acknowledged", "all waves done"],
-    "split_kernel producer": ["entry", "record here", "K part summed", "partials published"],
-    "split_kernel consumer": ["entry", "record here", None, None, "loads issued", "wait over", "intermediate in LDS",
-                              "wave 0 first spans stored", "wave 0 stores acknowledged", "all waves done"],
-    "sgmv_shrink_kernel": ["entry", "record here", "token rows requested", "first slab and x batch requested",
-                           "first piece of the slab on its way to LDS", "first slice multiplied", "partial sums issued",
-                           "partial sums acknowledged"],
-    # (the expand's stamps sit in columns 8.. of the same rows)
-    "sgmv_expand_kernel": ["entry", "records here", "token rows and first partial sums here", "intermediate in LDS",
-                           "wave 0 last item stored", "wave 0 stores acknowledged", "wave 0 first item stored"],
-}
-
-
-def run_timeline(args) -> None:
-    """In-kernel timeline of the last launch of a step restricted to one projection (24 launches on
-    24 layers' own buffers, so the traced launch reads cold data): readings of the 100 MHz clock
-    taken by thread 0 of every workgroup at fixed points of the kernel, reported in ns after the
-    earliest workgroup entered the kernel (min / median / max over the workgroups that had work).
-    Needs the trace build of the library (make -C nanovllm-voxcpm_amd/csrc trace)."""
-    import torch
-
-    from nanovllm_voxcpm_amd import _hip
-
-    device = "cuda:0"
-    layers, slots, eff = build_workload(args.workload, device, args.rank or None, args.sequences)
-    if args.hot_layers > 0:
-        layers = [layers[i % args.hot_layers] for i in range(NUM_LAYERS)]
-    step, launches = make_step(layers, slots, args.form, args.timeline, eff=None if args.no_rank_vector else eff)
-    for _ in range(3):
-        step()
-    torch.cuda.synchronize()
-    buf = torch.zeros(8192, 16, dtype=torch.int64, device=device)
-    _hip.trace_set(buf)
-    step()
-    torch.cuda.synchronize()
-    _hip.trace_set(None)
-    t = buf.cpu()
-    rows = t[t[:, 1] != 0]  # workgroups that found a tile
-    t0 = int(t[t[:, 0] != 0][:, 0].min())
-    out = {"timeline_of": args.timeline, "workload": args.workload, "form": args.form,
-           "workgroups_launched": int((t[:, 0] != 0).sum()), "workgroups_with_work": int(rows.size(0)),
-           "unit": "ns after the first workgroup of the kernel entered", "kernels": {}}
-    first = {}  # column of a group's first stamp when it is not column 0
-    if int((t[:, 8] != 0).sum()) > 0 and int((t[:, 15] != 0).sum()) == 0 and int((t[:, 9] != 0).sum()) > 0 and args.form != "fused":
-        groups = {"sgmv_shrink_kernel": rows, "sgmv_expand_kernel": t[t[:, 9] != 0]}
-        first["sgmv_expand_kernel"] = 8
-    elif int((rows[:, 15] != 0).sum()) == 0:
-        groups = {"decode_kernel": rows}
-    else:
-        groups = {"split_kernel producer": rows[rows[:, 15] != 0], "split_kernel consumer": rows[rows[:, 15] == 0]}
-    for name, g in groups.items():
-        entry = {}
-        c0 = first.get(name, 0)
-        if c0:
-            t0 = int(t[t[:, c0] != 0][:, c0].min())
-        for i, label in enumerate(STAMPS[name]):
-            if label is None:
-                continue
-            col = g[:, c0 + i]
-            col = (col[col != 0] - t0) * 10
-            if col.numel():
-                entry[label] = [int(col.min()), int(col.median()), int(col.max())]
-        out["kernels"][name] = {"workgroups": int(g.size(0)), "min_median_max": entry}
-    print(json.dumps(out))
-
-
 def measure_backbone(steps: int, warmup: int) -> dict:
     """BASELINE configs[4]: decode-step latency of a synthetic 24-layer decoder (hidden 1024, 16 query /
     2 KV heads of 64, SwiGLU 4096, RMSNorm; 64 streams with context lengths U[128, 2048]; 32 rank-32
@@ -621,27 +553,15 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode", choices=sorted(WORKLOADS))
-    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | split | sgmv | fused | token")
+    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | slot | split | sgmv | fused | token")
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip what the default run adds after the headline: the prefill, mixed and backbone steps and the floor")
     ap.add_argument("--floor", action="store_true", help="print only the floor measurements (launch costs and stream rates)")
-    ap.add_argument("--hot-layers", type=int, default=0,
-                    help="diagnostic: let all 24 layers of the step reuse the buffers of the first N layers "
-                         "(N=1 keeps the working set inside the last-level cache); 0 = the workload's own set")
     ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
                     help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
-    ap.add_argument("--sequences", type=int, default=0,
-                    help="diagnostic (prefill workload): a batch of N sequences drawn like the 16 (1: 1011 tokens, "
-                         "2: 1620, 4: 2098, 8: 4511); 0 = all 16")
-    ap.add_argument("--no-rank-vector", action="store_true",
-                    help="diagnostic (mixed workload): do not tell the kernels the adapters' true ranks; the zero "
-                         "padding of the rank-64 buffers is then read and multiplied like any other data")
-    ap.add_argument("--timeline", default=None, choices=ORDER,
-                    help="diagnostic: in-kernel timeline of one projection's launch (decode, prefill or mixed workload) "
-                         "(needs the trace build of the library)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
                          "that rocprof byte counters of the same run are scaled by")
@@ -649,18 +569,12 @@ def main() -> None:
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; every box in this pool has one (use --gpus 1)")
 
-    if args.timeline:
-        os.environ.setdefault("MLORA_LIBRARY", str(ROOT / "nanovllm-voxcpm_amd" / "nanovllm_voxcpm_amd" / "libmlora_gfx950_trace.so"))
-
     import torch
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no ROCm GPU visible")
     device = "cuda:0"
     torch.cuda.set_device(0)
-    if args.timeline:
-        run_timeline(args)
-        return
     if args.workload == "backbone":
         run_backbone(args)
         return
@@ -680,8 +594,7 @@ def main() -> None:
     warmup = args.warmup if not heavy else max(1, min(args.warmup, 3))
     rank = args.rank if args.workload in ("decode", "prefill") else 0
     res, (layers, slots, rank, step) = measure_workload(args.workload, device, args.form, steps, warmup, only=args.only, rank=rank,
-                                                        hot_layers=args.hot_layers, eager=args.eager, rank_vector=not args.no_rank_vector,
-                                                        sequences=args.sequences if args.workload == "prefill" else 0)
+                                                        eager=args.eager)
     out = {
         "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
         "value": res["value"],
@@ -706,13 +619,16 @@ def main() -> None:
     torch.cuda.synchronize()
     out["split_waits_run_out"] = sum(
         int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
-        for buf in step.backend._scratch.values())
+        for buf in step.backend.scratch_buffers())
 
-    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.hot_layers and not args.eager and not args.rank
+    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.eager and not args.rank
     if default_run and not args.no_extras:
         # After the headline (outside its timed region): what one launch costs here and what a
         # stream reaches here, and the other configurations of the benchmark, a few replays each.
-        out["floor"] = measure_floor(device, res["algorithmic_bytes_per_step"], res["calls_per_step"])
+        try:  # (launches of known cost come from the diagnostic variant of the library)
+            out["floor"] = measure_floor(device, res["algorithmic_bytes_per_step"], res["calls_per_step"])
+        except RuntimeError as exc:
+            out["floor"] = {"unavailable": str(exc)}
         extra = {}
         for name in ("prefill", "mixed"):
             r, (wl_layers, wl_slots, _, _) = measure_workload(name, device, "auto", 5, 2, per_projection=True)

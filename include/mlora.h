@@ -122,8 +122,10 @@ int mlora_add_lora(const MloraAddArgs* args);
  * MLORA_STATIC_SCRATCH_BYTES bytes that lives in the library's device image, one copy per GPU, held
  * until the process ends.  The call allocates and frees nothing.  It returns MLORA_E_TOO_LARGE when
  * one fp32 copy of the rank-r intermediate (num_tokens x num_slices x r x 4 bytes) does not fit the
- * array.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
- * streams, two threads) race on it and must be ordered by the caller. */
+ * array, whatever form the call would take.  Every call on a GPU shares that GPU's array: calls that
+ * overlap in time on one GPU (two streams, two threads) race on it and must be ordered by the
+ * caller.  The first call on a device looks the array's address up and must be made outside stream
+ * capture (a call with num_tokens = 0 is enough); a first call inside a capture is refused. */
 #define MLORA_STATIC_SCRATCH_BYTES (16u << 20)
 int mlora_add_lora_static(const MloraAddArgs* args);
 
@@ -139,8 +141,11 @@ size_t mlora_add_workspace_bytes(int32_t num_tokens, int32_t num_slices, int32_t
  * workgroups of MLORA_FORM_FUSED put on the partial sums they wrote.  mlora_workspace_init enqueues one kernel that clears the head and writes the
  * signature; call it once after allocation (it is a kernel, not a memset, so it may be recorded
  * into a graph).  Launches leave the head ready for the next launch.  A workspace whose head
- * does not carry the signature is still safe to pass: the kernels then compute every
- * intermediate locally and never read the exchange area.  No counterpart in the reference. */
+ * is not in the state the initialisation or a launch left it in (no signature, or a generation,
+ * arrival count and check word that do not fit each other) is still safe to pass: the kernels
+ * then compute every intermediate locally and never read the exchange area.  Initialise every
+ * workspace once all the same: memory that held a workspace before is not told apart from one
+ * by more than those words.  No counterpart in the reference. */
 #define MLORA_WORKSPACE_HEAD_BYTES (16384 + (4 << 20) + (64 << 10))
 int mlora_workspace_init(void* workspace, int64_t workspace_bytes, void* stream);
 
@@ -291,27 +296,6 @@ int mlora_install_slot(const MloraInstallArgs* args);
  * capturing.  No counterpart in the reference: lets a host-side cache tell work recorded
  * into one capture from work run eagerly or recorded into another capture. */
 uint64_t mlora_stream_capture_id(void* stream);
-
-/* Diagnostic knobs (the MLORA_* environment variables) are read once per process and kept;
- * this makes the next call read them again.  No counterpart in the reference. */
-void mlora_reload_knobs(void);
-
-/* Launches of known cost (measurement aid, no counterpart in the reference): kind 0 enqueues a
- * kernel that does nothing with the given grid and workgroup size (what a launch costs by itself);
- * kind 1 a read-modify-write stream over `bytes` of 16-bit elements at `buf` (every element read,
- * incremented, written back once: the access pattern of y); kind 2 a read-only stream over them;
- * kind 3 a kernel of the given grid whose workgroups each write the number of the XCD they run on
- * to `buf` (int32 per workgroup, linear workgroup order: the placement the kernels' grids of x
- * extent 8 rely on can be checked).  bench.py quotes kinds 0-2 beside the real kernels. */
-int mlora_probe_launch(void* stream, int32_t kind, void* buf, int64_t bytes, int32_t grid_x, int32_t grid_y, int32_t grid_z,
-                       int32_t threads);
-
-/* In-kernel timelines (diagnostic, no counterpart in the reference).  The library variant built
- * with `make trace` (libmlora_gfx950_trace.so) records, per workgroup of the small-tile kernels,
- * up to 16 readings of the 100 MHz clock at fixed points of the kernel into `buf` (uint64
- * [workgroups][16], device memory the caller zeroes; NULL switches recording off).  The regular
- * library returns MLORA_E_UNSUPPORTED. */
-int mlora_trace_set(void* buf);
 
 /* Library identification and diagnostics. */
 int mlora_abi_version(void);

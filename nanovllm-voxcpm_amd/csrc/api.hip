@@ -12,6 +12,7 @@
 
 #include "common.h"
 #include "launch.h"
+#include "mlora_diag.h"
 
 namespace mlora {
 
@@ -270,7 +271,7 @@ void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU (n
 std::mutex g_scratch_mutex;
 
 // Address of the current device's copy of `scratch`; nullptr (and the error text set) on failure.
-void* static_scratch() {
+void* static_scratch(hipStream_t stream) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -279,6 +280,14 @@ void* static_scratch() {
   }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
+    // The look-up may load the code object, which a stream capture in progress does not survive:
+    // the first call on a device has to be made outside any capture (one with num_tokens = 0 will do).
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) == hipSuccess && status == hipStreamCaptureStatusActive) {
+      set_error("mlora_add_lora_static: the first call on a device must be made outside stream capture (call once with num_tokens = 0 before capturing)");
+      return nullptr;
+    }
+    (void)hipGetLastError();
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr) {
@@ -301,7 +310,7 @@ extern "C" int mlora_add_lora_static(const MloraAddArgs* a) {
               one_copy, static_cast<unsigned>(MLORA_STATIC_SCRATCH_BYTES - MLORA_WORKSPACE_HEAD_BYTES));
     return MLORA_E_TOO_LARGE;
   }
-  void* ptr = static_scratch();
+  void* ptr = static_scratch(static_cast<hipStream_t>(a->stream));
   if (!ptr) return MLORA_E_INVALID;
   MloraAddArgs b = *a;
   b.workspace = ptr;
@@ -333,21 +342,6 @@ extern "C" uint64_t mlora_stream_capture_id(void* stream) {
     return 0;
   }
   return status == hipStreamCaptureStatusActive ? static_cast<uint64_t>(id) : 0;
-}
-
-extern "C" int mlora_trace_set(void* buf) {
-#ifdef MLORA_TRACE
-  decode_trace_set(buf);
-  slot_trace_set(buf);
-  split_trace_set(buf);
-  fused_trace_set(buf);
-  sgmv_trace_set(buf);
-  return 0;
-#else
-  (void)buf;
-  set_error("mlora_trace_set: this library was built without MLORA_TRACE (make trace builds the variant that records timelines)");
-  return MLORA_E_UNSUPPORTED;
-#endif
 }
 
 extern "C" void mlora_reload_knobs(void) { ++g_knob_generation; }

@@ -222,6 +222,15 @@ __device__ __forceinline__ void count_rejected_plan(const int32_t* plan, bool he
 // workspace: whatever an earlier launch left anywhere in the area, in whatever layout, carries a
 // tag below the current one.
 constexpr uint32_t kWsMagic = 0x4d4c5733u;  // "MLW3"
+// Third word of the {generation, arrivals} pair: generation ^ kWsGenCheck, rewritten with every
+// advance of the generation.  A head is believed only if signature, this word and an arrival count
+// below the grid size all fit: memory that once was a workspace and was handed out again in between
+// can keep the signature while the pair holds something else, and a generation that never advances
+// would make the next launch accept what the last one left.
+constexpr uint32_t kWsGenCheck = 0x9e3779b9u;
+__device__ __forceinline__ bool ws_state_ok(uint32_t signature, uint32_t generation, uint32_t arrivals, uint32_t check, uint32_t grid) {
+  return signature == kWsMagic && check == (generation ^ kWsGenCheck) && arrivals < grid;
+}
 constexpr int kWsTimeoutsWord = 1;
 constexpr int kWsTileOff = 256;
 constexpr int kWsTiles = 1024;

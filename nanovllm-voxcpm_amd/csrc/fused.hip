@@ -121,6 +121,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   // earlier launch left anywhere (whatever its layout was) carries a tag below this launch's
   uint32_t* const ustate = ws + kWsTileOff / 4;
   const uint32_t tag = ustate[0] + 1u;
+  const uint32_t arrivals0 = ustate[1], gen_check = ustate[2];
   const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
   int slot[G], start[G], m[G], any = 0;
 #pragma unroll
@@ -146,15 +147,18 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   // One exit test, the same for every workgroup of a unit
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(any > 0);
-  const bool xok = trusted | (signature == kWsMagic);  // seals and generations can be used
+  // seals and generations can be used: the head is in the state a launch (or the initialisation) left it in
+  const bool xok = trusted | ws_state_ok(signature, tag - 1u, arrivals0, gen_check, gridDim.x * gridDim.y * gridDim.z);
   // every workgroup of the grid reports exactly once that it is done (also the ones without work);
   // the last one advances the generation, which makes every seal of this launch stale
   auto count_done = [&]() {
     if (xok && tid == 0) {
       const uint32_t before = __hip_atomic_fetch_add(ustate + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (before + 1u == gridDim.x * gridDim.y * gridDim.z) {
+        const uint32_t next = tag == 0xffffffffu ? 0u : tag;  // generation + 1, the next tag, is never 0
         __hip_atomic_store(ustate + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(ustate, tag == 0xffffffffu ? 0u : tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // generation + 1, the next tag, is never 0
+        __hip_atomic_store(ustate + 2, next ^ kWsGenCheck, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(ustate, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   };

@@ -4,6 +4,7 @@
 // kernels.
 #include "common.h"
 #include "launch.h"
+#include "mlora_diag.h"
 
 namespace mlora {
 

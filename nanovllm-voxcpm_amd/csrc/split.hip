@@ -115,13 +115,15 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
   // tag below this launch's
   uint32_t* const tstate = ws + kWsTileOff / 4;
   const uint32_t tag = tstate[0] + 1u;
+  const uint32_t arrivals0 = tstate[1], gen_check = tstate[2];
   const int slot = rec0[0], m = rec0[1];
   const int n_tiles = hdr1[MLORA_PLAN_TILES_SHORT - 4] + hdr2[MLORA_PLAN_TILES_LONG_SMALL - 8] * include_long;
   // One exit test, the same for every workgroup of a tile
   const int usable = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
                      int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(tile < n_tiles) & int(m > 0) & int(slot >= 0) &
                      int(slot < num_slots);
-  const bool xok = trusted | (signature == kWsMagic);  // the exchange area can be used
+  // the exchange area can be used: the head is in the state a launch (or the initialisation) left it in
+  const bool xok = trusted | ws_state_ok(signature, tag - 1u, arrivals0, gen_check, gridDim.x * gridDim.y * gridDim.z);
   // Every workgroup of the grid reports exactly once that it is done with the exchange area (also
   // the ones without work); the last one advances the generation.  Counted by the last wavefront,
   // which has the least other work: the count comes back from the memory system long after it was
@@ -130,8 +132,10 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
     if (xok && tid == kNT - kWave) {
       const uint32_t before = xadd(tstate + 1, 1u, wide);
       if (before + 1u == gridDim.x * gridDim.y * gridDim.z) {
+        const uint32_t next = tag == 0xffffffffu ? 0u : tag;  // so that generation + 1, the next tag, is never 0
         xstore32(tstate + 1, 0u, wide);
-        xstore32(tstate, tag == 0xffffffffu ? 0u : tag, wide);  // so that generation + 1, the next tag, is never 0
+        xstore32(tstate + 2, next ^ kWsGenCheck, wide);
+        xstore32(tstate, next, wide);
       }
     }
   };
@@ -485,7 +489,8 @@ __global__ __launch_bounds__(kNT) void split_kernel(const int32_t* __restrict__ 
 // the signature.
 __global__ __launch_bounds__(256) void workspace_init_kernel(uint32_t* ws) {
   const int words = MLORA_WORKSPACE_HEAD_BYTES / 4;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x) ws[i] = i == 0 ? kWsMagic : 0u;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
+    ws[i] = i == 0 ? kWsMagic : i == kWsTileOff / 4 + 2 ? kWsGenCheck : 0u;  // generation 0 and its check word
 }
 
 struct SplitLaunch {

@@ -62,13 +62,16 @@ EXPORTS = (
     "mlora_meta_build",
     "mlora_install_slot",
     "mlora_stream_capture_id",
-    "mlora_reload_knobs",
-    "mlora_trace_set",
-    "mlora_probe_launch",
     "mlora_abi_version",
     "mlora_last_error",
     "mlora_build_info",
 )
+
+
+# include/mlora_diag.h: measurement and test aids.  The product library exports the first only; the
+# diag and trace variants export all three.
+DIAG_EXPORTS = ("mlora_reload_knobs", "mlora_probe_launch", "mlora_trace_set")
+DIAG_LIB_NAME = "libmlora_gfx950_diag.so"
 
 
 class MloraSlice(C.Structure):
@@ -227,12 +230,7 @@ def load() -> C.CDLL:
     lib.mlora_workspace_init.restype = C.c_int
     lib.mlora_stream_capture_id.argtypes = [C.c_void_p]
     lib.mlora_stream_capture_id.restype = C.c_uint64
-    lib.mlora_probe_launch.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
-    lib.mlora_probe_launch.restype = C.c_int
-    lib.mlora_trace_set.argtypes = [C.c_void_p]
-    lib.mlora_trace_set.restype = C.c_int
-    lib.mlora_reload_knobs.argtypes = []
-    lib.mlora_reload_knobs.restype = None
+    _declare_diag(lib)
     lib.mlora_abi_version.argtypes = []
     lib.mlora_abi_version.restype = C.c_int
     lib.mlora_last_error.argtypes = []
@@ -240,6 +238,40 @@ def load() -> C.CDLL:
     lib.mlora_build_info.argtypes = []
     lib.mlora_build_info.restype = C.c_char_p
     _LIB = lib
+    return lib
+
+
+def _declare_diag(lib: C.CDLL) -> None:
+    lib.mlora_reload_knobs.argtypes = []
+    lib.mlora_reload_knobs.restype = None
+    if hasattr(lib, "mlora_probe_launch"):
+        lib.mlora_probe_launch.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+        lib.mlora_probe_launch.restype = C.c_int
+    if hasattr(lib, "mlora_trace_set"):
+        lib.mlora_trace_set.argtypes = [C.c_void_p]
+        lib.mlora_trace_set.restype = C.c_int
+
+
+_DIAG_LIB: C.CDLL | None = None
+
+
+def load_diag() -> C.CDLL:
+    """The library that exports the measurement aids of include/mlora_diag.h: the loaded library
+    itself when it is a diagnostic variant (MLORA_LIBRARY names the trace build), else the diag
+    variant built next to it by `make diag`.  Raises when there is none."""
+    global _DIAG_LIB
+    if _DIAG_LIB is not None:
+        return _DIAG_LIB
+    lib = load()
+    if not hasattr(lib, "mlora_probe_launch"):
+        path = Path(os.environ.get("MLORA_DIAG_LIBRARY") or LIB_PATH.with_name(DIAG_LIB_NAME))
+        if not path.exists():
+            raise RuntimeError(f"diagnostic variant of the library not built: {path} is missing (run `make -C nanovllm-voxcpm_amd/csrc diag`)")
+        lib = C.CDLL(str(path))
+        _declare_diag(lib)
+        lib.mlora_last_error.argtypes = []
+        lib.mlora_last_error.restype = C.c_char_p
+    _DIAG_LIB = lib
     return lib
 
 
@@ -597,15 +629,21 @@ def probe_launch(kind: int, buf: torch.Tensor | None = None, grid: tuple[int, in
     per workgroup, linear workgroup order)."""
     dev = buf.device if buf is not None else (device or torch.device("cuda", torch.cuda.current_device()))
     nbytes = buf.numel() * buf.element_size() if buf is not None else 0
+    lib = load_diag()
     with _on(dev):
-        _check(load().mlora_probe_launch(_stream(dev), kind, buf.data_ptr() if buf is not None else None, nbytes, *grid, threads),
-               "mlora_probe_launch")
+        rc = lib.mlora_probe_launch(_stream(dev), kind, buf.data_ptr() if buf is not None else None, nbytes, *grid, threads)
+    if rc != 0:
+        raise RuntimeError(f"mlora_probe_launch failed (code {rc}): {lib.mlora_last_error().decode('utf-8', 'replace')}")
 
 
 def trace_set(buf: torch.Tensor | None) -> None:
     """Hand the trace build of the library a zeroed uint64 [workgroups, 16] buffer to record
-    in-kernel timelines into (None switches recording off).  Raises with the regular build."""
-    _check(load().mlora_trace_set(buf.data_ptr() if buf is not None else None), "mlora_trace_set")
+    in-kernel timelines into (None switches recording off).  The kernels that record are the
+    loaded library's own, so this needs MLORA_LIBRARY to name the trace build; raises otherwise."""
+    lib = load()
+    if not hasattr(lib, "mlora_trace_set"):
+        raise RuntimeError("in-kernel timelines need the trace build of the library (make trace; MLORA_LIBRARY=.../libmlora_gfx950_trace.so)")
+    _check(lib.mlora_trace_set(buf.data_ptr() if buf is not None else None), "mlora_trace_set")
 
 
 def build_info() -> str:

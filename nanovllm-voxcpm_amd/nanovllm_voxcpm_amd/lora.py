@@ -132,7 +132,7 @@ class HipLoRABackend:
         self.form = name
         self._scratch: dict = {}
         self._spares: dict = {}          # device -> initialised buffer kept for the next graph capture
-        self._graph_scratch: list = []   # buffers captured graphs refer to
+        self._graph_scratch: dict = {}   # device -> buffers captured graphs refer to (the last one is in use)
         self._sites = threading.local()  # per thread: weight buffers -> _CallSite
 
     # -- capability ---------------------------------------------------------------------
@@ -218,41 +218,57 @@ class HipLoRABackend:
     def _scratch_for(self, x: torch.Tensor, num_slices: int, rank: int, stream: int | None = None,
                      capture: int | None = None) -> torch.Tensor:
         """Device scratch for the rank-r intermediate (between the two launches of the
-        long-segment form, or between producer and consumer workgroups of the split form).  One
-        buffer per (device, stream), grown on demand: calls on one stream are ordered, so they can
-        share it.  A graph being captured gets a buffer of its own (its replays may run beside
-        eager calls of any stream): preferably one that was allocated and initialised outside the
-        capture — every eager call keeps such a spare ready — so that the graph holds no
-        initialisation launch; the graph refers to it for as long as it lives, so it is never
-        freed.  Without a spare the buffer comes from the graph's own pool and its initialisation
-        is recorded with it."""
+        long-segment form, or between producer and consumer workgroups of the split form).
+
+        Eager calls: one buffer per (device, stream), grown on demand - calls on one stream are
+        ordered, so they can share it.  When the table is full its oldest entry goes, not all.
+
+        Graphs being captured: one buffer per device, shared by every graph this backend captures
+        there and always allocated and initialised OUTSIDE the capture (every eager call keeps
+        one ready), so that no graph holds an initialisation launch or memory of its own for it.
+        The graphs refer to it for as long as they live, so it is only ever replaced by a larger
+        one (the smaller stays alive with them).  Sharing is safe under the rule that holds for
+        every workspace - launches that use it are ordered on one stream: the engine replays its
+        graphs one after the other on one stream.  Without a buffer ready (a capture as the very
+        first call, or one that needs more than any eager call did) the buffer comes from the
+        graph's own pool and its initialisation is recorded with it."""
         nbytes = _hip.add_workspace_bytes(x.size(0), num_slices, rank, x.dtype)
         if stream is None:
             stream = _hip.current_stream_handle(x.device)
         if capture is None:
             capture = _hip.stream_capture_id(x.device, stream)
-        key = (x.device, stream, capture)
-        buf = self._scratch.get(key)
-        if buf is not None and buf.numel() >= nbytes:
-            if not capture and x.device not in self._spares:  # a capture took the spare: make the next one
-                self._spares[x.device] = self._new_scratch(x.device, buf.numel(), stream)
-            return buf
+        device = x.device
         if capture:
-            spare = self._spares.pop(x.device, None)
+            held = self._graph_scratch.get(device)
+            if held is not None and held[-1].numel() >= nbytes:
+                return held[-1]
+            spare = self._spares.pop(device, None)
             if spare is not None and spare.numel() >= nbytes:
-                self._graph_scratch.append(spare)
-                self._scratch[key] = spare
+                self._graph_scratch.setdefault(device, []).append(spare)
                 return spare
             if spare is not None:
-                self._spares[x.device] = spare
-        if len(self._scratch) >= 8:
-            self._scratch.clear()
-        buf = self._scratch[key] = self._new_scratch(x.device, nbytes, stream)
-        if not capture:
-            spare = self._spares.get(x.device)
-            if spare is None or spare.numel() < buf.numel():
-                self._spares[x.device] = self._new_scratch(x.device, buf.numel(), stream)
+                self._spares[device] = spare
+            key = (device, stream, capture)  # from the graph's own pool, initialisation recorded
+            buf = self._scratch.get(key)
+            if buf is None or buf.numel() < nbytes:
+                buf = self._scratch[key] = self._new_scratch(device, nbytes, stream)
+            return buf
+        key = (device, stream, 0)
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < nbytes:
+            if buf is None and len(self._scratch) >= 8:
+                del self._scratch[next(iter(self._scratch))]  # the oldest entry (its stream's work is queued behind it)
+            buf = self._scratch[key] = self._new_scratch(device, nbytes, stream)
+        # a buffer for the next capture, as large as the largest eager one: made here, outside any capture
+        need = buf.numel()
+        held = self._graph_scratch.get(device)
+        if (held is None or held[-1].numel() < need) and (device not in self._spares or self._spares[device].numel() < need):
+            self._spares[device] = self._new_scratch(device, need, stream)
         return buf
+
+    def scratch_buffers(self) -> list[torch.Tensor]:
+        """Every scratch buffer this backend holds (eager ones and those captured graphs refer to)."""
+        return list(self._scratch.values()) + [buf for held in self._graph_scratch.values() for buf in held] + list(self._spares.values())
 
     @staticmethod
     def _vectorisable(x: torch.Tensor, y: torch.Tensor, a_list, b_list, cols) -> bool:

@@ -32,6 +32,25 @@ def test_library_exports_every_declared_symbol():
     assert "gfx950" in _hip.build_info()
 
 
+def test_measurement_aids_live_in_the_diagnostic_variant_only():
+    """include/mlora.h is the product's C-ABI; what include/mlora_diag.h declares is exported by
+    the diagnostic variant of the library (the knob reload, which the tests of one process need,
+    by the product library too) and nothing else of it by the product library."""
+    from nanovllm_voxcpm_amd import _hip
+
+    diag_header = HEADER.with_name("mlora_diag.h")
+    text = re.sub(r"/\*.*?\*/", "", diag_header.read_text(), flags=re.S)
+    declared = sorted(set(re.findall(r"\b(mlora_[a-z_]+)\s*\(", text)))
+    assert set(declared) == set(_hip.DIAG_EXPORTS)
+    assert not set(declared) & set(_declared_functions())
+    lib = _hip.load()
+    assert hasattr(lib, "mlora_reload_knobs")
+    assert not hasattr(lib, "mlora_probe_launch") and not hasattr(lib, "mlora_trace_set")
+    diag = _hip.load_diag()
+    for name in _hip.EXPORTS + _hip.DIAG_EXPORTS:
+        assert hasattr(diag, name), name
+
+
 def test_ctypes_structs_match_the_c_layout(tmp_path):
     """Compile a probe against the header with the host compiler and compare sizeof / offsetof."""
     from nanovllm_voxcpm_amd import _hip

@@ -36,7 +36,7 @@ def _waits_run_out(backend) -> int:
 
     torch.cuda.synchronize()
     return sum(int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
-               for buf in backend._scratch.values())
+               for buf in backend.scratch_buffers())
 
 
 def _backend(form="auto"):
@@ -251,15 +251,23 @@ def test_split_form_producers_and_consumers(name, rank, kpart, wide, sym, monkey
         assert torch.equal(runs[0], other)
     (scratch,) = backend._scratch.values()
     head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
-    state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} of the workspace, then reserved words
-    assert all(arrivals == 0 for _, arrivals in state)
-    assert state[0][0] == len(runs) and all(generation == 0 for generation, _ in state[1:])  # one step per launch
+    state = head[256 // 4 : 256 // 4 + 2 * 1024].tolist()  # generation, arrivals, generation ^ check constant, then reserved words
+    check = lambda gen: ((gen ^ 0x9E3779B9) + (1 << 31)) % (1 << 32) - (1 << 31)  # noqa: E731  (as the int32 word reads)
+    assert state[:3] == [len(runs), 0, check(len(runs))] and not any(state[3:])  # one step per launch, arrivals back at zero
+    # a head whose pair no longer fits its check word, or whose arrival count is impossible (memory that
+    # was a workspace once and was handed out again in between can keep the signature): not believed,
+    # not touched, same bits
+    _knobs(monkeypatch, MLORA_SPLIT_SPIN_TICKS=20000)
+    for gen, arrivals, chk in ((len(runs) + 5, 0, check(len(runs))), (len(runs), 1 << 20, check(len(runs)))):
+        head[256 // 4 : 256 // 4 + 3] = torch.tensor([gen, arrivals, chk], dtype=torch.int32, device="cuda")
+        assert torch.equal(run(), runs[0])
+        assert head[256 // 4 : 256 // 4 + 3].tolist() == [gen, arrivals, chk]
+    head[256 // 4 : 256 // 4 + 3] = torch.tensor(state[:3], dtype=torch.int32, device="cuda")
     # a workspace without the signature: same bits, nothing published, nobody waits
     scratch[:4].zero_()
-    _knobs(monkeypatch, MLORA_SPLIT_SPIN_TICKS=20000)
     assert torch.equal(run(), runs[0])
     assert _waits_run_out(backend) == 0
-    assert head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist() == state
+    assert head[256 // 4 : 256 // 4 + 2 * 1024].tolist() == state
 
 
 def test_split_form_ignores_what_a_launch_of_another_layout_left():
@@ -522,15 +530,15 @@ def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
             assert torch.allclose(got.float(), two.float(), rtol=RTOL, atol=ATOL)
         (scratch,) = backend._scratch.values()
         head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
-        state = head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist()  # {generation, arrivals} of the workspace, then reserved words
-        assert all(arrivals == 0 for _, arrivals in state)
-        assert state[0][0] == len(runs) and all(generation == 0 for generation, _ in state[1:])  # one step per launch
+        state = head[256 // 4 : 256 // 4 + 2 * 1024].tolist()  # generation, arrivals, generation ^ check constant, then reserved words
+        want_check = ((len(runs) ^ 0x9E3779B9) + (1 << 31)) % (1 << 32) - (1 << 31)
+        assert state[:3] == [len(runs), 0, want_check] and not any(state[3:])  # one step per launch, arrivals back at zero
         # a workspace without the signature: nobody seals, nobody waits, same bits
         scratch[:4].zero_()
         _knobs(monkeypatch, MLORA_FUSED_SPIN_TICKS=50000)
         assert torch.equal(run(), got)
         assert _waits_run_out(backend) == 0
-        assert head[256 // 4 : 256 // 4 + 2 * 1024].view(-1, 2).tolist() == state
+        assert head[256 // 4 : 256 // 4 + 2 * 1024].tolist() == state
 
 
 @pytest.mark.parametrize("rank,expected", [(16, "mfma"), (64, "sgmv")])

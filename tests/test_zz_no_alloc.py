@@ -42,6 +42,7 @@ def test_static_scratch_entry_matches_the_regular_entry(name, rank):
     dev = "cuda"
     proj = synthetic.make_projection(name, 6, rank, torch.bfloat16, seed=70 + rank, device=dev)
     workspace = torch.empty(_hip.STATIC_SCRATCH_BYTES, dtype=torch.uint8, device=dev)
+    _hip.workspace_init(workspace)  # as every caller-owned workspace is, once, after allocation
     outs = []
     for tokens, seed in ((1500, 71), (130, 72)):  # two calls in a row, the second one smaller
         x, y0 = synthetic.make_activations(tokens, proj.k, sum(proj.widths), torch.bfloat16, seed=seed, device=dev)
@@ -76,3 +77,35 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
     slots = torch.zeros(tokens, dtype=torch.int32, device=dev)
     with pytest.raises(RuntimeError, match="exceed the static scratch"):
         _hip.add_lora(y, x, a, b, [0, 8], slots, None, 1.0, static_scratch=True)
+
+
+def test_static_scratch_entry_under_graph_capture_after_a_warm_up_call():
+    """The address of the library's scratch is looked up on the first call on a device, which must
+    not happen inside a capture (the library refuses that with a clear error): one call with no
+    tokens, outside any capture, is the warm-up.  After it the entry point can be captured; every
+    replay gives the bits of the eager call."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
+    from nanovllm_voxcpm_amd.lora_ops.segment_meta import build_segment_plan
+
+    dev = "cuda"
+    proj = synthetic.make_projection("o", 6, 16, torch.bfloat16, seed=75, device=dev)
+    tokens = 96
+    x, y0 = synthetic.make_activations(tokens, proj.k, sum(proj.widths), torch.bfloat16, seed=76, device=dev)
+    g = torch.Generator().manual_seed(77)
+    slots = torch.randint(-1, 6, (tokens,), generator=g, dtype=torch.int32).to(dev)
+    plan = build_segment_plan(slots, 6).workspace
+    empty = torch.zeros(0, proj.k, dtype=torch.bfloat16, device=dev)
+    _hip.add_lora(y0[:0], empty, proj.a, proj.b, [0], slots[:0], None, 1.0, static_scratch=True)  # warm-up: no tokens, no launch
+    eager = y0.clone()
+    _hip.add_lora(eager, x, proj.a, proj.b, [0], slots, plan, 1.0, _hip.FORM_AUTO, None, static_scratch=True)
+    torch.cuda.synchronize()
+    y = y0.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _hip.add_lora(y, x, proj.a, proj.b, [0], slots, plan, 1.0, _hip.FORM_AUTO, None, static_scratch=True,
+                      stream=_hip.current_stream_handle(x.device))
+    for _ in range(3):
+        y.copy_(y0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)
