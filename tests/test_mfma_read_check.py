@@ -61,3 +61,21 @@ def test_a_branch_a_few_instructions_behind_the_mfma_is_followed(tmp_path):
     )
     join = ".LBB0_2:\n\tds_write_b128 v144, v[46:49] offset:64\n\ts_endpgm\n"
     assert _count(tmp_path, HEAD + run + join) == 1
+
+
+def test_a_wait_instruction_behind_the_branch_is_not_taken_for_a_delay(tmp_path):
+    """A wait that finds its counter at zero returns at once: the read behind it is as early as
+    without it."""
+    join = ".LBB0_2:\n\ts_waitcnt vmcnt(0)\n\tv_mov_b64_e32 v[100:101], v[48:49]\n\ts_endpgm\n"
+    assert _count(tmp_path, HEAD + RUN + join) == 1
+
+
+def test_the_distance_asked_for_follows_from_the_variant(tmp_path):
+    """Seven wait states behind the branch are too few for a 16x16 variant (never less than eight
+    are asked for); a 32x32 variant (8 passes + 3) asks for eleven, an unknown one for the most."""
+    sc = _scanner()
+    assert sc.need_of("v_mfma_f32_16x16x32_bf16") == 8 and sc.need_of("v_mfma_f32_16x16x16_bf16") == 8
+    assert sc.need_of("v_mfma_f32_32x32x16_bf16") == 11 and sc.need_of("v_mfma_f32_unknown") == sc.NEED_MAX
+    for nops, found in ((5, 1), (6, 0)):  # the branch itself is one state
+        join = f".LBB0_2:\n\ts_nop {nops}\n\tv_mov_b64_e32 v[100:101], v[48:49]\n\ts_endpgm\n"
+        assert _count(tmp_path, HEAD + RUN + join) == found, nops
