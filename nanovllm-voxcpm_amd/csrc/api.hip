@@ -198,9 +198,12 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (form == MLORA_FORM_SPLIT && a->form != MLORA_FORM_SPLIT &&
       (knobs().no_split || !split_supported(a) || ((static_cast<long long>(a->r) * a->k < knobs().split_min_rk || a->num_tokens > knobs().split_max_tokens) && knobs().force_form != MLORA_FORM_SPLIT)))
     form = MLORA_FORM_MFMA;
-  // small tiles with the grid laid over the slots where the shape allows it and slot ids are few
-  if (form == MLORA_FORM_MFMA && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_MFMA && slot_supported(a) &&
-      a->num_slots <= knobs().slot_max_slots)
+  // small tiles with the grid laid over the slots where the shape allows it and slot ids are few.
+  // Also where the split form would be taken: at K = 4096 the slot-major kernel shares K out between
+  // the workgroups of a tile itself (down, decode batch, us per call, slot-major / split form:
+  // rank 32: 8.1 / 10.6, rank 64: 10.7 / 17.0).
+  if ((form == MLORA_FORM_MFMA || form == MLORA_FORM_SPLIT) && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_MFMA &&
+      knobs().force_form != MLORA_FORM_SPLIT && slot_supported(a) && a->num_slots <= knobs().slot_max_slots)
     form = MLORA_FORM_SLOT;
   // long-segment batches in one launch, on request
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))
@@ -222,10 +225,11 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
       if (form == MLORA_FORM_SLOT) {
         if (!slot_supported(a)) {
-          set_error("mlora_add_lora: the slot-major form needs one or two non-empty slices and K = 1024 (any rank) or 4096 (rank <= 16)");
+          set_error("mlora_add_lora: the slot-major form needs one or two non-empty slices and K = 1024, or K = 4096 with rank <= 16 or with "
+                    "one slice of at most 4096 columns and an initialised workspace");
           return MLORA_E_UNSUPPORTED;
         }
-        return launch_slot(a);
+        return launch_slot(a, trusted_workspace);
       }
       if (form == MLORA_FORM_SPLIT) {
         if (!split_supported(a)) {

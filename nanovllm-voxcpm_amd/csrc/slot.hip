@@ -21,6 +21,18 @@
 // Tiles behind a slot's first sixteen tokens are taken by further workgroups of the same launch
 // (z beyond the slot layers), which learn their slot from their record like the tile-major
 // kernel: a batch with every token on one adapter spreads over as many workgroups as before.
+//
+// Long K (KP > 1).  What a compute unit can take in per unit of time is what bounds a decode
+// launch (about 35 bytes per cycle, whether the lines come from HBM or from the L2), and with one
+// workgroup per column range every range pulls ALL of x's tile and of A[slot]: at K = 4096 that is
+// 256 KB per workgroup against 16 KB of B and y.  With KP > 1 the KP workgroups of a tile each take
+// one K part AND one column range: a workgroup multiplies its part, publishes the 16 x r partial
+// sums as tagged 64-bit words in the workspace's exchange area, picks up the other parts'
+// words, adds all parts in part order (so every workgroup of the tile holds the same bits) and
+// expands its columns.  The hand-over follows the protocol of split.hip: words are valid when
+// their tag is the workspace's generation + 1, every workgroup of the grid counts itself once,
+// the last one advances the generation, nothing is ever cleared.  Waiting is bounded: a workgroup
+// whose partners' words are not there in time multiplies their parts itself, in their order.
 #include "common.h"
 #include "launch.h"
 
@@ -44,18 +56,31 @@ struct Range {
 // The operand path is the staged one of decode.hip: x rows and A rows of a wavefront's K range are
 // fetched row-contiguously (sixteen lanes per 256 bytes of a row), turned into MFMA operand layout
 // through a private LDS block per wavefront, and the expand runs with the tokens as MFMA rows.
-template <typename T, int R, int KSPW, bool MASKED, int SA, bool EARLY>
+// What the workgroups of a tile need to hand each other partial sums (KP > 1).
+struct Exchange {
+  uint32_t* ws;    // workspace head
+  int spin_ticks;  // bound of the wait for the partners' words, in ticks of the 100 MHz clock (< 0: never accept any)
+  int trusted;     // the head is known to be in a launch's or the initial state without carrying the signature
+};
+
+typedef unsigned long long u64;
+
+template <typename T, int R, int KSPW, int KP, bool MASKED, int SA, bool EARLY>
 __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const int slot_early, const int early_ok, const Range sp,
-                                          const int y_col0, const int y_col1, const bool second, const void* __restrict__ xv, void* __restrict__ yv_, const int64_t xs, const int64_t ys,
+                                          const int y_col0, const int y_col1, const bool second, const void* __restrict__ xv,
+                                          void* __restrict__ yv_, const int64_t xs, const int64_t ys,
                                           const int num_slots, const float scaling, const int32_t* __restrict__ eff_rank,
-                                          const uint32_t check, int32_t* __restrict__ plan_hdr, float* __restrict__ s_red,
-                                          T* __restrict__ s_hi, T* __restrict__ s_lo, i32x4* __restrict__ s_stage) {
+                                          const uint32_t check, int32_t* __restrict__ plan_hdr, const Exchange xc, float* __restrict__ s_red,
+                                          T* __restrict__ s_hi, T* __restrict__ s_lo, i32x4* __restrict__ s_stage, int* __restrict__ s_ok) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
   constexpr int NT = kNW * kWave;
   constexpr int ROUNDS = KSPW / 4;       // groups of four k-steps per wavefront
-  constexpr int K = 32 * kNW * KSPW;
+  constexpr int KPART = 32 * kNW * KSPW;  // columns of x and A one workgroup multiplies
+  constexpr int K = KPART * KP;           // row length of A[slot]
+  constexpr int WORDS = RB * 256;         // partial sums of one (tile, K part), in the order of the shared sum below
+  constexpr int EPT = (WORDS + NT - 1) / NT;  // of which a thread holds this many
   constexpr int kStageRow = 17;          // 16 chunks of 16 bytes + one of padding
   constexpr int SB = RB < 2 ? RB : 2;    // 16-rank blocks of A staged together
   constexpr bool K16 = R == 16;          // expand on the 16x16x16 MFMA: 64-bit operand pieces
@@ -74,7 +99,17 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   const RankPrefetch ranks = rank_prefetch((MASKED && !EARLY) ? eff_rank : nullptr, num_slots, lane);
   if constexpr (EARLY) __builtin_amdgcn_sched_barrier(0);  // the record's requests go out first
 
-  const int ks0 = wave * KSPW;
+  const int kp = KP > 1 ? static_cast<int>(blockIdx.y) : 0;  // this workgroup's K part (and column range)
+  const int ks0 = kp * (KPART / 32) + wave * KSPW;
+  // the workspace's {generation, arrivals, check word} and signature (KP > 1): requested with the record
+  uint32_t* const tstate = KP > 1 ? xc.ws + kWsTileOff / 4 : nullptr;
+  uint32_t signature = 0, generation = 0, arrivals0 = 0, gen_check = 0;
+  if constexpr (KP > 1) {
+    signature = xc.ws[0];
+    generation = tstate[0];
+    arrivals0 = tstate[1];
+    gen_check = tstate[2];
+  }
   i32x4 ast[RB][4 * ROUNDS];
   Pack8 bop[SA][4][KSTEPS];
   // every A line of this wavefront's K range and the B rows of its spans
@@ -148,7 +183,37 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   // waits for the record in the middle of the requests for the weights)
   const int usable = matches & early_ok & int(m > 0) & int(slot >= 0) & int(slot < num_slots) & int(sp.n0 < sp.n1) &
                      int(__builtin_amdgcn_readfirstlane(rows4[0]) >= 0) & int(rec0[2] >= 0) & int(!EARLY || rec0[0] == slot_early);
+  // KP > 1: the exchange area can be used when the head is in the state a launch (or the
+  // initialisation) left it in.  Every workgroup of the grid, with or without work, reports once
+  // that it reads the area no more; the last one advances the generation.
+  const uint32_t tag = generation + 1u;
+  const bool xok = KP > 1 && (xc.trusted | ws_state_ok(signature, generation, arrivals0, gen_check, gridDim.x * gridDim.y * gridDim.z));
+  // The count comes back from the memory system long after it was sent: a working workgroup sends
+  // it behind its last barrier (count_sent, by the last wavefront, which has the fewest spans to
+  // expand) and looks at what came back when its stores are out (count_seen).
+  const bool counter = KP > 1 && xok && tid == NT - kWave;
+  uint32_t arrivals_before = 0;
+  auto count_sent = [&]() {
+    if constexpr (KP > 1) {
+      if (counter) arrivals_before = __hip_atomic_fetch_add(tstate + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  auto count_seen = [&]() {
+    if constexpr (KP > 1) {
+      if (counter && arrivals_before + 1u == gridDim.x * gridDim.y * gridDim.z) {
+        const uint32_t next = tag == 0xffffffffu ? 0u : tag;  // so that generation + 1, the next tag, is never 0
+        __hip_atomic_store(tstate + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(tstate + 2, next ^ kWsGenCheck, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(tstate, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  };
+  auto count_done = [&]() {
+    count_sent();
+    count_seen();
+  };
   if (!usable) {
+    count_done();
     // a plan that was built for another batch shape (or never built): count the launch that found
     // it so, once (the first workgroup's record exists in every plan)
     if (!matches && EARLY && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0 && plan_hdr)
@@ -170,6 +235,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
       eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
     }
     if (eff == 0) {
+      count_done();
       if constexpr (EARLY) settle_requests();
       return;
     }
@@ -197,65 +263,192 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   MLORA_STAMP(2);  // every load is issued
 
   // ---- shrink: H[token, rank] partial over this wavefront's K range ----------------------------
-  f32x4 acc[RB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  Pack8 xa[4], aw[RB][4];
   i32x4* stage = s_stage + wave * (1 + SB) * 16 * kStageRow;
+  // x rows and A rows, fetched row-contiguously, through the wavefront's LDS block into operand
+  // layout, and multiplied: k-steps in ascending order
+  auto stage_and_multiply = [&](const i32x4(&xs_)[4 * ROUNDS], const i32x4(&as_)[RB][4 * ROUNDS], f32x4(&acc)[RB], const bool clear_blocks) {
+    Pack8 xa[4], aw[RB][4];
 #pragma unroll
-  for (int r = 0; r < ROUNDS; ++r) {
+    for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xst[4 * r + i];
+    for (int r = 0; r < ROUNDS; ++r) {
 #pragma unroll
-    for (int p = 0; p < RB / SB; ++p) {
+      for (int i = 0; i < 4; ++i) stage[(4 * lg + i) * kStageRow + (lane & 15)] = xs_[4 * r + i];
+#pragma unroll
+      for (int p = 0; p < RB / SB; ++p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+          for (int sb = 0; sb < SB; ++sb) {
+            i32x4 v = as_[p * SB + sb][4 * r + i];
+            // rank blocks the adapter does not have were requested before its rank was known: they
+            // never reach a multiplier
+            if (MASKED && RB > 1 && clear_blocks && p * SB + sb >= rb_n) v = i32x4{0, 0, 0, 0};
+            stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = v;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
+#pragma unroll
+          for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
+        }
+        __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass or round (and later by the expand)
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int sb = 0; sb < SB; ++sb) {
-          i32x4 v = ast[p * SB + sb][4 * r + i];
-          // rank blocks the adapter does not have were requested before its rank was known: they
-          // never reach a multiplier
-          if (MASKED && EARLY && RB > 1 && p * SB + sb >= rb_n) v = i32x4{0, 0, 0, 0};
-          stage[((1 + sb) * 16 + 4 * lg + i) * kStageRow + (lane & 15)] = v;
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+      }
+    }
+  };
+  // Sum of the wavefronts' partial tiles, wavefront 0 first: out[j] is word tid + j * NT.
+  // D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
+  auto sum_wavefronts = [&](const f32x4(&acc)[RB], float(&out)[EPT]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
+    MLORA_STAMP(3);
+    __syncthreads();
+    MLORA_STAMP(4);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = tid + j * NT;
+      float sum = 0.f;
+      if (WORDS % NT == 0 || e < WORDS) {
+        const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+#pragma unroll
+        for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
+      }
+      out[j] = sum;
+    }
+  };
+  f32x4 acc[RB];
+  float total[EPT];
+  if (KP > 1 && tid == 0) *s_ok = 1;  // (seen by everyone behind the barrier of the sum below)
+  stage_and_multiply(xst, ast, acc, EARLY);
+  sum_wavefronts(acc, total);
+
+  if constexpr (KP > 1) {
+    // ---- the other K parts: from the tile's other workgroups, or multiplied here -----------------
+    u64* const xchg = reinterpret_cast<u64*>(reinterpret_cast<char*>(xc.ws) + kWsXchgOff) +
+                      static_cast<int64_t>(blockIdx.z * 8 + blockIdx.x) * (KP * WORDS);  // the KP parts of this tile
+    float part[KP][EPT];
+#pragma unroll
+    for (int q = 0; q < KP; ++q)
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) part[q][j] = 0.f;
+    if (xok) {
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        const int e = tid + j * NT;
+        if (WORDS % NT == 0 || e < WORDS)
+          __hip_atomic_store(xchg + kp * WORDS + e, (static_cast<u64>(tag) << 32) | __float_as_uint(total[j]), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+    MLORA_STAMP(9);  // this workgroup's partial sums are on their way to the L2
+    int ok = xok && xc.spin_ticks >= 0;
+    if (ok) {
+      const long long t0 = wall_clock64();
+      for (;;) {
+        // every part's words are requested together, this workgroup's own among them (a request
+        // behind a test on the part number is a round trip of its own); its own are not looked at
+        u64 w[KP][EPT];
+#pragma unroll
+        for (int q = 0; q < KP; ++q) {
+#pragma unroll
+          for (int j = 0; j < EPT; ++j) {
+            const int e = (WORDS % NT == 0 || tid + j * NT < WORDS) ? tid + j * NT : 0;
+            w[q][j] = __hip_atomic_load(xchg + q * WORDS + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+        bool all = true;
+#pragma unroll
+        for (int q = 0; q < KP; ++q) {
+#pragma unroll
+          for (int j = 0; j < EPT; ++j) {
+            const bool mine = !(WORDS % NT == 0 || tid + j * NT < WORDS) || q == kp;
+            all &= mine | (static_cast<uint32_t>(w[q][j] >> 32) == tag);
+            part[q][j] = __uint_as_float(static_cast<uint32_t>(w[q][j]));
+          }
+        }
+        if (__builtin_amdgcn_ballot_w64(all) == __builtin_amdgcn_ballot_w64(true)) break;
+        if (wall_clock64() - t0 >= xc.spin_ticks) { ok = 0; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (!ok && xc.spin_ticks > 0 && lane == 0) atomicAdd(xc.ws + kWsTimeoutsWord, 1u);  // diagnostic: a wait ran out
+    }
+    MLORA_STAMP(10);  // the wait for the partners is over
+    // one verdict for the workgroup (through a flag in LDS: the library's block-wide AND reads the
+    // launch's shape from memory first, two trips); the barrier also ends the reading of s_red
+    if (!ok) *s_ok = 0;
+    __syncthreads();
+    ok = *s_ok;
+    if (!ok) {
+      // every other part multiplied here as its own workgroup multiplies it
+      for (int q = 0; q < KP; ++q) {
+        if (q == kp) continue;
+        i32x4 xo[4 * ROUNDS], ao[RB][4 * ROUNDS];
+        const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+          const int64_t koff = static_cast<int64_t>(q * (KPART / 32) + wave * KSPW + 4 * r) * 32 + (lane & 15) * 8;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            xo[4 * r + i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+              const int rr = rb * 16 + 4 * lg + i;
+              if (!MASKED || RB == 1 || rb < rb_n) ao[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+              else ao[rb][4 * r + i] = i32x4{0, 0, 0, 0};
+            }
+          }
+        }
+        f32x4 acc2[RB];
+        float got[EPT];
+        stage_and_multiply(xo, ao, acc2, false);
+        sum_wavefronts(acc2, got);
+        __syncthreads();  // s_red is rewritten by the next part
+#pragma unroll
+        for (int qq = 0; qq < KP; ++qq) {
+          if (qq == q) {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) part[qq][j] = got[j];
+          }
         }
       }
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (p == 0) xa[i].raw = stage[lr * kStageRow + 4 * i + lg];
-#pragma unroll
-        for (int sb = 0; sb < SB; ++sb) aw[p * SB + sb][i].raw = stage[((1 + sb) * 16 + lr) * kStageRow + 4 * i + lg];
-      }
-      __builtin_amdgcn_wave_barrier();  // the block is rewritten by the next pass or round (and later by the expand)
     }
+    // all parts added up in part order, this workgroup's own at its place
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int j = 0; j < EPT; ++j) {
+      const float own = total[j];
+      float sum = 0.f;
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) acc[rb] = Mma<T>::run(xa[i], aw[rb][i], acc[rb]);
+      for (int q = 0; q < KP; ++q) sum += q == kp ? own : part[q][j];
+      total[j] = sum;
     }
   }
-
-  // Sum the K-partials of the wavefronts.  D layout: lane holds H[token 4*(lane/16)+i][rank lane%16].
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(&s_red[((wave * RB + rb) * 64 + lane) * 4]) = acc[rb];
-  MLORA_STAMP(3);
-  __syncthreads();
-  MLORA_STAMP(4);
-  for (int e = tid; e < RB * 256; e += NT) {
-    const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-    float sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < kNW; ++w) sum += s_red[((w * RB + rb) * 64 + ln) * 4 + i];
-    const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
-    if (r < R) {
-      const float v = (!MASKED || r < eff) ? sum * scaling : 0.f;  // ranks the adapter does not have contribute nothing
-      const T hi = from_f32<T>(v);
-      s_hi[tok * HSTRIDE + r] = hi;
-      s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+  for (int j = 0; j < EPT; ++j) {
+    const int e = tid + j * NT;
+    if (WORDS % NT == 0 || e < WORDS) {
+      const int rb = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+      const int tok = 4 * (ln >> 4) + i, r = rb * 16 + (ln & 15);
+      if (r < R) {
+        const float v = (!MASKED || r < eff) ? total[j] * scaling : 0.f;  // ranks the adapter does not have contribute nothing
+        const T hi = from_f32<T>(v);
+        s_hi[tok * HSTRIDE + r] = hi;
+        s_lo[tok * HSTRIDE + r] = from_f32<T>(v - to_f32(hi));
+      }
     }
   }
   __syncthreads();
   MLORA_STAMP(5);  // the intermediate is in LDS
+  // This workgroup reads the exchange area no more.  Sent behind the last barrier: the compiler
+  // waits for the count on the spot (it is requested inside a branch), and in front of a barrier
+  // the whole workgroup would wait with the wavefront that sent it.
+  count_sent();
 
   // ---- expand: tokens as MFMA rows, lane holds out[token 4 * lg + i][column c0 + 4 * lr + j] ----
   Pack8 hop[KSTEPS], hlo[KSTEPS];
@@ -339,6 +532,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
     if (c0 < sp.n1) finish_span(c0, bop[s], yq[s]);
   }
   MLORA_STAMP(6);
+  count_seen();
 #ifdef MLORA_TRACE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   MLORA_STAMP(7);
@@ -350,13 +544,15 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
 // Leading arguments up to `packed` (13 dwords) arrive preloaded in scalar registers: everything the
 // early requests need.  packed = columns per range / 64 | ranges of slice 0 << 8 | slots << 16.
 // A launch of one slice passes n1 = 0 (blockIdx.y never reaches a second slice).
-template <typename T, int R, int KSPW, bool MASKED, int SA>
+// KP > 1: one slice, blockIdx.y is the workgroup's K part and column range alike (ranges of slice 0 = KP).
+template <typename T, int R, int KSPW, int KP, bool MASKED, int SA>
 __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restrict__ recs, const void* __restrict__ a0,
                                                           const void* __restrict__ b0, const void* __restrict__ a1,
                                                           const void* __restrict__ b1, int n0, int n1, uint32_t packed,
                                                           const void* __restrict__ xv, void* __restrict__ yv_, int64_t xs, int64_t ys,
                                                           int y_col0, int y_col1, uint32_t check, float scaling,
-                                                          const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr) {
+                                                          const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr,
+                                                          uint32_t* __restrict__ ws, int spin_ticks, int trusted) {
   constexpr int RB = (R + 15) / 16;
   constexpr int HSTRIDE = R + 8;
   constexpr int kStageRow = 17;
@@ -365,6 +561,7 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restr
   __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
   __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
   __shared__ __attribute__((aligned(16))) i32x4 s_stage[kNW * (1 + SB) * 16 * kStageRow];
+  __shared__ int s_ok;
   MLORA_STAMP(0);
 
   const int nt = static_cast<int>(packed & 255u) * 64, ranges0 = static_cast<int>((packed >> 8) & 255u);
@@ -382,15 +579,16 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restr
   // grid (8, column ranges, slot layers + layers of further tiles): blockIdx.x is the XCD, so a
   // slot's column ranges share an L2
   const int zslots = (num_slots + 7) >> 3;
+  const Exchange xc{ws, spin_ticks, trusted};
   if (static_cast<int>(blockIdx.z) < zslots) {
     const int s = blockIdx.z * 8 + blockIdx.x;  // its record exists: the list is rounded up to eight
     const int slot = s < num_slots ? s : num_slots - 1;
-    slot_tile<T, R, KSPW, MASKED, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
-                                            scaling, eff_rank, check, plan_hdr, s_red, s_hi, s_lo, s_stage);
+    slot_tile<T, R, KSPW, KP, MASKED, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), sp, y_col0, y_col1, second, xv, yv_,
+                                                xs, ys, num_slots, scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   } else {
     const int q = zslots * 8 + (blockIdx.z - zslots) * 8 + blockIdx.x;
-    slot_tile<T, R, KSPW, MASKED, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots, scaling,
-                                             eff_rank, check, plan_hdr, s_red, s_hi, s_lo, s_stage);
+    slot_tile<T, R, KSPW, KP, MASKED, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
+                                                 scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   }
 }
 
@@ -399,44 +597,53 @@ struct Launch {
   dim3 grid;
   uint32_t packed;
   int widest;
+  int spin_ticks, trusted;
 };
 
-template <typename T, int R, int KSPW, bool MASKED, int SA>
+template <typename T, int R, int KSPW, int KP, bool MASKED, int SA>
 void launch_spans(const Launch& l) {
   const MloraAddArgs* a = l.a;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
   const MloraSlice& s0 = a->slices[0];
   const MloraSlice s1 = a->num_slices > 1 ? a->slices[1] : MloraSlice{nullptr, nullptr, 0, 0};
-  hipLaunchKernelGGL((slot_kernel<T, R, KSPW, MASKED, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+  hipLaunchKernelGGL((slot_kernel<T, R, KSPW, KP, MASKED, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan + lay.slotrec_off, s0.a, s0.b, s1.a, s1.b, s0.n, s1.n, l.packed, a->x, a->y, a->x_stride, a->y_stride,
                      s0.y_col, s1.y_col, static_cast<uint32_t>(MLORA_PLAN_CHECK(a->num_tokens, a->num_slots)), a->scaling,
-                     a->effective_rank, const_cast<int32_t*>(a->plan));
+                     a->effective_rank, const_cast<int32_t*>(a->plan), static_cast<uint32_t*>(a->workspace), l.spin_ticks, l.trusted);
 }
 
-template <typename T, int R, int KSPW>
+template <typename T, int R, int KSPW, int KP>
 void launch_one(const Launch& l) {
   if (l.a->effective_rank) {
-    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, true, 1>(l);
-    else launch_spans<T, R, KSPW, true, 2>(l);
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, true, 1>(l);
+    else launch_spans<T, R, KSPW, KP, true, 2>(l);
   } else {
-    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, false, 1>(l);
-    else launch_spans<T, R, KSPW, false, 2>(l);
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, false, 1>(l);
+    else launch_spans<T, R, KSPW, KP, false, 2>(l);
   }
 }
 
+// kp: K parts (1: every workgroup multiplies the whole of K).
 template <typename T>
-bool launch_rank(const Launch& l, int r, int kspw) {
-  if (kspw == 4) {
+bool launch_rank(const Launch& l, int r, int kspw, int kp) {
+  if (kspw == 4 && kp == 1) {
     switch (r) {
-      case 8: launch_one<T, 8, 4>(l); return true;
-      case 16: launch_one<T, 16, 4>(l); return true;
-      case 32: launch_one<T, 32, 4>(l); return true;
-      case 64: launch_one<T, 64, 4>(l); return true;
+      case 8: launch_one<T, 8, 4, 1>(l); return true;
+      case 16: launch_one<T, 16, 4, 1>(l); return true;
+      case 32: launch_one<T, 32, 4, 1>(l); return true;
+      case 64: launch_one<T, 64, 4, 1>(l); return true;
     }
-  } else if (kspw == 16) {
+  } else if (kspw == 4 && kp == 4) {
     switch (r) {
-      case 8: launch_one<T, 8, 16>(l); return true;
-      case 16: launch_one<T, 16, 16>(l); return true;
+      case 8: launch_one<T, 8, 4, 4>(l); return true;
+      case 16: launch_one<T, 16, 4, 4>(l); return true;
+      case 32: launch_one<T, 32, 4, 4>(l); return true;
+      case 64: launch_one<T, 64, 4, 4>(l); return true;
+    }
+  } else if (kspw == 16 && kp == 1) {
+    switch (r) {
+      case 8: launch_one<T, 8, 16, 1>(l); return true;
+      case 16: launch_one<T, 16, 16, 1>(l); return true;
     }
   }
   return false;
@@ -444,10 +651,40 @@ bool launch_rank(const Launch& l, int r, int kspw) {
 
 int kspw_of(const MloraAddArgs* a) { return a->k % (32 * kNW) == 0 ? a->k / (32 * kNW) : 0; }
 
+// Diagnostic knobs, read from the environment once per process.
+struct SlotKnobs {
+  int generation = -1, kparts, spin_ticks;
+  void read() {
+    generation = knob_generation();
+    kparts = env_int("MLORA_SLOT_KPARTS", 4);          // 1: never share K out between workgroups
+    spin_ticks = env_int("MLORA_SLOT_SPIN_TICKS", 20000);  // 200 us; 0: do not wait; < 0: never accept a partner's words
+  }
+};
+SlotKnobs& slot_knobs() {
+  static SlotKnobs k;
+  if (k.generation != knob_generation()) k.read();
+  return k;
+}
+
+// K parts of a launch: four for K = 4096 when the tile's workgroups can hand each other partial
+// sums (one slice of at most 4096 columns, a workspace whose exchange area holds every tile's parts),
+// else one.
+int k_parts(const MloraAddArgs* a) {
+  if (a->k != 4096 || a->num_slices != 1 || slot_knobs().kparts != 4) return 1;
+  if (a->slices[0].n > 4 * 1024 || a->slices[0].n < 4 * 64) return 1;
+  if (a->r == 64 && a->slices[0].n > 4 * 512) return 1;  // (two spans per wavefront at rank 64 do not fit the registers beside the parts)
+  if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 255) || a->workspace_bytes < MLORA_WORKSPACE_HEAD_BYTES) return 1;
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+  const long long words = static_cast<long long>(lay.cap_slotrec + lay.cap_over) * 4 * ((a->r + 15) / 16) * 256;
+  if (words * 8 > kWsXchgBytes) return 1;
+  return 4;
+}
+
 }  // namespace
 
-// K = 1024 at every rank, K = 4096 up to rank 16 (what fits the register file as one batch of
-// loads), one or two slices (what fits the preloaded arguments), 16-bit elements.
+// K = 1024 at every rank; K = 4096 at every rank with the K parts of a tile shared out between its
+// workgroups, else up to rank 16 (what fits the register file as one batch of loads); one or two
+// slices (what fits the preloaded arguments); 16-bit elements.
 bool slot_supported(const MloraAddArgs* a) {
   if (a->dtype != MLORA_DTYPE_BF16 && a->dtype != MLORA_DTYPE_F16) return false;
   if (a->num_slices < 1 || a->num_slices > 2 || !a->plan) return false;
@@ -457,9 +694,10 @@ bool slot_supported(const MloraAddArgs* a) {
     cols += a->slices[i].n;
   }
   if (cols > 200 * 1024) return false;  // at most 255 column ranges of up to 1024 columns
+  if (a->r != 8 && a->r != 16 && a->r != 32 && a->r != 64) return false;
   const int kspw = kspw_of(a);
-  if (kspw == 4) return a->r == 8 || a->r == 16 || a->r == 32 || a->r == 64;
-  if (kspw == 16) return a->r == 8 || a->r == 16;
+  if (kspw == 4) return true;
+  if (kspw == 16) return a->r <= 16 || k_parts(a) == 4;
   return false;
 }
 
@@ -471,6 +709,7 @@ void slot_trace_set(void* buf) {
 #endif
 }
 
+namespace {
 // Columns per range: as in the tile-major launch, sized for 150-250 workgroups; at most 1024 (two
 // 64-column spans per wavefront, all loads in registers).
 int range_columns(const MloraAddArgs* a) {
@@ -491,11 +730,14 @@ int range_columns(const MloraAddArgs* a) {
   }
   return nt > 1024 ? 1024 : nt;
 }
+}  // namespace
 
-int launch_slot(const MloraAddArgs* a) {
+int launch_slot(const MloraAddArgs* a, bool trusted_workspace) {
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  const int nt = range_columns(a);
-  const int ranges0 = (a->slices[0].n + nt - 1) / nt;
+  const int kp = k_parts(a);
+  // with K parts the tile's workgroups are its K parts and its column ranges alike
+  const int nt = kp > 1 ? ((a->slices[0].n + kp - 1) / kp + 63) & ~63 : range_columns(a);
+  const int ranges0 = kp > 1 ? kp : (a->slices[0].n + nt - 1) / nt;
   const int total = ranges0 + (a->num_slices > 1 ? (a->slices[1].n + nt - 1) / nt : 0);
   if (total > 255) {
     set_error("mlora_add_lora(slot-major): %d column ranges exceed 255", total);
@@ -509,9 +751,11 @@ int launch_slot(const MloraAddArgs* a) {
     const int w = a->slices[i].n < nt ? a->slices[i].n : nt;
     if (w > l.widest) l.widest = w;
   }
+  l.spin_ticks = slot_knobs().spin_ticks;
+  l.trusted = trusted_workspace ? 1 : 0;
   l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>((lay.cap_slotrec + lay.cap_over) / 8));
-  const int kspw = kspw_of(a);
-  const bool ok = a->dtype == MLORA_DTYPE_BF16 ? launch_rank<__bf16>(l, a->r, kspw) : launch_rank<_Float16>(l, a->r, kspw);
+  const int kspw = kspw_of(a) / kp;
+  const bool ok = a->dtype == MLORA_DTYPE_BF16 ? launch_rank<__bf16>(l, a->r, kspw, kp) : launch_rank<_Float16>(l, a->r, kspw, kp);
   if (!ok) {
     set_error("mlora_add_lora(slot-major): unsupported rank %d / K %d", a->r, a->k);
     return MLORA_E_UNSUPPORTED;

@@ -161,7 +161,7 @@ def _slot_form_batches(T, L, seed):
 
 @pytest.mark.parametrize("name,rank,T,L", [("o", 16, 256, 32), ("gate_up", 16, 256, 32), ("down", 16, 256, 32), ("o", 32, 64, 32),
                                            ("gate_up", 64, 100, 5), ("o", 8, 37, 13), ("down", 8, 300, 9), ("gate_up", 32, 19, 64)])
-def test_slot_major_grid_gives_the_bits_of_the_tile_major_grid(name, rank, T, L):
+def test_slot_major_grid_gives_the_bits_of_the_tile_major_grid(name, rank, T, L, monkeypatch):
     """The slot-major form requests a slot's weights before its record has arrived; what it computes
     is the small-tile form's arithmetic in the same order, so its results are the oracle's and,
     bit for bit, those of the tile-major grid - for slots without tokens, slot ids that are not a
@@ -176,7 +176,57 @@ def test_slot_major_grid_gives_the_bits_of_the_tile_major_grid(name, rank, T, L)
         got = _apply("slot", proj, x, y0.clone(), slots)
         exact, mag = _exact(proj, x, y0, slots)
         _check(got, y0, exact, mag, slots, f"slot-major/{name}/r{rank}/{tag}")
-        assert torch.equal(got, _apply("mfma", proj, x, y0.clone(), slots)), tag
+        if proj.k == 4096:  # the tile's workgroups share K out: another order of additions than one workgroup's
+            _knobs(monkeypatch, MLORA_SLOT_KPARTS=1)
+            assert torch.equal(_apply("slot", proj, x, y0.clone(), slots), _apply("mfma", proj, x, y0.clone(), slots)), tag
+            _knobs(monkeypatch, MLORA_SLOT_KPARTS=None)
+        else:
+            assert torch.equal(got, _apply("mfma", proj, x, y0.clone(), slots)), tag
+
+
+@pytest.mark.parametrize("rank,T,L", [(16, 256, 32), (8, 90, 12), (32, 200, 24), (64, 64, 7)])
+def test_slot_major_grid_shares_long_k_out_between_the_workgroups_of_a_tile(rank, T, L, monkeypatch):
+    """K = 4096: the four workgroups of a tile each multiply a quarter of K, publish their partial
+    sums in the workspace, pick the others' up and expand a quarter of the columns.  Checked: the
+    oracle's result; the same bits from one launch to the next, with the partners' words accepted,
+    never accepted (every workgroup multiplies all parts itself) and not waited for; no wait running
+    out in the ordinary runs; the workspace's generation one step on per launch with the arrival
+    count back at zero; the same bits on a workspace that was never initialised; slot -1 rows untouched."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
+
+    proj = _make("down", L, rank, torch.bfloat16, seed=180 + rank)
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=181, device="cuda")
+    for tag, slots in _slot_form_batches(T, L, 182 + T).items():
+        print(f"slot-major, K parts, r={rank} T={T} L={L} {tag}", flush=True)
+        slots = slots.cuda()
+        backend = _backend("slot")
+        meta = _metadata(slots)
+
+        def run():
+            y = y0.clone()
+            backend.add_lora([y], x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)
+            return y
+
+        runs = []
+        for spin in (20000, 20000, -1, 0):
+            _knobs(monkeypatch, MLORA_SLOT_SPIN_TICKS=spin)
+            runs.append(run())
+            if spin > 0:
+                assert _waits_run_out(backend) == 0, "a workgroup gave up waiting for its partners"
+        exact, mag = _exact(proj, x, y0, slots)
+        _check(runs[0], y0, exact, mag, slots, f"slot-major K parts/r{rank}/{tag}")
+        for other in runs[1:]:
+            assert torch.equal(runs[0], other), tag
+        (scratch,) = backend._scratch.values()
+        head = scratch[: _hip.WORKSPACE_HEAD_BYTES].view(torch.int32)
+        want_check = ((len(runs) ^ 0x9E3779B9) + (1 << 31)) % (1 << 32) - (1 << 31)
+        assert head[256 // 4 : 256 // 4 + 3].tolist() == [len(runs), 0, want_check]
+        scratch[:4].zero_()  # no signature: nobody publishes, nobody waits
+        _knobs(monkeypatch, MLORA_SLOT_SPIN_TICKS=20000)
+        assert torch.equal(run(), runs[0])
+        assert _waits_run_out(backend) == 0
+        assert head[256 // 4 : 256 // 4 + 3].tolist() == [len(runs), 0, want_check]
+    _knobs(monkeypatch, MLORA_SLOT_SPIN_TICKS=None)
 
 
 @pytest.mark.parametrize("rank", [16, 64])
@@ -559,6 +609,22 @@ def test_auto_form_follows_rank_and_width(rank, expected):
     exact, mag = _exact(proj, x, y0, slots)
     _check(got, y0, exact, mag, slots, f"auto/r{rank}")
     assert torch.equal(got, _apply(expected, proj, x, y0.clone(), slots))
+
+
+@pytest.mark.parametrize("rank", [16, 32, 64])
+def test_auto_shares_k_of_4096_out_in_the_slot_major_form(rank):
+    """down of the decode batch: AUTO takes the slot-major form, whose workgroups share K out between
+    them, at every rank (where the split form used to be taken for ranks 32 and 64)."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"auto, K = 4096, r={rank}", flush=True)
+    proj = _make("down", 32, rank, torch.bfloat16, seed=345 + rank)
+    x, y0 = synthetic.make_activations(256, proj.k, sum(proj.widths), torch.bfloat16, seed=346, device="cuda")
+    slots = synthetic.decode_slots(256, 32, seed=347).cuda()
+    got = _apply("auto", proj, x, y0.clone(), slots)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, f"auto/down/r{rank}")
+    assert torch.equal(got, _apply("slot", proj, x, y0.clone(), slots))
 
 
 @pytest.mark.parametrize("rank", [16, 32])
