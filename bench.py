@@ -560,8 +560,8 @@ def main() -> None:
     ap.add_argument("--no-extras", action="store_true",
                     help="skip what the default run adds after the headline: the prefill, mixed and backbone steps and the floor")
     ap.add_argument("--floor", action="store_true", help="print only the floor measurements (launch costs and stream rates)")
-    ap.add_argument("--rank", type=int, default=0, choices=(0, 8, 16, 32, 64),
-                    help="diagnostic: the decode or prefill workload at another adapter rank; 0 = the workload's own")
+    ap.add_argument("--rank", type=int, default=0,
+                    help="the decode or prefill workload at another adapter rank (buffers of that rank); 0 = the workload's own")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device tensor copy, as the known-size reference "
                          "that rocprof byte counters of the same run are scaled by")

@@ -63,7 +63,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 bool vector_ok(const MloraAddArgs* a) {
   if (a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) return false;
   if (!a->plan) return false;
-  if (a->r != 8 && a->r != 16 && a->r != 32 && a->r != 64) return false;
+  if (!padded_rank(a->r)) return false;  // 8, 16, 24, ... 64: rows of B start on 16-byte boundaries
   if (a->k % 8 || a->x_stride % 8 || a->y_stride % 8) return false;
   if (!aligned16(a->x) || !aligned16(a->y)) return false;
   for (int i = 0; i < a->num_slices; ++i) {
@@ -212,7 +212,8 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     case MLORA_FORM_TOKEN:
       return launch_token_add(a);
     case MLORA_FORM_BGMV:
-      if (a->effective_rank && a->form == MLORA_FORM_AUTO) return launch_token_add(a);  // the vector-ALU tiles read whole rank-r rows
+      if ((a->effective_rank || !exact_rank(a->r)) && a->form == MLORA_FORM_AUTO) return launch_token_add(a);  // the vector-ALU tiles read whole rank-r rows
+      if (!exact_rank(a->r)) { set_error("mlora_add_lora: the BGMV form takes ranks 8, 16, 32 and 64"); return MLORA_E_UNSUPPORTED; }
       if (a->effective_rank) { set_error("mlora_add_lora: the BGMV form does not take effective_rank"); return MLORA_E_UNSUPPORTED; }
       if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
       return launch_bgmv(a, /*include_long=*/true);
@@ -221,7 +222,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     case MLORA_FORM_SPLIT:
     case MLORA_FORM_SLOT:
     case MLORA_FORM_MFMA: {
-      if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, rank in {8,16,32,64} and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
+      if (!vec || !mfma_supported(a)) { set_error("mlora_add_lora: MFMA forms need 16-bit elements, a plan, a rank that is a multiple of 8 up to 64 and K %% 32 == 0"); return MLORA_E_UNSUPPORTED; }
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
       if (form == MLORA_FORM_SLOT) {
         if (!slot_supported(a)) {
@@ -233,13 +234,13 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
       }
       if (form == MLORA_FORM_SPLIT) {
         if (!split_supported(a)) {
-          set_error("mlora_add_lora: the split form needs K %% 512 == 0, at most 8 K parts, no empty slice and a 256-byte aligned "
+          set_error("mlora_add_lora: the split form needs a rank of 8, 16, 32 or 64, K %% 512 == 0, at most 8 K parts, no empty slice and a 256-byte aligned "
                     "workspace of at least %d bytes whose exchange area holds every tile's partial sums", MLORA_WORKSPACE_HEAD_BYTES);
           return MLORA_E_UNSUPPORTED;
         }
         return launch_split(a, /*include_long=*/true, trusted_workspace);
       }
-      if (!sgmv_supported(a)) { set_error("mlora_add_lora: SGMV form needs K %% 128 == 0"); return MLORA_E_UNSUPPORTED; }
+      if (!sgmv_supported(a)) { set_error("mlora_add_lora: SGMV form needs K %% 128 == 0 and a rank of 8, 16, 32 or 64"); return MLORA_E_UNSUPPORTED; }
       if (!sgmv_workspace_ok(a)) {
         set_error("mlora_add_lora: SGMV form needs a 16-byte aligned workspace of %zu bytes and no empty slice",
                   sgmv_workspace_bytes(a->num_tokens, a->num_slices, a->r, a->dtype));

@@ -66,11 +66,17 @@ struct DecodeSplits {
 // SA: spans per wavefront requested up front.  A launch whose column ranges are at most 512 columns
 // wide (one span per wavefront) takes the instance with SA = 1: the second span's requests, though
 // clamped to a line or two, cost 0.2 us per launch (o 4.31 -> 4.07, qkv 4.44 -> 4.25, down 7.02 -> 6.81).
-template <typename T, int R, int KSPW, bool TR, bool MASKED, int SA>
+//
+// GR (with MASKED): the buffers' rank is `rbuf_arg` < R, a multiple of eight (24 in the instance for
+// 32; 40, 48, 56 in the one for 64): rows of A[slot] are rbuf * K apart, B rows rbuf elements long, and
+// whatever lies beyond rbuf is treated like the ranks beyond an adapter's own (requests clamped
+// into the buffers, values masked).
+template <typename T, int R, int KSPW, bool TR, bool MASKED, int SA, bool GR = false>
 __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __restrict__ plan, const void* __restrict__ xv,
                                                             void* __restrict__ yv_, int64_t xs, int64_t ys, int small_off,
                                                             int include_long, int T_, int K, int num_slots, float scaling,
-                                                            const int32_t* __restrict__ eff_rank, DecodeSplits splits) {
+                                                            const int32_t* __restrict__ eff_rank, int rbuf_arg, DecodeSplits splits) {
+  static_assert(!GR || (MASKED && R >= 32), "buffers of a rank between the instances' take the masked code of the next instance up");
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks of the shrink output
   constexpr int KSTEPS = (R + 31) / 32;  // MFMA k-steps of the expand
   constexpr int HSTRIDE = R + 8;         // padded LDS row of the intermediate
@@ -88,6 +94,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
+  const int rbuf = GR ? rbuf_arg : R;  // rank of the buffers: row count of A[slot], row length of B
   MLORA_STAMP(0);  // first instruction
 
   // grid (8, column ranges, tiles / 8): linear workgroup ids advance along x first and
@@ -128,20 +135,21 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
   // rank of the adapter in this slot (requested together with the record, see rank_prefetch)
   // (MASKED = false is the instance for callers that gave no rank vector: eff is the constant R
   // there and every test on it below folds away)
-  const int eff = MASKED ? rank_pick(ranks, eff_rank, num_slots, slot, R) : R;
+  int eff = MASKED ? rank_pick(ranks, eff_rank, num_slots, slot, R) : R;
+  if (GR && eff > rbuf) eff = rbuf;
   if (MASKED && eff == 0) return;
   const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
 
   const bool live = lr < m;  // this lane's token exists
   const T* xrow = static_cast<const T*>(xv) + static_cast<int64_t>(row) * xs + lg * 8;
-  const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+  const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * rbuf * K;
   const T* arow[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int rr = rb * 16 + lr;
-    arow[rb] = A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + lg * 8;
+    arow[rb] = A + static_cast<int64_t>(rr < rbuf ? rr : rbuf - 1) * K + lg * 8;
   }
-  const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
+  const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * rbuf;
   T* yrow = static_cast<T*>(yv_) + static_cast<int64_t>(row) * ys + sp.y_col + 16 * lg;
 
   // ---- round trip 2: issue every load ---------------------------------------------------------
@@ -162,7 +170,7 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           const int rr = rb * 16 + 4 * lg + i;
-          if (!MASKED || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          if (!MASKED || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < rbuf ? rr : rbuf - 1) * K + koff);
           else ast[rb][4 * r + i] = i32x4{0, 0, 0, 0};
         }
       }
@@ -203,8 +211,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int kc = (lg + 4 * ks) & (R / 8 - 1);
-          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          int kc = (lg + 4 * ks) & (R / 8 - 1);
+          if (GR && kc * 8 >= rbuf) kc = rbuf / 8 - 1;  // (masked where it is used)
+          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * rbuf + kc * 8);
         }
       }
     }
@@ -231,8 +240,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
           for (int ks = 0; ks < KSTEPS; ++ks) {
             // lanes whose chunk lies beyond the rank fetch a valid chunk anyway: their H operand is
             // zero, and an unconditional load keeps the whole batch of loads in flight together
-            const int kc = (lg + 4 * ks) & (R / 8 - 1);
-            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+            int kc = (lg + 4 * ks) & (R / 8 - 1);
+            if (GR && kc * 8 >= rbuf) kc = rbuf / 8 - 1;  // (masked where it is used)
+            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * rbuf + kc * 8);
           }
         }
 #pragma unroll
@@ -469,8 +479,9 @@ __global__ __launch_bounds__(kNW* kWave) void decode_kernel(const int32_t* __res
         n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int kc = (lg + 4 * ks) & (R / 8 - 1);
-          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+          int kc = (lg + 4 * ks) & (R / 8 - 1);
+          if (GR && kc * 8 >= rbuf) kc = rbuf / 8 - 1;  // (masked where it is used)
+          bo[j][ks].raw = load128(B + static_cast<int64_t>(n) * rbuf + kc * 8);
         }
       }
 #pragma unroll
@@ -495,12 +506,12 @@ struct Launch {
   const DecodeSplits* splits;
 };
 
-template <typename T, int R, int KSPW, bool TR, bool MASKED, int SA>
+template <typename T, int R, int KSPW, bool TR, bool MASKED, int SA, bool GR = false>
 void launch_spans(const Launch& l) {
   const MloraAddArgs* a = l.a;
-  hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR, MASKED, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+  hipLaunchKernelGGL((decode_kernel<T, R, KSPW, TR, MASKED, SA, GR>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
                      a->plan, a->x, a->y, a->x_stride, a->y_stride, l.small_off, l.include_long, a->num_tokens, a->k,
-                     a->num_slots, a->scaling, a->effective_rank, *l.splits);
+                     a->num_slots, a->scaling, a->effective_rank, a->r, *l.splits);
 }
 
 // One span per wavefront up front when no column range holds more (staged form; the other form
@@ -524,6 +535,17 @@ void launch_one(const Launch& l) {
 // and 16 (K = 4096) where the loads of sixteen steps still fit the register file.
 template <typename T, int R>
 void launch_kspw(const Launch& l, int kspw) {
+  if constexpr (R >= 32) {
+    if (l.a->r != R) {
+      // buffers of a rank between the instances' (24; 40, 48, 56): the masked code of this instance
+      // with the buffers' rank as stride, in the staged form for K = 1024 and the general one else
+      if (l.staged && kspw == 4) {
+        if (l.widest <= kNW * 64) return launch_spans<T, R, 4, true, true, 1, true>(l);
+        return launch_spans<T, R, 4, true, true, kSpansAheadMax, true>(l);
+      }
+      return launch_spans<T, R, 0, false, true, kSpansAheadMax, true>(l);
+    }
+  }
   if (l.staged) {
     // staged operands, the k-steps of a wavefront four at a time (rank 64 in two passes of 32 ranks
     // through the same LDS block); how many k-steps fit is a matter of registers: every load of
@@ -548,7 +570,7 @@ void launch_kspw(const Launch& l, int kspw) {
 
 template <typename T>
 void launch_rank(const Launch& l, int r, int kspw) {
-  switch (r) {
+  switch (compute_rank(r)) {
     case 8: launch_kspw<T, 8>(l, kspw); break;
     case 16: launch_kspw<T, 16>(l, kspw); break;
     case 32: launch_kspw<T, 32>(l, kspw); break;

@@ -8,6 +8,14 @@
 namespace mlora {
 
 int env_int(const char* name, int fallback);
+
+// Ranks the kernels are instantiated for.  Buffers of another rank that is a multiple of eight and
+// at most 64 (24, 40, 48, 56) run on the next instance up in the small-tile kernels, with the
+// buffers' rank as the run-time stride and everything beyond it masked as for an adapter of lower
+// rank; the other forms take exact ranks only.
+inline bool exact_rank(int r) { return r == 8 || r == 16 || r == 32 || r == 64; }
+inline bool padded_rank(int r) { return r >= 8 && r <= 64 && r % 8 == 0; }
+inline int compute_rank(int r) { return r <= 8 ? 8 : r <= 16 ? 16 : r <= 32 ? 32 : 64; }
 // Diagnostic knobs are read from the environment once and kept; mlora_reload_knobs() advances
 // this number, and a holder whose copy is older reads its variables again.
 int knob_generation();

@@ -242,7 +242,7 @@ void sgmv_trace_set(void* buf) {
 #endif
 }
 
-bool sgmv_supported(const MloraAddArgs* a) { return a->k % 128 == 0 && a->k >= 128; }
+bool sgmv_supported(const MloraAddArgs* a) { return a->k % 128 == 0 && a->k >= 128 && exact_rank(a->r); }
 
 // A workspace that holds at least one partial can be used (fewer K parts are taken then).
 bool sgmv_workspace_ok(const MloraAddArgs* a) {

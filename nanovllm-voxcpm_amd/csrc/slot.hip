@@ -65,8 +65,11 @@ struct Exchange {
 
 typedef unsigned long long u64;
 
-template <typename T, int R, int KSPW, int KP, bool MASKED, int SA, bool EARLY>
-__device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const int slot_early, const int early_ok, const Range sp,
+// GR (with MASKED): the buffers' rank is `rbuf` < R, a multiple of eight: rows of A[slot] are rbuf * K
+// apart and B rows rbuf elements long; whatever lies beyond rbuf is treated like the ranks beyond
+// an adapter's own (requests clamped into the buffers, values masked).
+template <typename T, int R, int KSPW, int KP, bool MASKED, bool GR, int SA, bool EARLY>
+__device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const int slot_early, const int early_ok, const int rbuf_arg, const Range sp,
                                           const int y_col0, const int y_col1, const bool second, const void* __restrict__ xv,
                                           void* __restrict__ yv_, const int64_t xs, const int64_t ys,
                                           const int num_slots, const float scaling, const int32_t* __restrict__ eff_rank,
@@ -84,10 +87,12 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   constexpr int kStageRow = 17;          // 16 chunks of 16 bytes + one of padding
   constexpr int SB = RB < 2 ? RB : 2;    // 16-rank blocks of A staged together
   constexpr bool K16 = R == 16;          // expand on the 16x16x16 MFMA: 64-bit operand pieces
+  static_assert(!GR || (MASKED && R >= 32), "buffers of a rank between the instances' take the masked code of the next instance up");
   static_assert(KSPW >= 4 && KSPW % 4 == 0, "the k-steps of a wavefront are taken four at a time");
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int lr = lane & 15, lg = lane >> 4;
+  const int rbuf = GR ? rbuf_arg : R;  // rank of the buffers: row count of A[slot], row length of B
 
   // ---- requests that depend on nothing but the workgroup index --------------------------------
   // (the token rows as a vector load, four per lane group: all sixteen through the scalar cache
@@ -95,7 +100,9 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   const i32x4 rows4 = *reinterpret_cast<const i32x4*>(rec + MLORA_SMALL_TILE_ROWS + 4 * lg);  // tokens 4*lg .. 4*lg+3
   const i32x4 rec0 = *reinterpret_cast<const i32x4*>(rec);                                     // slot, count, start, check
   int eff_early = R;
-  if constexpr (MASKED && EARLY) eff_early = eff_rank[slot_early];
+  if constexpr (MASKED && EARLY) {
+    if (eff_rank) eff_early = eff_rank[slot_early];
+  }
   const RankPrefetch ranks = rank_prefetch((MASKED && !EARLY) ? eff_rank : nullptr, num_slots, lane);
   if constexpr (EARLY) __builtin_amdgcn_sched_barrier(0);  // the record's requests go out first
 
@@ -114,7 +121,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   Pack8 bop[SA][4][KSTEPS];
   // every A line of this wavefront's K range and the B rows of its spans
   auto request_weights = [&](const int slot, const int rb_n) {
-    const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+    const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * rbuf * K;
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
       const int64_t koff = static_cast<int64_t>(ks0 + 4 * r) * 32 + (lane & 15) * 8;
@@ -123,12 +130,12 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           const int rr = rb * 16 + 4 * lg + i;
-          if (!MASKED || EARLY || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+          if (!MASKED || EARLY || RB == 1 || rb < rb_n) ast[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < rbuf ? rr : rbuf - 1) * K + koff);
           else ast[rb][4 * r + i] = i32x4{0, 0, 0, 0};
         }
       }
     }
-    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * R;
+    const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * rbuf;
 #pragma unroll
     for (int s = 0; s < SA; ++s) {
       const int c0 = sp.n0 + (wave + s * kNW) * 64;
@@ -148,8 +155,9 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
           n = n < sp.n1 ? n : sp.n1 - 1;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int kc = (lg + 4 * ks) & (R / 8 - 1);
-            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * R + kc * 8);
+            int kc = (lg + 4 * ks) & (R / 8 - 1);
+            if (GR && kc * 8 >= rbuf) kc = rbuf / 8 - 1;  // (masked where it is used)
+            bop[s][j][ks].raw = load128(B + static_cast<int64_t>(n) * rbuf + kc * 8);
           }
         }
       }
@@ -234,6 +242,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
     } else {
       eff = rank_pick(ranks, eff_rank, num_slots, slot, R);
     }
+    if (GR && eff > rbuf) eff = rbuf;
     if (eff == 0) {
       count_done();
       if constexpr (EARLY) settle_requests();
@@ -390,7 +399,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
       for (int q = 0; q < KP; ++q) {
         if (q == kp) continue;
         i32x4 xo[4 * ROUNDS], ao[RB][4 * ROUNDS];
-        const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * R * K;
+        const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * rbuf * K;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
           const int64_t koff = static_cast<int64_t>(q * (KPART / 32) + wave * KSPW + 4 * r) * 32 + (lane & 15) * 8;
@@ -400,7 +409,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
               const int rr = rb * 16 + 4 * lg + i;
-              if (!MASKED || RB == 1 || rb < rb_n) ao[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < R ? rr : R - 1) * K + koff);
+              if (!MASKED || RB == 1 || rb < rb_n) ao[rb][4 * r + i] = load128(A + static_cast<int64_t>(rr < rbuf ? rr : rbuf - 1) * K + koff);
               else ao[rb][4 * r + i] = i32x4{0, 0, 0, 0};
             }
           }
@@ -541,14 +550,14 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
 #endif
 }
 
-// Leading arguments up to `packed` (13 dwords) arrive preloaded in scalar registers: everything the
+// Leading arguments up to `rbuf` (14 dwords) arrive preloaded in scalar registers: everything the
 // early requests need.  packed = columns per range / 64 | ranges of slice 0 << 8 | slots << 16.
 // A launch of one slice passes n1 = 0 (blockIdx.y never reaches a second slice).
 // KP > 1: one slice, blockIdx.y is the workgroup's K part and column range alike (ranges of slice 0 = KP).
-template <typename T, int R, int KSPW, int KP, bool MASKED, int SA>
+template <typename T, int R, int KSPW, int KP, bool MASKED, bool GR, int SA>
 __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restrict__ recs, const void* __restrict__ a0,
                                                           const void* __restrict__ b0, const void* __restrict__ a1,
-                                                          const void* __restrict__ b1, int n0, int n1, uint32_t packed,
+                                                          const void* __restrict__ b1, int n0, int n1, uint32_t packed, int rbuf,
                                                           const void* __restrict__ xv, void* __restrict__ yv_, int64_t xs, int64_t ys,
                                                           int y_col0, int y_col1, uint32_t check, float scaling,
                                                           const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr,
@@ -583,11 +592,11 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restr
   if (static_cast<int>(blockIdx.z) < zslots) {
     const int s = blockIdx.z * 8 + blockIdx.x;  // its record exists: the list is rounded up to eight
     const int slot = s < num_slots ? s : num_slots - 1;
-    slot_tile<T, R, KSPW, KP, MASKED, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), sp, y_col0, y_col1, second, xv, yv_,
+    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), rbuf, sp, y_col0, y_col1, second, xv, yv_,
                                                 xs, ys, num_slots, scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   } else {
     const int q = zslots * 8 + (blockIdx.z - zslots) * 8 + blockIdx.x;
-    slot_tile<T, R, KSPW, KP, MASKED, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
+    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, rbuf, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
                                                  scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   }
 }
@@ -600,32 +609,40 @@ struct Launch {
   int spin_ticks, trusted;
 };
 
-template <typename T, int R, int KSPW, int KP, bool MASKED, int SA>
+template <typename T, int R, int KSPW, int KP, bool MASKED, bool GR, int SA>
 void launch_spans(const Launch& l) {
   const MloraAddArgs* a = l.a;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
   const MloraSlice& s0 = a->slices[0];
   const MloraSlice s1 = a->num_slices > 1 ? a->slices[1] : MloraSlice{nullptr, nullptr, 0, 0};
-  hipLaunchKernelGGL((slot_kernel<T, R, KSPW, KP, MASKED, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
-                     a->plan + lay.slotrec_off, s0.a, s0.b, s1.a, s1.b, s0.n, s1.n, l.packed, a->x, a->y, a->x_stride, a->y_stride,
+  hipLaunchKernelGGL((slot_kernel<T, R, KSPW, KP, MASKED, GR, SA>), l.grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream),
+                     a->plan + lay.slotrec_off, s0.a, s0.b, s1.a, s1.b, s0.n, s1.n, l.packed, a->r, a->x, a->y, a->x_stride, a->y_stride,
                      s0.y_col, s1.y_col, static_cast<uint32_t>(MLORA_PLAN_CHECK(a->num_tokens, a->num_slots)), a->scaling,
                      a->effective_rank, const_cast<int32_t*>(a->plan), static_cast<uint32_t*>(a->workspace), l.spin_ticks, l.trusted);
 }
 
 template <typename T, int R, int KSPW, int KP>
 void launch_one(const Launch& l) {
+  if constexpr (R >= 32) {
+    if (l.a->r != R) {  // buffers of a rank between the instances': the masked code with the buffers' rank as stride
+      if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, true, true, 1>(l);
+      else launch_spans<T, R, KSPW, KP, true, true, 2>(l);
+      return;
+    }
+  }
   if (l.a->effective_rank) {
-    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, true, 1>(l);
-    else launch_spans<T, R, KSPW, KP, true, 2>(l);
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, true, false, 1>(l);
+    else launch_spans<T, R, KSPW, KP, true, false, 2>(l);
   } else {
-    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, false, 1>(l);
-    else launch_spans<T, R, KSPW, KP, false, 2>(l);
+    if (l.widest <= kNW * 64) launch_spans<T, R, KSPW, KP, false, false, 1>(l);
+    else launch_spans<T, R, KSPW, KP, false, false, 2>(l);
   }
 }
 
 // kp: K parts (1: every workgroup multiplies the whole of K).
 template <typename T>
-bool launch_rank(const Launch& l, int r, int kspw, int kp) {
+bool launch_rank(const Launch& l, int rank, int kspw, int kp) {
+  const int r = compute_rank(rank);
   if (kspw == 4 && kp == 1) {
     switch (r) {
       case 8: launch_one<T, 8, 4, 1>(l); return true;
@@ -672,10 +689,10 @@ SlotKnobs& slot_knobs() {
 int k_parts(const MloraAddArgs* a) {
   if (a->k != 4096 || a->num_slices != 1 || slot_knobs().kparts != 4) return 1;
   if (a->slices[0].n > 4 * 1024 || a->slices[0].n < 4 * 64) return 1;
-  if (a->r == 64 && a->slices[0].n > 4 * 512) return 1;  // (two spans per wavefront at rank 64 do not fit the registers beside the parts)
+  if (a->r > 32 && a->slices[0].n > 4 * 512) return 1;  // (two spans per wavefront at rank 64 do not fit the registers beside the parts)
   if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 255) || a->workspace_bytes < MLORA_WORKSPACE_HEAD_BYTES) return 1;
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  const long long words = static_cast<long long>(lay.cap_slotrec + lay.cap_over) * 4 * ((a->r + 15) / 16) * 256;
+  const long long words = static_cast<long long>(lay.cap_slotrec + lay.cap_over) * 4 * ((compute_rank(a->r) + 15) / 16) * 256;
   if (words * 8 > kWsXchgBytes) return 1;
   return 4;
 }
@@ -694,7 +711,7 @@ bool slot_supported(const MloraAddArgs* a) {
     cols += a->slices[i].n;
   }
   if (cols > 200 * 1024) return false;  // at most 255 column ranges of up to 1024 columns
-  if (a->r != 8 && a->r != 16 && a->r != 32 && a->r != 64) return false;
+  if (!padded_rank(a->r)) return false;
   const int kspw = kspw_of(a);
   if (kspw == 4) return true;
   if (kspw == 16) return a->r <= 16 || k_parts(a) == 4;

@@ -579,7 +579,7 @@ static int pick_kpart(const MloraAddArgs* a, int wanted) {
 // exchange area).
 bool split_supported(const MloraAddArgs* a) {
   if (!a->workspace || (reinterpret_cast<uintptr_t>(a->workspace) & 255) || a->workspace_bytes < MLORA_WORKSPACE_HEAD_BYTES) return false;
-  if (a->k % 512 != 0 || a->k < 512) return false;
+  if (a->k % 512 != 0 || a->k < 512 || !exact_rank(a->r)) return false;
   if (plan_layout(a->num_tokens, a->num_slots).cap_small > kWsTiles) return false;
   for (int i = 0; i < a->num_slices; ++i)
     if (a->slices[i].n <= 0) return false;

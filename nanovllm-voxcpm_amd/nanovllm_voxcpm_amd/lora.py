@@ -94,7 +94,7 @@ class _UnavailableBackend:
     shrink = expand = add_lora = _refuse
 
 
-_VECTOR_RANKS = (8, 16, 32, 64)
+_VECTOR_RANKS = (8, 16, 24, 32, 40, 48, 56, 64)  # rows of B start on 16-byte boundaries and an instance of the kernels covers them
 _PLAN_ATTR = "_mlora_segment_plans"
 _CONTEXT_PLANS_ATTR = "_mlora_context_plans"  # plan table of the LoRAContext a metadata object was made from
 

@@ -397,6 +397,69 @@ def test_ranks_and_dtypes_small(rank, dtype, form):
     _check(got, y0, exact, mag, slots, f"rank{rank}/{dtype}/{form}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [24, 40, 48, 56])
+def test_ranks_between_the_kernel_instances_run_on_the_matrix_cores(rank, dtype):
+    """Buffers of rank 24, 40, 48, 56 (the reference takes any max_lora_rank): the small-tile kernels
+    of the next rank up take them with the buffers' rank as stride and everything beyond it masked.
+    Ragged widths at K = 256 (the general instance), the four projection shapes at decode size (staged
+    instance, slot-major grid, K shared out at 4096) and a 1500-token batch; NaN beyond every slot's
+    own rank; a slot vector with rows without adapter.  AUTO and the forms it picks from give the
+    fp64 result; the forms that take exact ranks only say so."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"in-between rank {rank} {dtype}", flush=True)
+    shapes = {"p": (256, [64, 136, 8])}
+    proj = synthetic.make_projection("p", 6, rank, dtype, seed=17 + rank, device="cuda", shapes=shapes)
+    x, y0 = synthetic.make_activations(75, 256, 208, dtype, seed=19, device="cuda")
+    g = torch.Generator().manual_seed(rank)
+    slots = torch.randint(-1, 6, (75,), generator=g, dtype=torch.int32).cuda()
+    exact, mag = _exact(proj, x, y0, slots, scaling=0.5)
+    for form in ("auto", "mfma", "token"):
+        _check(_apply(form, proj, x, y0.clone(), slots, scaling=0.5), y0, exact, mag, slots, f"rank{rank}/{dtype}/{form}")
+    for form in ("sgmv", "split", "bgmv"):
+        with pytest.raises(RuntimeError, match="rank"):
+            _apply(form, proj, x, y0.clone(), slots)
+    for name, T in (("qkv", 256), ("o", 256), ("gate_up", 256), ("down", 256), ("o", 1500)):
+        true_ranks = [rank, 8, rank - 8, rank, 16, 0, rank, rank - 4]
+        clean = _make(name, len(true_ranks), rank, dtype, seed=27 + rank, true_ranks=true_ranks)
+        a_nan, b_nan = [t.clone() for t in clean.a], [t.clone() for t in clean.b]
+        for sl, r in enumerate(true_ranks):
+            for t in a_nan:
+                t[sl, r:] = float("nan")
+            for t in b_nan:
+                t[sl, :, r:] = float("nan")
+        x, y0 = synthetic.make_activations(T, clean.k, sum(clean.widths), dtype, seed=29, device="cuda")
+        slots = torch.randint(-1, len(true_ranks), (T,), generator=g, dtype=torch.int32).cuda()
+        exact, mag = _exact(clean, x, y0, slots)
+        eff = torch.tensor(true_ranks, dtype=torch.int32, device="cuda")
+        forms = ["auto", "mfma"] + (["slot"] if name != "qkv" else [])
+        for form in forms:
+            # without the rank vector (zero padding inside the buffers' rank) and with it (NaN there)
+            _check(_apply(form, clean, x, y0.clone(), slots), y0, exact, mag, slots, f"rank{rank}/{name}/T{T}/{form}")
+            y = y0.clone()
+            blocks = list(y.split(clean.widths, dim=-1))
+            _backend(form).add_lora(blocks, x, a_nan, b_nan, indices=slots, metadata=_metadata(slots), scaling=1.0,
+                                    y_packed=y if len(blocks) > 1 else None, effective_rank=eff)
+            assert torch.isfinite(y.float()).all()
+            _check(y, y0, exact, mag, slots, f"rank{rank}/{name}/T{T}/{form}/masked")
+
+
+@pytest.mark.parametrize("rank", [1, 3, 4, 12, 72, 128])
+def test_ranks_the_vector_kernels_do_not_take_go_through_the_token_kernel(rank):
+    """Ranks that are not a multiple of eight (rows of B then do not start on 16-byte boundaries) or
+    lie above 64: AUTO takes the one-workgroup-per-token kernel, with the oracle's result."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    shapes = {"p": (256, [64, 136, 8])}
+    proj = synthetic.make_projection("p", 5, rank, torch.bfloat16, seed=37 + rank, device="cuda", shapes=shapes)
+    x, y0 = synthetic.make_activations(60, 256, 208, torch.bfloat16, seed=39, device="cuda")
+    g = torch.Generator().manual_seed(rank)
+    slots = torch.randint(-1, 5, (60,), generator=g, dtype=torch.int32).cuda()
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(_apply("auto", proj, x, y0.clone(), slots), y0, exact, mag, slots, f"rank{rank}/auto")
+
+
 @pytest.mark.parametrize("staged", ["1", "0"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rank", [8, 16, 32, 64])
