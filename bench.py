@@ -72,7 +72,7 @@ def algorithmic_flops(k: int, widths: list[int], t_lora: int, rank: int, token_r
     return 2 * (t_lora * rank if token_rank_sum is None else token_rank_sum) * (len(widths) * k + sum(widths))
 
 
-def build_workload(name: str, device: str, rank: int | None = None, sequences: int = 0):
+def build_workload(name: str, device: str, rank: int | None = None, sequences: int = 0, slot_ids: int = 0):
     """Per-layer (projection weights, x, y) for the distinct layers of the workload and the
     batch's slot vector.  Layers beyond the distinct ones reuse buffers round-robin (the distinct
     set alone exceeds the 256 MB last-level cache)."""
@@ -82,6 +82,7 @@ def build_workload(name: str, device: str, rank: int | None = None, sequences: i
 
     spec = WORKLOADS[name]
     rank = rank or spec["rank"]
+    num_slots = max(slot_ids, spec["slots"]) if name == "decode" else spec["slots"]  # decode: buffers with more slot ids than adapters in use
     if name == "decode":
         slots = synthetic.decode_slots(256, spec["slots"], seed=7)
         ranks = None
@@ -96,7 +97,7 @@ def build_workload(name: str, device: str, rank: int | None = None, sequences: i
     for layer in range(spec["distinct_layers"]):
         entry = {}
         for j, proj_name in enumerate(ORDER):
-            proj = synthetic.make_projection(proj_name, spec["slots"], rank, torch.bfloat16,
+            proj = synthetic.make_projection(proj_name, num_slots, rank, torch.bfloat16,
                                              seed=1000 + 16 * layer + j, device=device, true_ranks=ranks)
             x, y = synthetic.make_activations(num_tokens, proj.k, sum(proj.widths), torch.bfloat16,
                                               seed=5000 + 16 * layer + j, device=device)
@@ -308,7 +309,7 @@ def run_backbone(args) -> None:
 
 
 KERNELS = {
-    "decode": "decode_kernel<bf16,16>",
+    "decode": "slot_kernel<bf16,16> (o, gate_up, down) + decode_kernel<bf16,16> (qkv)",
     "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
     "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
 }
@@ -340,14 +341,14 @@ def recorded_traffic(workload: str):
 
 
 def measure_workload(name: str, device: str, form: str, steps: int, warmup: int, *, only=None, rank=0, hot_layers=0, eager=False,
-                     per_projection=True, rank_vector=True, sequences=0) -> tuple[dict, tuple]:
+                     per_projection=True, rank_vector=True, sequences=0, slot_ids=0) -> tuple[dict, tuple]:
     """Time one workload: its step replayed as a captured graph (or eagerly), per-projection steps,
     bytes, flops and the roofline object.  Returns (result, (layers, slots, rank, step))."""
     import torch
 
     spec = WORKLOADS[name]
     rank = rank or spec["rank"]
-    layers, slots, eff = build_workload(name, device, rank, sequences)
+    layers, slots, eff = build_workload(name, device, rank, sequences, slot_ids)
     if not rank_vector:
         eff = None
     if hot_layers > 0:
@@ -396,13 +397,14 @@ def measure_workload(name: str, device: str, form: str, steps: int, warmup: int,
     calls = launches
     launch_bytes = step_bytes / calls
     call_us = ms * 1e3 / calls
-    default_shape = form == "auto" and not only and not hot_layers and rank == spec["rank"] and not sequences
+    default_shape = form == "auto" and not only and not hot_layers and rank == spec["rank"] and not sequences and not slot_ids
     result = {
         "value": round(value, 2),
         "ms_per_step": round(ms, 5),
         "config": {
             "workload": spec["text"] if rank == spec["rank"] else spec["text"] + f" -- run at rank {rank} instead",
             "tokens": num_tokens, "tokens_with_adapter": t_lora, "adapters": spec["slots"], "adapters_in_batch": used,
+            "slot_ids_of_the_buffers": max(slot_ids, spec["slots"]) if name == "decode" else spec["slots"],
             "rank": rank, "layers": NUM_LAYERS, "projections": names, "form": form,
             "launch": "eager" if eager else "graph replay",
             "distinct_layer_buffers": hot_layers or spec["distinct_layers"],
@@ -556,6 +558,9 @@ def main() -> None:
     ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | slot | split | sgmv | fused | token")
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
+    ap.add_argument("--slot-ids", type=int, default=0,
+                    help="decode workload: weight buffers with this many slot ids (the batch still uses 32 adapters): what slot ids "
+                         "nobody uses cost the slot-major grid (MLORA_SLOT_MAX_SLOTS bounds where AUTO takes it)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip what the default run adds after the headline: the prefill, mixed and backbone steps and the floor")
@@ -594,7 +599,7 @@ def main() -> None:
     warmup = args.warmup if not heavy else max(1, min(args.warmup, 3))
     rank = args.rank if args.workload in ("decode", "prefill") else 0
     res, (layers, slots, rank, step) = measure_workload(args.workload, device, args.form, steps, warmup, only=args.only, rank=rank,
-                                                        eager=args.eager)
+                                                        eager=args.eager, slot_ids=args.slot_ids if args.workload == "decode" else 0)
     out = {
         "metric": "multi-LoRA shrink+expand HBM GB/s (% peak); us per decode step, 1 GPU",
         "value": res["value"],
@@ -621,7 +626,7 @@ def main() -> None:
         int(buf[: 4 * (_hip.WORKSPACE_TIMEOUTS_WORD + 1)].view(torch.int32)[_hip.WORKSPACE_TIMEOUTS_WORD].item())
         for buf in step.backend.scratch_buffers())
 
-    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.eager and not args.rank
+    default_run = args.workload == "decode" and args.form == "auto" and not args.only and not args.eager and not args.rank and not args.slot_ids
     if default_run and not args.no_extras:
         # After the headline (outside its timed region): what one launch costs here and what a
         # stream reaches here, and the other configurations of the benchmark, a few replays each.

@@ -86,7 +86,9 @@ typedef struct MloraAddArgs {
   const int32_t* token_to_slot; /* [T] on device */
   const int32_t* plan;    /* workspace filled by mlora_meta_build for this token_to_slot, or NULL
                              (NULL is accepted by MLORA_FORM_TOKEN and makes AUTO choose it).  Read-only
-                             for mlora_add_lora too: calls on any number of streams may share one plan */
+                             for mlora_add_lora too, but for the header word MLORA_PLAN_REJECTED (an
+                             atomic count): calls on any number of streams may share one plan.  A return
+                             value of 0 does not say that the plan matched the call: see that word */
   int32_t num_tokens;     /* T */
   int32_t k;              /* K, input features */
   int32_t r;              /* rank dimension of the A/B buffers (max_lora_rank) */

@@ -137,6 +137,25 @@ static bool small_batch(const MloraAddArgs* a) {
   return a->num_tokens * width <= limit;
 }
 
+// Where the slot-major grid pays.  Its workgroups request the weights of EVERY slot id, with or
+// without tokens, so what it costs grows with the slot ids nobody uses: measured on decode batches of
+// 4..256 tokens over 32 slot ids (us per call, slot-major / tile-major): gate_up, whose slots weigh
+// 327 KB each, 5.9 / 3.9 at 4 tokens, 5.6 / 5.2 at 64, 6.1 / 6.0 at 128, 6.7 / 6.8 at 256; o (64 KB per
+// slot) 3.5 / 3.4 at 4 tokens, 3.7 / 3.8 at 64, 3.8 / 4.1 at 256; over 8 slot ids it is the faster
+// grid at every batch size and every projection; with 128 slot ids of which 32 are in use it
+// takes 967 us per decode step against 629.  With K shared out between a tile's workgroups (down) it
+// is the faster one throughout (5.2 / 5.6 at 4 tokens, 6.4 / 6.8 at 256).  So: always with K parts;
+// else while all slots together weigh at most 3 MB, or when the batch has four tokens per slot id.
+static bool slot_major_pays(const MloraAddArgs* a) {
+  if (a->num_slots > knobs().slot_max_slots) return false;
+  if (slot_k_parts(a) > 1) return true;
+  double cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+  const double per_slot = 2.0 * a->r * (static_cast<double>(a->num_slices) * a->k + cols);
+  if (a->num_slots * per_slot <= 3.0e6) return true;
+  return a->num_tokens >= 4 * a->num_slots;
+}
+
 namespace {
 
 int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace);
@@ -203,7 +222,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   // the workgroups of a tile itself (down, decode batch, us per call, slot-major / split form:
   // rank 32: 8.1 / 10.6, rank 64: 10.7 / 17.0).
   if ((form == MLORA_FORM_MFMA || form == MLORA_FORM_SPLIT) && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_MFMA &&
-      knobs().force_form != MLORA_FORM_SPLIT && slot_supported(a) && a->num_slots <= knobs().slot_max_slots)
+      knobs().force_form != MLORA_FORM_SPLIT && slot_supported(a) && slot_major_pays(a))
     form = MLORA_FORM_SLOT;
   // long-segment batches in one launch, on request
   if (form == MLORA_FORM_SGMV && a->form == MLORA_FORM_AUTO && knobs().force_form != MLORA_FORM_SGMV && knobs().auto_fused && fused_supported(a))

@@ -35,6 +35,7 @@ int launch_decode(const MloraAddArgs* a, bool include_long);
 // slot.hip: the same small tiles, the grid laid over the slots: weights are requested from the
 // workgroup index alone, before the slot's record has arrived.
 bool slot_supported(const MloraAddArgs* a);
+int slot_k_parts(const MloraAddArgs* a);  // 4 when the workgroups of a tile would share K out, else 1
 int launch_slot(const MloraAddArgs* a, bool trusted_workspace);
 
 // split.hip: the same small tiles, producers and consumers of the intermediate in one launch.

@@ -718,6 +718,8 @@ bool slot_supported(const MloraAddArgs* a) {
   return false;
 }
 
+int slot_k_parts(const MloraAddArgs* a) { return k_parts(a); }
+
 void slot_trace_set(void* buf) {
 #ifdef MLORA_TRACE
   (void)hipMemcpyToSymbol(HIP_SYMBOL(trace_buf), &buf, sizeof(buf));
