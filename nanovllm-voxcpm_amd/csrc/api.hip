@@ -245,8 +245,9 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
       if (form == MLORA_FORM_MFMA) return launch_decode(a, /*include_long=*/true);
       if (form == MLORA_FORM_SLOT) {
         if (!slot_supported(a)) {
-          set_error("mlora_add_lora: the slot-major form needs one or two non-empty slices and K = 1024, or K = 4096 with rank <= 16 or with "
-                    "one slice of at most 4096 columns and an initialised workspace");
+          set_error("mlora_add_lora: the slot-major form needs one or two non-empty slices and K = 1024 (three at an exact rank with column "
+                    "ranges of at most 512 columns), or K = 4096 with rank <= 16 or with one slice of at most 4096 columns and an "
+                    "initialised workspace");
           return MLORA_E_UNSUPPORTED;
         }
         return launch_slot(a, trusted_workspace);

@@ -70,7 +70,7 @@ typedef unsigned long long u64;
 // an adapter's own (requests clamped into the buffers, values masked).
 template <typename T, int R, int KSPW, int KP, bool MASKED, bool GR, int SA, bool EARLY>
 __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const int slot_early, const int early_ok, const int rbuf_arg, const Range sp,
-                                          const int y_col0, const int y_col1, const bool second, const void* __restrict__ xv,
+                                          const int y_col0, const int y_col1, const int y_col2, const int slice, const void* __restrict__ xv,
                                           void* __restrict__ yv_, const int64_t xs, const int64_t ys,
                                           const int num_slots, const float scaling, const int32_t* __restrict__ eff_rank,
                                           const uint32_t check, int32_t* __restrict__ plan_hdr, const Exchange xc, float* __restrict__ s_red,
@@ -232,7 +232,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   MLORA_STAMP(1);
   // (the column offset of the slice inside y comes with the arguments that are not preloaded:
   // selected here, behind the wait for the record, it holds nothing up)
-  const int y_col = second ? y_col1 : y_col0;
+  const int y_col = slice == 0 ? y_col0 : slice == 1 ? y_col1 : y_col2;
 
   int eff = R;
   if constexpr (MASKED) {
@@ -592,12 +592,62 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restr
   if (static_cast<int>(blockIdx.z) < zslots) {
     const int s = blockIdx.z * 8 + blockIdx.x;  // its record exists: the list is rounded up to eight
     const int slot = s < num_slots ? s : num_slots - 1;
-    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), rbuf, sp, y_col0, y_col1, second, xv, yv_,
+    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), rbuf, sp, y_col0, y_col1, 0, int(second), xv, yv_,
                                                 xs, ys, num_slots, scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   } else {
     const int q = zslots * 8 + (blockIdx.z - zslots) * 8 + blockIdx.x;
-    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, rbuf, sp, y_col0, y_col1, second, xv, yv_, xs, ys, num_slots,
+    slot_tile<T, R, KSPW, KP, MASKED, GR, SA, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, rbuf, sp, y_col0, y_col1, 0, int(second), xv, yv_, xs, ys, num_slots,
                                                  scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
+  }
+}
+
+// Three slices (the stacked q | k | v projection): six pointers do not fit the fourteen preloaded
+// dwords, so the second and third slice's travel as 32-bit offsets from the first one's, in units of
+// 16 bytes (the launcher takes this kernel only when they fit), and the widths as 16-bit counts of
+// eight columns.  widths01 = n0 / 8 | n1 / 8 << 16; widths2 = n2 / 8 | ranges of slice 0 << 16 |
+// ranges of slices 0 and 1 << 24; packed = columns per range / 64 | slots << 16.
+template <typename T, int R, bool MASKED>
+__global__ __launch_bounds__(kNW* kWave) void slot_kernel3(const int32_t* __restrict__ recs, const void* __restrict__ a0,
+                                                           const void* __restrict__ b0, int aoff1, int aoff2, int boff1, int boff2,
+                                                           uint32_t widths01, uint32_t widths2, uint32_t packed,
+                                                           const void* __restrict__ xv, void* __restrict__ yv_, int64_t xs, int64_t ys,
+                                                           int y_col0, int y_col1, int y_col2, uint32_t check, float scaling,
+                                                           const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr) {
+  constexpr int RB = (R + 15) / 16;
+  constexpr int HSTRIDE = R + 8;
+  constexpr int kStageRow = 17;
+  constexpr int SB = RB < 2 ? RB : 2;
+  __shared__ __attribute__((aligned(16))) float s_red[kNW * RB * 64 * 4];
+  __shared__ __attribute__((aligned(16))) T s_hi[16 * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) T s_lo[16 * HSTRIDE];
+  __shared__ __attribute__((aligned(16))) i32x4 s_stage[kNW * (1 + SB) * 16 * kStageRow];
+  __shared__ int s_ok;
+  MLORA_STAMP(0);
+
+  const int nt = static_cast<int>(packed & 255u) * 64, num_slots = static_cast<int>(packed >> 16);
+  const int cum1 = static_cast<int>((widths2 >> 16) & 255u), cum2 = static_cast<int>(widths2 >> 24);
+  const int ri = blockIdx.y;
+  const int slice = int(ri >= cum1) + int(ri >= cum2);
+  const int64_t ao = slice == 0 ? 0 : slice == 1 ? aoff1 : aoff2, bo = slice == 0 ? 0 : slice == 1 ? boff1 : boff2;
+  Range sp;
+  sp.a = static_cast<const char*>(a0) + ao * 16;
+  sp.b = static_cast<const char*>(b0) + bo * 16;
+  sp.n = 8 * static_cast<int>(slice == 0 ? widths01 & 0xffffu : slice == 1 ? widths01 >> 16 : widths2 & 0xffffu);
+  sp.y_col = 0;  // (selected inside, late)
+  sp.n0 = (ri - (slice == 0 ? 0 : slice == 1 ? cum1 : cum2)) * nt;
+  sp.n1 = sp.n0 + nt < sp.n ? sp.n0 + nt : sp.n;
+
+  const int zslots = (num_slots + 7) >> 3;
+  const Exchange xc{nullptr, 0, 0};
+  if (static_cast<int>(blockIdx.z) < zslots) {
+    const int s = blockIdx.z * 8 + blockIdx.x;
+    const int slot = s < num_slots ? s : num_slots - 1;
+    slot_tile<T, R, 4, 1, MASKED, false, 1, true>(recs + s * MLORA_SMALL_TILE_WORDS, slot, int(s < num_slots), R, sp, y_col0, y_col1, y_col2, slice, xv,
+                                                  yv_, xs, ys, num_slots, scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
+  } else {
+    const int q = zslots * 8 + (blockIdx.z - zslots) * 8 + blockIdx.x;
+    slot_tile<T, R, 4, 1, MASKED, false, 1, false>(recs + q * MLORA_SMALL_TILE_WORDS, 0, 1, R, sp, y_col0, y_col1, y_col2, slice, xv, yv_, xs, ys,
+                                                   num_slots, scaling, eff_rank, check, plan_hdr, xc, s_red, s_hi, s_lo, s_stage, &s_ok);
   }
 }
 
@@ -608,6 +658,40 @@ struct Launch {
   int widest;
   int spin_ticks, trusted;
 };
+
+// Offsets of slice i's A and B from slice 0's, in units of 16 bytes, when they fit 32 bits.
+bool offsets16(const MloraAddArgs* a, int i, int* ao, int* bo) {
+  const long long da = static_cast<const char*>(a->slices[i].a) - static_cast<const char*>(a->slices[0].a);
+  const long long db = static_cast<const char*>(a->slices[i].b) - static_cast<const char*>(a->slices[0].b);
+  if ((da & 15) || (db & 15)) return false;
+  const long long qa = da / 16, qb = db / 16;
+  if (qa < INT32_MIN || qa > INT32_MAX || qb < INT32_MIN || qb > INT32_MAX) return false;
+  *ao = static_cast<int>(qa);
+  *bo = static_cast<int>(qb);
+  return true;
+}
+
+template <typename T, int R>
+void launch_three(const MloraAddArgs* a, dim3 grid, int nt, int cum1, int cum2) {
+  const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
+  int ao1 = 0, ao2 = 0, bo1 = 0, bo2 = 0;
+  (void)offsets16(a, 1, &ao1, &bo1);
+  (void)offsets16(a, 2, &ao2, &bo2);
+  const uint32_t w01 = static_cast<uint32_t>(a->slices[0].n / 8) | (static_cast<uint32_t>(a->slices[1].n / 8) << 16);
+  const uint32_t w2 = static_cast<uint32_t>(a->slices[2].n / 8) | (static_cast<uint32_t>(cum1) << 16) | (static_cast<uint32_t>(cum2) << 24);
+  const uint32_t packed = static_cast<uint32_t>(nt / 64) | (static_cast<uint32_t>(a->num_slots) << 16);
+  const uint32_t check = static_cast<uint32_t>(MLORA_PLAN_CHECK(a->num_tokens, a->num_slots));
+  if (a->effective_rank)
+    hipLaunchKernelGGL((slot_kernel3<T, R, true>), grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream), a->plan + lay.slotrec_off,
+                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
+                       a->slices[0].y_col, a->slices[1].y_col, a->slices[2].y_col, check, a->scaling, a->effective_rank,
+                       const_cast<int32_t*>(a->plan));
+  else
+    hipLaunchKernelGGL((slot_kernel3<T, R, false>), grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream), a->plan + lay.slotrec_off,
+                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
+                       a->slices[0].y_col, a->slices[1].y_col, a->slices[2].y_col, check, a->scaling, a->effective_rank,
+                       const_cast<int32_t*>(a->plan));
+}
 
 template <typename T, int R, int KSPW, int KP, bool MASKED, bool GR, int SA>
 void launch_spans(const Launch& l) {
@@ -666,6 +750,27 @@ bool launch_rank(const Launch& l, int rank, int kspw, int kp) {
   return false;
 }
 
+// Columns per range: as in the tile-major launch, sized for 150-250 workgroups; at most 1024 (two
+// 64-column spans per wavefront, all loads in registers).
+int range_columns(const MloraAddArgs* a) {
+  long long cols = 0;
+  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
+  const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
+  const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
+  const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
+  int nt = static_cast<int>(cols * tiles / 160);
+  if (nt > 1024) nt = 1024;
+  if (nt < 128) nt = 128;
+  nt = (nt + 63) & ~63;
+  while (nt < 1024) {
+    int total = 0;
+    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
+    if (total <= 32) break;
+    nt *= 2;
+  }
+  return nt > 1024 ? 1024 : nt;
+}
+
 int kspw_of(const MloraAddArgs* a) { return a->k % (32 * kNW) == 0 ? a->k / (32 * kNW) : 0; }
 
 // Diagnostic knobs, read from the environment once per process.
@@ -701,10 +806,11 @@ int k_parts(const MloraAddArgs* a) {
 
 // K = 1024 at every rank; K = 4096 at every rank with the K parts of a tile shared out between its
 // workgroups, else up to rank 16 (what fits the register file as one batch of loads); one or two
-// slices (what fits the preloaded arguments); 16-bit elements.
+// slices with their pointers as arguments, three (K = 1024) with the later two's as offsets from
+// the first one's; 16-bit elements.
 bool slot_supported(const MloraAddArgs* a) {
   if (a->dtype != MLORA_DTYPE_BF16 && a->dtype != MLORA_DTYPE_F16) return false;
-  if (a->num_slices < 1 || a->num_slices > 2 || !a->plan) return false;
+  if (a->num_slices < 1 || a->num_slices > 3 || !a->plan) return false;
   long long cols = 0;
   for (int i = 0; i < a->num_slices; ++i) {
     if (a->slices[i].n <= 0) return false;
@@ -713,6 +819,15 @@ bool slot_supported(const MloraAddArgs* a) {
   if (cols > 200 * 1024) return false;  // at most 255 column ranges of up to 1024 columns
   if (!padded_rank(a->r)) return false;
   const int kspw = kspw_of(a);
+  if (a->num_slices == 3) {
+    // q | k | v: K = 1024, an exact rank, offsets that fit 32 bits, widths that fit 16-bit counts of
+    // eight columns, and column ranges of at most 512 columns (one span per wavefront)
+    int ao, bo;
+    if (kspw != 4 || !exact_rank(a->r) || !offsets16(a, 1, &ao, &bo) || !offsets16(a, 2, &ao, &bo)) return false;
+    for (int i = 0; i < 3; ++i)
+      if (a->slices[i].n % 8 || a->slices[i].n / 8 > 0xffff) return false;
+    return range_columns(a) <= kNW * 64;
+  }
   if (kspw == 4) return true;
   if (kspw == 16) return a->r <= 16 || k_parts(a) == 4;
   return false;
@@ -728,36 +843,14 @@ void slot_trace_set(void* buf) {
 #endif
 }
 
-namespace {
-// Columns per range: as in the tile-major launch, sized for 150-250 workgroups; at most 1024 (two
-// 64-column spans per wavefront, all loads in registers).
-int range_columns(const MloraAddArgs* a) {
-  long long cols = 0;
-  for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
-  const int segs = a->num_slots < a->num_tokens ? a->num_slots : a->num_tokens;
-  const int by_tokens = (a->num_tokens + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL;
-  const long long tiles = segs > by_tokens ? segs : by_tokens;  // about the number of tiles in use
-  int nt = static_cast<int>(cols * tiles / 160);
-  if (nt > 1024) nt = 1024;
-  if (nt < 128) nt = 128;
-  nt = (nt + 63) & ~63;
-  while (nt < 1024) {
-    int total = 0;
-    for (int i = 0; i < a->num_slices; ++i) total += (a->slices[i].n + nt - 1) / nt;
-    if (total <= 32) break;
-    nt *= 2;
-  }
-  return nt > 1024 ? 1024 : nt;
-}
-}  // namespace
-
 int launch_slot(const MloraAddArgs* a, bool trusted_workspace) {
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
   const int kp = k_parts(a);
   // with K parts the tile's workgroups are its K parts and its column ranges alike
   const int nt = kp > 1 ? ((a->slices[0].n + kp - 1) / kp + 63) & ~63 : range_columns(a);
   const int ranges0 = kp > 1 ? kp : (a->slices[0].n + nt - 1) / nt;
-  const int total = ranges0 + (a->num_slices > 1 ? (a->slices[1].n + nt - 1) / nt : 0);
+  const int ranges1 = a->num_slices > 1 ? (a->slices[1].n + nt - 1) / nt : 0;
+  const int total = ranges0 + ranges1 + (a->num_slices > 2 ? (a->slices[2].n + nt - 1) / nt : 0);
   if (total > 255) {
     set_error("mlora_add_lora(slot-major): %d column ranges exceed 255", total);
     return MLORA_E_UNSUPPORTED;
@@ -773,6 +866,22 @@ int launch_slot(const MloraAddArgs* a, bool trusted_workspace) {
   l.spin_ticks = slot_knobs().spin_ticks;
   l.trusted = trusted_workspace ? 1 : 0;
   l.grid = dim3(8, static_cast<unsigned>(total), static_cast<unsigned>((lay.cap_slotrec + lay.cap_over) / 8));
+  if (a->num_slices == 3) {
+    switch (a->r) {
+#define MLORA_THREE(R)                                                                                      \
+  case R:                                                                                                   \
+    if (a->dtype == MLORA_DTYPE_BF16) launch_three<__bf16, R>(a, l.grid, nt, ranges0, ranges0 + ranges1);   \
+    else launch_three<_Float16, R>(a, l.grid, nt, ranges0, ranges0 + ranges1);                              \
+    break;
+      MLORA_THREE(8)
+      MLORA_THREE(16)
+      MLORA_THREE(32)
+      MLORA_THREE(64)
+#undef MLORA_THREE
+      default: set_error("mlora_add_lora(slot-major): unsupported rank %d for three slices", a->r); return MLORA_E_UNSUPPORTED;
+    }
+    return check_launch("mlora_add_lora(small tiles, one workgroup per slot and column range, three slices)");
+  }
   const int kspw = kspw_of(a) / kp;
   const bool ok = a->dtype == MLORA_DTYPE_BF16 ? launch_rank<__bf16>(l, a->r, kspw, kp) : launch_rank<_Float16>(l, a->r, kspw, kp);
   if (!ok) {

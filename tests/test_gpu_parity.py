@@ -160,7 +160,8 @@ def _slot_form_batches(T, L, seed):
 
 
 @pytest.mark.parametrize("name,rank,T,L", [("o", 16, 256, 32), ("gate_up", 16, 256, 32), ("down", 16, 256, 32), ("o", 32, 64, 32),
-                                           ("gate_up", 64, 100, 5), ("o", 8, 37, 13), ("down", 8, 300, 9), ("gate_up", 32, 19, 64)])
+                                           ("gate_up", 64, 100, 5), ("o", 8, 37, 13), ("down", 8, 300, 9), ("gate_up", 32, 19, 64),
+                                           ("qkv", 16, 256, 32), ("qkv", 32, 64, 32), ("qkv", 8, 37, 13), ("qkv", 64, 100, 5)])
 def test_slot_major_grid_gives_the_bits_of_the_tile_major_grid(name, rank, T, L, monkeypatch):
     """The slot-major form requests a slot's weights before its record has arrived; what it computes
     is the small-tile form's arithmetic in the same order, so its results are the oracle's and,

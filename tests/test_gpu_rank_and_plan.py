@@ -42,8 +42,6 @@ def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, 
 
     if form == "split" and tokens > 256:
         pytest.skip("the split form takes decode-sized batches only (its exchange area holds ~128 rank-64 partial tiles)")
-    if form == "slot" and name in ("qkv", "down"):
-        pytest.skip("the slot-major form takes one or two slices, and K = 4096 up to rank 16 only")
     print(f"rank masking {name} T={tokens} form={form}", flush=True)
     ranks = [8, 12, 16, 32, 40, 64, 0, 24]
     clean = _make(name, len(ranks), 64, torch.bfloat16, seed=800, true_ranks=ranks)
@@ -65,8 +63,14 @@ def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, 
     backend = _backend(form)
     y = y0.clone()
     blocks = list(y.split(clean.widths, dim=-1))
-    backend.add_lora(blocks, x, a_nan, b_nan, indices=slots, metadata=_metadata(slots), scaling=1.0,
-                     y_packed=y if len(blocks) > 1 else None, effective_rank=eff)
+    try:
+        backend.add_lora(blocks, x, a_nan, b_nan, indices=slots, metadata=_metadata(slots), scaling=1.0,
+                         y_packed=y if len(blocks) > 1 else None, effective_rank=eff)
+    except RuntimeError as e:
+        if form == "slot" and "slot-major form needs" in str(e):
+            pytest.skip("the slot-major form refuses this shape (column ranges too wide for three slices, or K = 4096 at a rank and "
+                        "width its K parts do not take), as AUTO knows: " + str(e))
+        raise
     assert torch.isfinite(y.float()).all(), "a value beyond a slot's rank reached the output"
     _check(y, y0, exact, mag, slots, f"masked/{name}/T{tokens}/{form}")
     # the empty slot (rank 0) is a no-op even though its buffers are all NaN
