@@ -226,8 +226,16 @@ size_t mlora_plan_workspace_bytes(int32_t num_tokens, int32_t max_slots);
  * all sixteen name rows of the tile itself), then padding.
  * A big tile is four words {slot, first position in sorted_idx, token count, 0}; behind the
  * big-tile records lies one list of MLORA_TILE_BIG token indices per big tile (its tokens in
- * order, 0 past the count: a valid row to read), at a place that follows from the tile's number
- * alone: a workgroup requests it together with the record. */
+ * order, 0 past the count: a valid row to read), at a place that follows from the tile's place
+ * alone: a workgroup requests it together with the record.  The list of big tiles (capacity: with
+ * most = num_tokens / 64 + min(max_slots, num_tokens) and root the smallest integer with
+ * 8 root^2 >= most, (most + 8 (root + 2) + 31) & ~31) is cut into eight equal blocks, one per
+ * XCD (workgroup (x, ., z) of a launch takes place x * capacity / 8 + z).  The big tiles of a plan are
+ * sorted by slot; runs of consecutive tiles go to the blocks in turn (tile t of run i = t / run at
+ * (i % 8) * capacity / 8 + (i / 8) * run + t % run), where run = ceil(n / (8 k)) for n tiles and
+ * k = ceil(n / (8 * floor(n / slots that have big tiles))): runs about as long as a slot's segment
+ * has tiles, so that a slot meets few XCDs and its weights are fetched into few L2s, and of one tile
+ * when the slots have one tile each.  Places without a tile hold {-1, 0, 0, 0}. */
 #define MLORA_SMALL_TILE_WORDS 32
 #define MLORA_SMALL_TILE_ROWS 4 /* word index of the first token index inside a record */
 #define MLORA_BIG_TILE_WORDS 4

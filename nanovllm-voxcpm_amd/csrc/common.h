@@ -181,6 +181,35 @@ struct PlanLayout {
 
 __host__ __device__ inline int round_up4(int v) { return (v + 3) & ~3; }
 
+// Where the 64-token tiles lie in their list.  The list is cut into eight equal blocks, one per
+// XCD: workgroup (x, ., z) of a launch takes place x * (capacity / 8) + z.  The tiles are sorted by
+// slot; runs of consecutive tiles go to the blocks in turn (run i to block i % 8, behind the runs
+// the block already holds).  With long runs the tiles of a slot meet few XCDs and its weights are
+// fetched into few L2s; with runs of one tile the XCDs take the tiles in turn.  Workgroups are
+// dispatched layer by layer (z), every XCD's z-th tile together, so a layer costs what its most
+// expensive tile costs: runs may be as long as the slots' segments are (then a layer holds tiles
+// of the same kind, mostly full ones), and no longer than an eighth of the list.
+//   run length: the tiles split into 8 k runs, k the smallest for which a run is no longer than
+//   the average number of tiles of a slot that has any.
+__host__ __device__ inline int big_tile_run(int n_big, int slots_with_tiles) {
+  if (n_big <= 0) return 1;
+  const int avg = n_big / (slots_with_tiles > 0 ? slots_with_tiles : 1);  // >= 1
+  const int k = (n_big + 8 * avg - 1) / (8 * avg);
+  return (n_big + 8 * k - 1) / (8 * k);
+}
+__host__ __device__ inline int big_tile_place(int t, int run, int cap_big) {
+  const int i = t / run;
+  return (i & 7) * (cap_big >> 3) + (i >> 3) * run + t % run;
+}
+// Places for at most `most` tiles: a block holds ceil(runs / 8) runs, less than most / 8 + run
+// places, and a run is at most ceil(most / (8 k)) with k runs a block: most / 8 + sqrt(most / 8) + 1
+// places bound both; a multiple of 32.
+__host__ __device__ inline int big_tile_capacity(int most) {
+  int root = 1;
+  while (root * root * 8 < most) ++root;
+  return (most + 8 * (root + 2) + 31) & ~31;
+}
+
 __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   PlanLayout p;
   const int segs = L < T ? L : T;
@@ -192,7 +221,9 @@ __host__ __device__ inline PlanLayout plan_layout(int T, int L) {
   // tile per XCD), and every record such a grid may touch has to exist
   p.cap_small = ((T + MLORA_TILE_SMALL - 1) / MLORA_TILE_SMALL + segs + 7) & ~7;
   p.big_off = p.small_off + MLORA_SMALL_TILE_WORDS * p.cap_small;
-  p.cap_big = (T / MLORA_TILE_BIG + segs + 31) & ~31;  // groups of up to four tiles, eight groups abreast
+  // groups of up to four tiles, eight blocks abreast (one per XCD), each block with room for an
+  // eighth of the tiles and a run of them (big_tile_place)
+  p.cap_big = big_tile_capacity(T / MLORA_TILE_BIG + segs);
   p.bigrows_off = p.big_off + MLORA_BIG_TILE_WORDS * p.cap_big;  // (a multiple of 32 words again)
   // the small tiles once more, by slot: one record per slot id, then one per further tile (a
   // further tile has sixteen tokens of its slot in front of it, so T / 16 bounds their number)

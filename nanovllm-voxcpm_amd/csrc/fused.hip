@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   T* const s_h = reinterpret_cast<T*>(s_raw);
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const int unit = tile_position(big_units);  // blockIdx.x is the XCD; a block of the list of units is G positions of the XCD's block of tiles
   const int c = blockIdx.y, W = gridDim.y;
   const bool is_big = unit < big_units;
   const int sidx = is_big ? 0 : unit - big_units;
@@ -122,11 +122,11 @@ __global__ __launch_bounds__(kFusedThreads, 2) void sgmv_fused_kernel(
   uint32_t* const ustate = ws + kWsTileOff / 4;
   const uint32_t tag = ustate[0] + 1u;
   const uint32_t arrivals0 = ustate[1], gen_check = ustate[2];
-  const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
+  const int n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
   int slot[G], start[G], m[G], any = 0;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    const bool have = is_big ? unit * G + g < n_big : (g == 0 && sidx < n_short);
+    const bool have = is_big ? true : (g == 0 && sidx < n_short);  // (places of the list of 64-token tiles that hold none carry count 0)
     slot[g] = is_big ? big[g][0] : small[0];
     start[g] = is_big ? big[g][1] : small[2];
     m[g] = is_big ? big[g][2] : small[1];

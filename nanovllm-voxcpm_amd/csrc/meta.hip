@@ -60,6 +60,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   int* ts_big = ts_long + NB + 1;      // [NB + 1]: first big tile of a long segment
   int* ts_over = ts_big + NB + 1;      // [NB + 1]: first of the small tiles behind a slot's first one
   __shared__ int s_bad, s_max;
+  __shared__ int s_nlong;              // slots with a long segment
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int T = p.T, L = p.L;
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   // Wave 0: exclusive scans over the buckets.
   const int b0 = p.no_lora_bucket ? 0 : 1;  // first bucket of the compact arrays
   if (wave == 0) {
-    int run0 = 0, run1 = 0, run2 = 0, run3 = 0, run4 = 0, run5 = 0, mx = 0;
+    int run0 = 0, run1 = 0, run2 = 0, run3 = 0, run4 = 0, run5 = 0, mx = 0, nlong = 0;
     for (int base = 0; base < NB; base += kWave) {
       int b = base + lane;
       int c_all = b < NB ? total[b] : 0;
@@ -152,6 +153,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       run3 += __shfl(i3, kWave - 1, kWave);
       run4 += __shfl(i4, kWave - 1, kWave);
       run5 += __shfl(i5, kWave - 1, kWave);
+      nlong += __popcll(__ballot(b < NB && !is_short));
       int m = c;
 #pragma unroll
       for (int o = 32; o >= 1; o >>= 1) { int n = __shfl_xor(m, o, kWave); m = n > m ? n : m; }
@@ -160,6 +162,7 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
     if (lane == 0) {
       off[NB] = run0; cidx[NB] = run1; ts_short[NB] = run2; ts_long[NB] = run3; ts_big[NB] = run4; ts_over[NB] = run5;
       s_max = mx;
+      s_nlong = nlong;
     }
   }
   __syncthreads();
@@ -227,8 +230,14 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
   // Tile lists of the plan.  A small-tile record starts with its header and zeroed row entries;
   // the scatter below fills all sixteen (the tile's tokens, repeated cyclically past its count).
   i32x4* small = p.plan ? reinterpret_cast<i32x4*>(p.plan + lay.small_off) : nullptr;
+  // place of big tile q (in slot order) in the list: runs of `run` consecutive tiles go to the
+  // blocks (XCDs) in turn
+  const int run = big_tile_run(n_big, s_nlong);
+  auto place_big = [&](int q) { return big_tile_place(q, run, lay.cap_big); };
   if (p.plan) {
     i32x4* big = reinterpret_cast<i32x4*>(p.plan + lay.big_off);
+    for (int q = tid; q < lay.cap_big; q += kMetaThreads) big[q] = i32x4{-1, 0, 0, 0};
+    __syncthreads();  // (a place is cleared by one thread and may be filled by another)
     for (int q = tid; q < n_short + n_long; q += kMetaThreads) {
       const bool is_short = q < n_short;
       const int* ts = is_short ? ts_short : ts_long;
@@ -245,11 +254,12 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
       int b = find_bucket(ts_big, NB, q);
       int j = q - ts_big[b], c = total[b];
       int left = c - j * MLORA_TILE_BIG;
-      big[q] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
+      big[place_big(q)] = i32x4{b - 1, off[b] + j * MLORA_TILE_BIG, left < MLORA_TILE_BIG ? left : MLORA_TILE_BIG, 0};
     }
     // row lists of the big tiles: cleared, the scatter below enters the tokens
     i32x4* rows = reinterpret_cast<i32x4*>(p.plan + lay.bigrows_off);
-    for (int q = tid; q < n_big * (MLORA_TILE_BIG / 4); q += kMetaThreads) rows[q] = i32x4{0, 0, 0, 0};
+    for (int q = tid; q < n_big * (MLORA_TILE_BIG / 4); q += kMetaThreads)
+      rows[place_big(q / (MLORA_TILE_BIG / 4)) * (MLORA_TILE_BIG / 4) + q % (MLORA_TILE_BIG / 4)] = i32x4{0, 0, 0, 0};
     // the small tiles once more, by slot: the record of every slot id (count 0 for a slot without
     // tokens and for the ids that round the list up to a multiple of eight), then the further
     // tiles of every slot, then count 0 up to the capacity
@@ -316,7 +326,8 @@ __global__ __launch_bounds__(kMetaThreads) void meta_kernel(MetaParams p) {
           // its entry in the row list of the segment's 64-token tile (entries past a tile's count
           // stay 0, a valid row: only the last tile of a segment has any, and repeating its tokens
           // there as in the small records is a loop of up to 64 stores in one lane)
-          if (c >= MLORA_SEGMENT_THRESHOLD) p.plan[lay.bigrows_off + (ts_big[key] + r / MLORA_TILE_BIG) * MLORA_TILE_BIG + r % MLORA_TILE_BIG] = t;
+          if (c >= MLORA_SEGMENT_THRESHOLD)
+            p.plan[lay.bigrows_off + place_big(ts_big[key] + r / MLORA_TILE_BIG) * MLORA_TILE_BIG + r % MLORA_TILE_BIG] = t;
         }
         if (p.sorted_idx) p.sorted_idx[n_neg + off[key] + r] = t;
       } else if (p.sorted_idx) {

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kShrinkWaves* kWave, 2) void sgmv_shrink_kernel(con
   // all_slices: the workgroup walks every slice of the projection with the x rows it holds in
   // registers (its K part is a single batch then), instead of one workgroup per slice
   const int slice0 = all_slices ? 0 : blockIdx.y / ksplit, kpart = all_slices ? blockIdx.y : blockIdx.y % ksplit;
-  const int tile = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const int tile = tile_position(big_cap);  // blockIdx.x is the XCD
   MLORA_STAMP(0);  // first instruction
   const int row = tile_row(plan, bigrows_off, small_off, big_cap, tile, (threadIdx.x / kWave) * 16 + (threadIdx.x & 15));
   const TileRef tr = fetch_tile(plan, big_off, small_off, big_cap, tile, T_, num_slots);
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
   const int lr = lane & 15, lg = lane >> 4;
   // A workgroup takes G consecutive 64-token tiles (consecutive tiles mostly belong to one slot,
   // whose B rows then stay in registers across them), or, past `big_units`, one short segment.
-  const int unit = blockIdx.z * 8 + blockIdx.x;  // blockIdx.x is the XCD
+  const int unit = tile_position(big_units);  // blockIdx.x is the XCD; a block of the list of units is G positions of the XCD's block of tiles
   MLORA_STAMP(8);  // expand: first instruction
   const bool is_big = unit < big_units;
   const int sidx = is_big ? 0 : unit - big_units;
@@ -118,11 +118,11 @@ __global__ __launch_bounds__(kExpandWaves* kWave, 2) void sgmv_expand_kernel(con
     }
   }
   const ExpandSplit sp = splits.split[blockIdx.y];
-  const int n_big = hdr2[MLORA_PLAN_TILES_LONG_BIG - 8], n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
+  const int n_short = hdr1[MLORA_PLAN_TILES_SHORT - 4];
   int slot[G], start[G], m[G], any = 0;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    const bool have = is_big ? unit * G + g < n_big : (g == 0 && sidx < n_short);
+    const bool have = is_big ? true : (g == 0 && sidx < n_short);  // (places of the list of 64-token tiles that hold none carry count 0)
     slot[g] = is_big ? big[g][0] : small[0];
     start[g] = is_big ? big[g][1] : small[2];
     m[g] = is_big ? big[g][2] : small[1];

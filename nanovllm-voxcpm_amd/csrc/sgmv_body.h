@@ -38,6 +38,14 @@ struct TileRef {
   int plan_ok;  // the plan's header is that of this call's batch shape
 };
 
+// Position in the tile lists of workgroup (x, ., z) of a grid (8, ., big_cap / 8 + short segments / 8):
+// the first big_cap / 8 layers take the 64-token tiles, XCD x its own block of the list; the layers
+// behind them take the short segments, eight abreast.  Positions from big_cap on are short segments.
+__device__ __forceinline__ int tile_position(int big_cap) {
+  const int blk = big_cap >> 3, z = blockIdx.z, x = blockIdx.x;
+  return z < blk ? x * blk + z : big_cap + (z - blk) * 8 + x;
+}
+
 __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, int big_off, int small_off, int big_cap, int tile,
                                               int T_, int num_slots) {
   // both candidate records and the header are requested together (every address is in bounds
@@ -53,10 +61,10 @@ __device__ __forceinline__ TileRef fetch_tile(const int32_t* __restrict__ plan, 
   t.slot = is_big ? big[0] : small[0];
   t.start = is_big ? big[1] : small[2];
   t.m = is_big ? big[2] : small[1];
-  const int limit = is_big ? hdr2[MLORA_PLAN_TILES_LONG_BIG - 8] : hdr1[MLORA_PLAN_TILES_SHORT - 4];
-  const int index = is_big ? tile : sidx;
+  // the position holds a tile of this plan: places of the list of 64-token tiles that hold none carry count 0
+  const bool present = is_big ? true : sidx < hdr1[MLORA_PLAN_TILES_SHORT - 4];
   t.ok = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
-         int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(index < limit) & int(t.m > 0) & int(t.slot >= 0) &
+         int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots) & int(present) & int(t.m > 0) & int(t.slot >= 0) &
          int(t.slot < num_slots);
   t.plan_ok = int(hdr0[MLORA_PLAN_MAGIC] == MLORA_PLAN_MAGIC_VALUE) & int(hdr0[MLORA_PLAN_NUM_TOKENS] == T_) &
               int(hdr0[MLORA_PLAN_MAX_SLOTS] == num_slots);

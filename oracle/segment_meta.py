@@ -103,6 +103,37 @@ def graph_layout(token_to_slot: list[int] | None, no_lora_flag: bool, max_rows: 
                 num_tokens_per_slot=counts, slot_start_offsets=offsets)
 
 
+def big_tile_capacity(num_tokens: int, max_slots: int, big: int = 64) -> int:
+    """Places in the plan's list of big tiles: at most ``most`` = num_tokens // big + min(max_slots,
+    num_tokens) tiles exist; an eighth of them, the smallest ``root`` with 8 root^2 >= most, and two
+    more fit every one of the eight blocks; rounded up to a multiple of 32."""
+    most = num_tokens // big + min(max_slots, num_tokens)
+    root = 1
+    while 8 * root * root < most:
+        root += 1
+    return (most + 8 * (root + 2) + 31) & ~31
+
+
+def big_tile_places(long_big: list[tuple[int, int, int]], num_tokens: int, max_slots: int, big: int = 64) -> list[int]:
+    """Places of the big tiles (``long_big`` of plan_tiles, in slot order) in the plan's list of big
+    tiles.  The list is cut into eight equal blocks, one per XCD.  The tiles are cut into runs of
+    consecutive tiles, and run i goes to block i % 8, behind the runs the block already holds.
+    Run length: the tiles split into 8 k runs, k the smallest for which a run is no longer than
+    the average number of tiles (rounded down) of a slot that has any."""
+    n = len(long_big)
+    if n == 0:
+        return []
+    blk = big_tile_capacity(num_tokens, max_slots, big) // 8
+    avg = n // len({slot for slot, _, _ in long_big})
+    k = -(-n // (8 * avg))
+    run = -(-n // (8 * k))
+    places = []
+    for t in range(n):
+        i = t // run
+        places.append((i % 8) * blk + (i // 8) * run + t % run)
+    return places
+
+
 def plan_tiles(token_to_slot: list[int], max_slots: int, threshold: int = 16, small: int = 16, big: int = 64):
     """Work lists the apply kernels walk, derived from the engine layout: for every slot in
     ascending order its segment is cut into tiles (slot, first position in sorted_idx, count).

@@ -147,7 +147,9 @@ def test_arguments_are_rejected_before_any_launch():
         r4 = lambda v: (v + 3) & ~3  # noqa: E731
         small_off = (16 + r4(t) + r4(l + 1) + r4(l + 2) + 31) & ~31
         cap_small = ((t + 15) // 16 + min(l, t) + 7) & ~7
-        cap_big = (t // 64 + min(l, t) + 31) & ~31
+        most = t // 64 + min(l, t)  # big tiles at most; an eighth of them + about the root of that + 2 fit each of eight blocks
+        root = next(v for v in range(1, most + 2) if 8 * v * v >= most)
+        cap_big = (most + 8 * (root + 2) + 31) & ~31
         return small_off + 32 * cap_small + (4 + 64) * cap_big + 32 * ((l + 7) & ~7) + 32 * ((t // 16 + 7) & ~7)
     for t, l in ((256, 32), (1, 1), (8192, 128), (20000, 1024), (15, 600)):
         assert lib.mlora_plan_workspace_bytes(t, l) == 4 * words(t, l), (t, l)

@@ -1057,7 +1057,7 @@ def test_metadata_bit_exact_random(T, L, p_neg):
     small_off = (offsets_off + r4(L + 2) + 31) & ~31
     cap_small = ((T + 15) // 16 + min(L, T) + 7) & ~7
     big_off = small_off + _hip.SMALL_TILE_WORDS * cap_small
-    cap_big = (T // 64 + min(L, T) + 31) & ~31
+    cap_big = meta_oracle.big_tile_capacity(T, L)
     bigrows_off = big_off + 4 * cap_big
     slotrec_off = bigrows_off + 64 * cap_big
     cap_slotrec = (L + 7) & ~7
@@ -1101,8 +1101,11 @@ def test_metadata_bit_exact_random(T, L, p_neg):
         assert rec[:4] == [slot, count, start, 0]
         own = s[start : start + count]
         assert rec[4:20] == [own[j % count] for j in range(16)] and rec[20:] == [0] * 12  # cyclic repeats past the count
-    assert [tuple(ws[big_off + 4 * i : big_off + 4 * i + 3]) for i in range(len(long_big))] == long_big
-    for q, (slot, start, count) in enumerate(long_big):  # the tile's tokens, then zeros (a valid row to read)
+    place = meta_oracle.big_tile_places(long_big, T, L)
+    assert len(set(place)) == len(place) and all(0 <= q < cap_big for q in place)
+    assert [tuple(ws[big_off + 4 * q : big_off + 4 * q + 3]) for q in place] == long_big
+    assert all(tuple(ws[big_off + 4 * q : big_off + 4 * q + 3]) == (-1, 0, 0) for q in set(range(cap_big)) - set(place))  # places without a tile
+    for q, (slot, start, count) in zip(place, long_big):  # the tile's tokens, then zeros (a valid row to read)
         own = s[start : start + count]
         assert ws[bigrows_off + 64 * q : bigrows_off + 64 * (q + 1)] == own + [0] * (64 - count)
 

@@ -260,3 +260,53 @@ def test_layouts_agree_with_brute_force_sort(seed):
         assert cnt == min(16, slots.count(sl))
         assert all(slots[s[p]] == sl for p in range(st, st + cnt))
     assert all(slots[s[p]] == sl for (sl, st, cnt) in further for p in range(st, st + cnt))
+
+
+def test_big_tiles_are_laid_out_in_runs_over_one_block_per_xcd():
+    """Properties of the placement that do not restate its rule: no two tiles share a place, all
+    places lie in the list, every block (an eighth of the list) is filled from its start, the
+    blocks' tile counts differ by at most one run, a block holds whole runs of consecutive tiles
+    (the last run of the batch aside), a batch of many one-tile slots is dealt out tile by tile
+    (every layer of eight places holds eight consecutive tiles), and a batch of few slots with many
+    tiles each lets a slot meet at most two blocks more than its share of an eighth of the tiles."""
+    rng = np.random.default_rng(77)
+
+    def check(slots, T, L):
+        _, _, long_big = meta_oracle.plan_tiles(slots, L)
+        n = len(long_big)
+        cap = meta_oracle.big_tile_capacity(T, L)
+        assert cap % 32 == 0
+        place = meta_oracle.big_tile_places(long_big, T, L)
+        assert len(place) == n
+        if n == 0:
+            return None
+        assert len(set(place)) == n and min(place) >= 0 and max(place) < cap
+        blk = cap // 8
+        by_block = {}
+        for t, q in enumerate(place):
+            by_block.setdefault(q // blk, {})[q % blk] = t
+        counts = []
+        for x, members in by_block.items():
+            assert sorted(members) == list(range(len(members)))  # filled from its start
+            counts.append(len(members))
+        tiles = [[members[j] for j in range(len(members))] for members in by_block.values()]
+        runs = [len(r) for ts in tiles for r in np.split(np.array(ts), np.nonzero(np.diff(ts) != 1)[0] + 1)]
+        run = max(runs)
+        assert sum(1 for r in runs if r != run) <= 1  # whole runs, but for the last of the batch
+        assert max(counts) - (min(counts) if len(counts) == 8 else 0) <= run
+        return long_big, place, blk, run
+
+    for T, L in [(64, 1), (700, 3), (9392, 8), (8192, 128), (4096, 64), (100000, 16), (300, 300)]:
+        lengths = rng.integers(1, max(2, 2 * T // max(1, L)), size=L)
+        slots = np.repeat(np.arange(L), lengths)[:T].tolist()
+        slots += [-1] * (T - len(slots))
+        check(slots, T, L)
+    # many slots of one tile each: tile by tile
+    slots = np.repeat(np.arange(100), 20).tolist()
+    long_big, place, blk, run = check(slots, len(slots), 100)
+    assert run == 1 and [q // blk for q in place[:16]] == list(range(8)) * 2
+    # six slots of twenty tiles each: a slot meets few blocks
+    slots = np.repeat(np.arange(6), 20 * 64).tolist()
+    long_big, place, blk, run = check(slots, len(slots), 6)
+    for s_ in range(6):
+        assert len({place[t] // blk for t in range(len(long_big)) if long_big[t][0] == s_}) <= 20 * 8 // len(long_big) + 2
