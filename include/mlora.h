@@ -51,6 +51,11 @@ extern "C" {
                               record of the slot's first sixteen tokens has arrived; further tiles of a slot are
                               taken by extra workgroups of the same launch */
 
+#define MLORA_FORM_WIDE 8  /* the tiles of MLORA_FORM_SGMV in one launch without anything passing between workgroups:
+                              one workgroup per (tile, column range) multiplies the tile's x rows by A[slot] of the
+                              range's slice over the whole of K, keeps the result in LDS and expands it into its
+                              range; needs no workspace */
+
 /* error codes (negative) */
 #define MLORA_E_INVALID (-1)     /* malformed argument (NULL pointer, negative size, bad dtype) */
 #define MLORA_E_UNSUPPORTED (-2) /* well-formed but outside what the selected form handles */

@@ -79,7 +79,7 @@ namespace {
 
 // Diagnostic knobs, read from the environment once per process.
 struct ApiKnobs {
-  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, split_max_tokens, auto_fused, slot_max_slots;
+  int generation = -1, small_batch_tokens, force_form, no_split, split_min_rk, split_max_tokens, auto_fused, slot_max_slots, no_wide;
   void read() {
     generation = knob_generation();
     small_batch_tokens = env_int("MLORA_SMALL_BATCH_TOKENS", 0);
@@ -91,6 +91,7 @@ struct ApiKnobs {
     // dependent slab fetches per workgroup, HBM nearly idle) and then expands; the saved launch
     // does not pay for the wait on the slowest role of each unit.  AUTO keeps the two launches.
     auto_fused = env_int("MLORA_AUTO_FUSED", 0);
+    no_wide = env_int("MLORA_NO_WIDE", 0);
     // The split form pays when A[slot], which every workgroup of a tile would otherwise fetch whole,
     // is large: rank x K >= 131072 elements (256 KB).  Measured on the decode batch (256 tokens, 32
     // adapters), one workgroup per (tile, column range) against the split form, us per call: rank 16,
@@ -174,7 +175,7 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   if (a->dtype != MLORA_DTYPE_F32 && a->dtype != MLORA_DTYPE_F16 && a->dtype != MLORA_DTYPE_BF16) {
     set_error("mlora_add_lora: unknown dtype %d", a->dtype); return MLORA_E_INVALID;
   }
-  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_SLOT) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
+  if (a->form < MLORA_FORM_AUTO || a->form > MLORA_FORM_WIDE) { set_error("mlora_add_lora: unknown form %d", a->form); return MLORA_E_INVALID; }
   if (a->num_slices > MLORA_MAX_SLICES) { set_error("mlora_add_lora: %d slices exceed %d", a->num_slices, MLORA_MAX_SLICES); return MLORA_E_TOO_LARGE; }
   if (a->r > MLORA_MAX_RANK) { set_error("mlora_add_lora: rank %d exceeds %d", a->r, MLORA_MAX_RANK); return MLORA_E_TOO_LARGE; }
   if (a->num_slots > MLORA_MAX_SLOTS) { set_error("mlora_add_lora: %d slots exceed %d", a->num_slots, MLORA_MAX_SLOTS); return MLORA_E_TOO_LARGE; }
@@ -200,14 +201,17 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
   const bool vec = vector_ok(a);
   if (form == MLORA_FORM_AUTO) {
     const int forced = knobs().force_form;
-    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_SLOT && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
+    if (forced >= MLORA_FORM_TOKEN && forced <= MLORA_FORM_WIDE && (forced == MLORA_FORM_TOKEN || vec)) form = forced;
   }
   if (form == MLORA_FORM_AUTO) {
     // Small batches (decode) are one launch over 16-token tiles; large ones split into 64-token
-    // tiles for the long segments and 16-token tiles for the rest, as two launches.
+    // tiles for the long segments and 16-token tiles for the rest: one launch whose workgroups do
+    // both products where a tile's column ranges repeat little of its shrink, else two launches.
     const bool small_tiles = mfma_supported(a) && decode_supported(a);
     const bool two_launches = mfma_supported(a) && sgmv_supported(a) && sgmv_workspace_ok(a);
+    const bool one_launch = mfma_supported(a) && wide_supported(a) && wide_pays(a) && !knobs().no_wide;
     if (!vec) form = MLORA_FORM_TOKEN;
+    else if (one_launch && !(small_tiles && small_batch(a))) form = MLORA_FORM_WIDE;
     else if (two_launches && !(small_tiles && small_batch(a))) form = MLORA_FORM_SGMV;
     else if (small_tiles) form = MLORA_FORM_SPLIT;
     else form = MLORA_FORM_BGMV;
@@ -236,6 +240,13 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
       if (a->effective_rank) { set_error("mlora_add_lora: the BGMV form does not take effective_rank"); return MLORA_E_UNSUPPORTED; }
       if (!vec) { set_error("mlora_add_lora: BGMV form needs 16-bit elements, a plan, rank in {8,16,32,64} and 16-byte aligned rows"); return MLORA_E_UNSUPPORTED; }
       return launch_bgmv(a, /*include_long=*/true);
+    case MLORA_FORM_WIDE:
+      if (!vec || !mfma_supported(a) || !wide_supported(a)) {
+        set_error("mlora_add_lora: the one-launch form over 64-token tiles needs 16-bit elements, a plan, a rank of 8, 16, 32 or 64, K %% 128 == 0 "
+                  "and no empty slice");
+        return MLORA_E_UNSUPPORTED;
+      }
+      return launch_wide(a);
     case MLORA_FORM_SGMV:
     case MLORA_FORM_FUSED:
     case MLORA_FORM_SPLIT:

@@ -13,6 +13,7 @@ extern "C" int mlora_trace_set(void* buf) {
   split_trace_set(buf);
   fused_trace_set(buf);
   sgmv_trace_set(buf);
+  wide_trace_set(buf);
   return 0;
 #else
   (void)buf;

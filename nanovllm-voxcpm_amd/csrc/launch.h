@@ -57,11 +57,17 @@ int launch_sgmv(const MloraAddArgs* a);
 bool fused_supported(const MloraAddArgs* a);
 int launch_fused(const MloraAddArgs* a, bool trusted_workspace);
 
+// wide.hip: the same tiles, one launch, one workgroup per (tile, column range) doing both products.
+bool wide_supported(const MloraAddArgs* a);
+bool wide_pays(const MloraAddArgs* a);
+int launch_wide(const MloraAddArgs* a);
+
 // in-kernel timeline of trace builds (no-ops otherwise)
 void decode_trace_set(void* buf);
 void slot_trace_set(void* buf);
 void split_trace_set(void* buf);
 void fused_trace_set(void* buf);
 void sgmv_trace_set(void* buf);
+void wide_trace_set(void* buf);
 
 }  // namespace mlora

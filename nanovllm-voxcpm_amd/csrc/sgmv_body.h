@@ -101,10 +101,15 @@ constexpr int kShrinkWaves = 4;
 //
 // SC1: the partial sums leave with agent-scope stores (they pass the compute unit's and the XCD's
 // caches on their way), for readers in other workgroups of the same launch.
-template <typename T, int R, int KR, int XW, bool DB, bool MASKED, bool SC1 = false>
+//
+// TO_LDS: the workgroup multiplies the whole of K for one slice and expands the result itself: the
+// sums do not leave the compute unit but go to LDS (`s_h`, which may be the memory of `s_a`) as the
+// expand wants its operand: scaled, split into a leading part and a remainder of operand precision,
+// zeros for positions past the tile's count and for ranks the adapter does not have.
+template <typename T, int R, int KR, int XW, bool DB, bool MASKED, bool SC1 = false, bool TO_LDS = false>
 __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __restrict__ xv, float* __restrict__ hws, int64_t xs, int T_, int K,
                                             int num_slices, int krange, int all_slices, const ShrinkSlices& sl, int slice0, int kpart, int slot,
-                                            int start, int m, int eff, int row) {
+                                            int start, int m, int eff, int row, T* s_h = nullptr, float scaling = 1.f) {
   constexpr int RB = (R + 15) / 16;      // 16-rank blocks
   constexpr int NT = kShrinkWaves * kWave;
   constexpr int ASTRIDE = KR + 8;        // padded LDS row: 16 rows x 16 bytes cover all banks once
@@ -161,6 +166,31 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
 
   // D layout: lane holds H[rank 16*rb + 4*(lane/16) + i][token lane%16]: four consecutive ranks
   auto write_partials = [&](const f32x4(&part)[RB], int si) {
+    if constexpr (TO_LDS) {
+      constexpr int HSTRIDE = 2 * R + 8;  // the expand's row: R leading parts, R remainders
+      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+      __syncthreads();  // every wavefront is done with the last slab: its memory may be the intermediate's
+      const float live = (active && ti < m) ? scaling : 0.f;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int r0 = rb * 16 + 4 * lg;
+        if (r0 < R) {
+          T hi[4], lo[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float v = r0 + i < eff ? part[rb][i] * live : 0.f;  // (eff = R unless the adapter has fewer ranks)
+            hi[i] = from_f32<T>(v);
+            lo[i] = from_f32<T>(v - to_f32(hi[i]));
+          }
+          u32x2_t h2, l2;
+          __builtin_memcpy(&h2, hi, 8);
+          __builtin_memcpy(&l2, lo, 8);
+          *reinterpret_cast<u32x2_t*>(&s_h[ti * HSTRIDE + r0]) = h2;
+          *reinterpret_cast<u32x2_t*>(&s_h[ti * HSTRIDE + R + r0]) = l2;
+        }
+      }
+      return;
+    }
     if (active && ti < m) {
       float* dst = hws + ((static_cast<int64_t>(kpart) * T_ + start + ti) * num_slices + slice0 + si) * R;
 #pragma unroll
@@ -374,7 +404,7 @@ __device__ __forceinline__ void shrink_body(T* __restrict__ s_a, const void* __r
       for (int b = 0; b < nbatch; ++b) run_batch(xa, xa, si, b);
     }
     if (si == 0) MLORA_STAMP(5);  // shrink: first slice multiplied
-    if (ACT) write_partials(acc, si);
+    if (ACT || TO_LDS) write_partials(acc, si);  // (to LDS: wavefronts without tokens enter zeros)
   }
   };
   if (active) batches(std::true_type{});
@@ -431,7 +461,9 @@ __device__ __forceinline__ void store_y(T* p, const YVec<T, N>& v) {
 //
 // SC1: the partial sums are fetched with agent-scope loads (past the compute unit's and the XCD's
 // caches): they were written by other workgroups of the same launch.
-template <typename T, int R, int CPL, int TPF, int G, bool MASKED, bool SC1 = false>
+//
+// PRE: the intermediate of the (one) tile is in `s_h` already, put there by this workgroup.
+template <typename T, int R, int CPL, int TPF, int G, bool MASKED, bool SC1 = false, bool PRE = false>
 __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict__ s_row, int* __restrict__ s_slot, int* __restrict__ s_m,
                                             int* __restrict__ s_eff, const int32_t* __restrict__ plan, const float* __restrict__ hws,
                                             void* __restrict__ yv_, int64_t ys, int T_, int num_slices, int ksplit,
@@ -645,7 +677,9 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
     if (tid == 0) { s_slot[g] = slot[g]; s_m[g] = m[g]; s_eff[g] = eff[g]; }
     if (m[g] > 0 && tid < MLORA_TILE_BIG) s_row[g * MLORA_TILE_BIG + tid] = rowv[g];
   }
-  if (m[0] > 0) request_h(0);
+  if constexpr (!PRE) {
+    if (m[0] > 0) request_h(0);
+  }
   __syncthreads();
   if constexpr (!SC1) MLORA_STAMP(10);  // expand: token rows (and the first partial sums) here
   first_step = next_step(-1);  // exists: some tile holds tokens
@@ -662,6 +696,7 @@ __device__ __forceinline__ void expand_body(T* __restrict__ s_h, int* __restrict
   // H tiles -> LDS: K partials summed (always in the same order), scaled, split into leading
   // part and remainder; absent tokens get zeros.  All loads of a tile are in flight together.
   auto stage_all = [&]() {
+    if constexpr (PRE) return;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       if (m[g] == 0) continue;

@@ -22,9 +22,9 @@ MAX_SLOTS = 1024
 MAX_RANK = 256
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
-FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT, FORM_FUSED, FORM_SLOT = 0, 1, 2, 3, 4, 5, 6, 7
+FORM_AUTO, FORM_TOKEN, FORM_BGMV, FORM_SGMV, FORM_MFMA, FORM_SPLIT, FORM_FUSED, FORM_SLOT, FORM_WIDE = 0, 1, 2, 3, 4, 5, 6, 7, 8
 FORMS = {"auto": FORM_AUTO, "token": FORM_TOKEN, "bgmv": FORM_BGMV, "sgmv": FORM_SGMV, "mfma": FORM_MFMA, "split": FORM_SPLIT,
-         "fused": FORM_FUSED, "slot": FORM_SLOT}
+         "fused": FORM_FUSED, "slot": FORM_SLOT, "wide": FORM_WIDE}
 
 PLAN_HEADER_WORDS = 16
 (

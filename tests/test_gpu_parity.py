@@ -131,7 +131,7 @@ def test_config1_fp32_matches_reference_torch_loop():
 # ---- config 2: decode, 256 tokens, 32 adapters of rank 16 -----------------------------------------
 
 
-@pytest.mark.parametrize("form", ["auto", "bgmv", "mfma", "split", "sgmv", "token"])
+@pytest.mark.parametrize("form", ["auto", "bgmv", "mfma", "split", "sgmv", "wide", "token"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 def test_config2_decode_bf16(name, form):
     from nanovllm_voxcpm_amd import synthetic
@@ -515,7 +515,7 @@ def test_odd_shapes_take_the_scalar_path(form):
 # ---- config 3: prefill, 16 sequences, 8 adapters of rank 64, a quarter without adapter ------------
 
 
-@pytest.mark.parametrize("form", ["auto", "mfma", "bgmv"])
+@pytest.mark.parametrize("form", ["auto", "sgmv", "wide", "mfma", "bgmv"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 def test_config3_prefill_bf16(name, form):
     from nanovllm_voxcpm_amd import synthetic
@@ -568,6 +568,38 @@ def test_long_segment_form_shapes(rank, dtype, knobs, monkeypatch):
         exact, mag = _exact(proj, x, y0, slots, scaling=0.75)
         _check(got, y0, exact, mag, slots, f"long/{name}/r{rank}/{dtype}/{knobs}")
         assert torch.equal(y._base[:, :16], yw[:, :16]) and torch.equal(y._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
+
+
+@pytest.mark.parametrize("nt", [0, 512, 2048])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rank", [8, 16, 32, 64])
+def test_one_launch_form_over_64_token_tiles_shapes(rank, dtype, nt, monkeypatch):
+    """The one-launch form whose workgroups shrink their tile themselves, on the shapes of the
+    two-launch form's test: segments of 1..130 tokens (short ones, exact tile multiples, tails),
+    rows without adapter, ragged slice widths, row-strided x and y views, K of 128- and 256-column
+    batches and of many batches, every rank, both 16-bit types, narrow and wide column ranges."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print(f"one-launch form over 64-token tiles r={rank} {dtype} nt={nt}", flush=True)
+    _knobs(monkeypatch, MLORA_WIDE_NT=nt or None)
+    shapes = {"p": (512, [72, 200, 8]), "q": (1024, [520]), "s": (640, [64, 72]), "t": (768, [264]), "u": (1536, [136]), "v": (2048, [64]),
+              "w": (256, [2600, 1032])}
+    lengths = [130, 1, 64, 15, 16, 65, 3, 128, 17, 7]
+    slot_of = [2, 0, 5, 1, 3, -1, 4, 2, -1, 6]  # slot 2 twice: two segments merge into one of 258
+    slots = torch.cat([torch.full((n,), s, dtype=torch.int32) for n, s in zip(lengths, slot_of)])
+    slots = slots[torch.randperm(slots.numel(), generator=torch.Generator().manual_seed(9))].cuda()
+    T = slots.numel()
+    for name in shapes:
+        proj = synthetic.make_projection(name, 7, rank, dtype, seed=900 + rank, device="cuda", shapes=shapes)
+        xw, yw = synthetic.make_activations(T, proj.k + 24, sum(proj.widths) + 40, dtype, seed=901, device="cuda")
+        x, y0 = xw[:, 8 : 8 + proj.k], yw[:, 16 : 16 + sum(proj.widths)]  # 16-byte aligned views of wider buffers
+        y = yw.clone()[:, 16 : 16 + sum(proj.widths)]
+        got = _apply("wide", proj, x, y, slots, scaling=0.75)
+        exact, mag = _exact(proj, x, y0, slots, scaling=0.75)
+        _check(got, y0, exact, mag, slots, f"wide/{name}/r{rank}/{dtype}/nt{nt}")
+        assert torch.equal(y._base[:, :16], yw[:, :16]) and torch.equal(y._base[:, 16 + sum(proj.widths):], yw[:, 16 + sum(proj.widths):])
+        assert torch.equal(got, _apply("wide", proj, x, yw.clone()[:, 16 : 16 + sum(proj.widths)], slots, scaling=0.75))  # the same bits again
+    _knobs(monkeypatch, MLORA_WIDE_NT=None)
 
 
 def test_workgroups_of_one_blockidx_x_share_an_xcd():
@@ -655,15 +687,16 @@ def test_long_segment_form_in_one_launch(rank, dtype, knobs, monkeypatch):
         assert head[256 // 4 : 256 // 4 + 2 * 1024].tolist() == state
 
 
-@pytest.mark.parametrize("rank,expected", [(16, "mfma"), (64, "sgmv")])
-def test_auto_form_follows_rank_and_width(rank, expected):
-    """A 3000-token prefill of three sequences through the o projection: at rank 16 the one-launch
-    small-tile form is the faster one up to far larger batches, at rank 64 the two-launch form
-    takes over near 8500 tokens (here 12000).  AUTO gives the oracle's result in both cases
-    and exactly what the form it is meant to pick gives."""
-    print(f"auto form r={rank}", flush=True)
+@pytest.mark.parametrize("name,rank,expected", [("o", 16, "mfma"), ("o", 64, "wide"), ("gate_up", 64, "sgmv"), ("down", 64, "sgmv")])
+def test_auto_form_follows_rank_and_width(name, rank, expected):
+    """A 3000-token prefill of three sequences: at rank 16 the one-launch small-tile form is the
+    faster one up to far larger batches; at rank 64 the forms over 64-token tiles take over near
+    8500 tokens (here 12000): the one-launch form where a tile's column ranges repeat little of its
+    shrink (o), the two-launch form elsewhere (gate_up: many ranges, down: a long K).  AUTO gives
+    the oracle's result in every case and exactly what the form it is meant to pick gives."""
+    print(f"auto form {name} r={rank}", flush=True)
     T = 3000 if rank == 16 else 12000
-    proj = _make("o", 4, rank, torch.bfloat16, seed=330 + rank)
+    proj = _make(name, 4, rank, torch.bfloat16, seed=330 + rank)
     slots = torch.cat([torch.full((T // 2,), 1, dtype=torch.int32), torch.full((T // 4,), -1, dtype=torch.int32),
                        torch.full((T - T // 2 - T // 4,), 3, dtype=torch.int32)]).cuda()
     from nanovllm_voxcpm_amd import synthetic
@@ -671,7 +704,7 @@ def test_auto_form_follows_rank_and_width(rank, expected):
     x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=331, device="cuda")
     got = _apply("auto", proj, x, y0.clone(), slots)
     exact, mag = _exact(proj, x, y0, slots)
-    _check(got, y0, exact, mag, slots, f"auto/r{rank}")
+    _check(got, y0, exact, mag, slots, f"auto/{name}/r{rank}")
     assert torch.equal(got, _apply(expected, proj, x, y0.clone(), slots))
 
 
@@ -741,7 +774,7 @@ def test_seeded_random_shapes_all_forms_agree_with_the_oracle(seed):
     yw = torch.randn(T, sum(widths) + 2 * pad_y, generator=g).to(dtype).cuda()
     x, y0 = xw[:, pad_x : pad_x + K], yw[:, pad_y : pad_y + sum(widths)]
     exact, mag = _exact(proj, x, y0, slots, scaling=0.5)
-    forms = ["auto", "token", "bgmv", "mfma"] + (["sgmv"] if K % 128 == 0 else [])
+    forms = ["auto", "token", "bgmv", "mfma"] + (["sgmv", "wide"] if K % 128 == 0 else [])
     for form in forms:
         y = yw.clone()[:, pad_y : pad_y + sum(widths)]
         got = _apply(form, proj, x, y, slots, scaling=0.5)

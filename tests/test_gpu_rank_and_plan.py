@@ -29,7 +29,7 @@ def _poisoned(proj, ranks):
     return a, b
 
 
-@pytest.mark.parametrize("form", ["auto", "split", "mfma", "slot", "sgmv", "token"])
+@pytest.mark.parametrize("form", ["auto", "split", "mfma", "slot", "sgmv", "wide", "token"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 @pytest.mark.parametrize("tokens", [200, 3000])
 def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, form):
@@ -82,7 +82,7 @@ def test_rank_masking_never_touches_what_lies_beyond_a_slots_rank(name, tokens, 
     assert _hip.FORMS[form] >= 0
 
 
-@pytest.mark.parametrize("form", ["auto", "sgmv", "fused", "mfma", "split"])
+@pytest.mark.parametrize("form", ["auto", "sgmv", "wide", "fused", "mfma", "split"])
 @pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
 def test_last_k_steps_of_every_k_part_count_for_adapters_of_every_rank(name, form):
     """x is zero except for the last 32 columns of every sixteenth of K (the last MFMA step of every
@@ -268,7 +268,7 @@ def test_context_plans_follow_an_in_place_refresh_of_graph_buffers():
         assert torch.allclose(y.double().cpu(), want, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("form", ["mfma", "slot", "split", "sgmv", "fused", "bgmv"])
+@pytest.mark.parametrize("form", ["mfma", "slot", "split", "sgmv", "wide", "fused", "bgmv"])
 def test_a_plan_of_another_batch_shape_is_counted_not_followed(form):
     """Through the C-ABI a plan built for another (num_tokens, max_slots) is only recognised on the
     device: the call returns 0, y keeps its bits, and the launch is counted in the header of the
