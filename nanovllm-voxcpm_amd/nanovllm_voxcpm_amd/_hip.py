@@ -284,6 +284,26 @@ def load_error() -> str | None:
     return None
 
 
+def load_fastcall():
+    """The module with the C++ host path of the usual add_lora call (csrc/fastcall.cpp, built beside
+    the library by ``make fastcall``), or None where it is not built or does not load: the Python
+    path then does every call.  It launches nothing itself: it calls the library's entry points."""
+    try:
+        from nanovllm_voxcpm_amd import _mlora_fastcall
+    except ImportError:
+        return None
+    return _mlora_fastcall
+
+
+def entry_point_addresses() -> tuple[int, int] | None:
+    """Addresses of mlora_add_lora and mlora_add_workspace_bytes in the loaded library, None without it."""
+    try:
+        lib = load()
+    except RuntimeError:
+        return None
+    return C.cast(lib.mlora_add_lora, C.c_void_p).value, C.cast(lib.mlora_add_workspace_bytes, C.c_void_p).value
+
+
 def _check(rc: int, what: str) -> None:
     if rc != 0:
         msg = load().mlora_last_error().decode("utf-8", "replace")
@@ -307,6 +327,24 @@ def _stream(device: torch.device) -> int:
 
 
 current_stream_handle = _stream
+
+# torch's own bindings for two questions asked on every call (a foreign call through ctypes costs
+# about a microsecond, these a fraction of it); None where this torch build lacks them
+_torch_is_capturing = getattr(torch._C, "_cuda_isCurrentStreamCapturing", None)
+_torch_get_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def current_device_index() -> int:
+    """Index of the calling thread's current GPU."""
+    return _torch_get_device() if _torch_get_device is not None else torch.cuda.current_device()
+
+
+def current_stream_capture_id(device: torch.device, stream: int) -> int:
+    """stream_capture_id for ``stream`` = torch's current stream on the calling thread's current
+    device ``device``: 0 straight from torch when no capture is in progress there."""
+    if _torch_is_capturing is not None and not _torch_is_capturing():
+        return 0
+    return stream_capture_id(device, stream)
 
 _SAME_DEVICE = contextlib.nullcontext()
 
@@ -396,6 +434,13 @@ def add_lora(
         raise ValueError(f"token_to_slot has {token_to_slot.numel()} entries for {x.size(0)} rows of x")
     if y.size(0) < x.size(0):
         raise ValueError(f"y has {y.size(0)} rows for {x.size(0)} rows of x")
+    # the shapes the reference's matmuls would object to (the kernels take K from x and the rank and
+    # the slot count from the first A slice: a buffer of another shape would be read with the wrong strides)
+    k, r, slots = x.size(1), a_slices[0].size(-2), a_slices[0].size(0)
+    for i, (a, b) in enumerate(zip(a_slices, b_slices)):
+        if a.dim() != 3 or b.dim() != 3 or a.size(-1) != k or a.size(-2) != r or a.size(0) != slots or b.size(-1) != r or b.size(0) != slots:
+            raise ValueError(f"lora_a[{i}] {tuple(a.shape)} / lora_b[{i}] {tuple(b.shape)} do not fit x [{x.size(0)}, {k}] with "
+                             f"{slots} slots of rank {r} ([slots, rank, K] and [slots, N, rank] are expected)")
     _require_cuda(x, "x")
     args = MloraAddArgs()
     args.stream = _stream(x.device) if stream is None else stream

@@ -13,6 +13,7 @@ There is no host fallback: without a GPU or without the built library the probed
 
 from __future__ import annotations
 
+import ctypes as C
 import os
 import struct
 import threading
@@ -134,6 +135,21 @@ class HipLoRABackend:
         self._spares: dict = {}          # device -> initialised buffer kept for the next graph capture
         self._graph_scratch: dict = {}   # device -> buffers captured graphs refer to (the last one is in use)
         self._sites = threading.local()  # per thread: weight buffers -> _CallSite
+        # the C++ host path of the usual call (optional: built beside the library; MLORA_NO_FASTCALL=1 keeps to Python)
+        self._fastcall = None if os.environ.get("MLORA_NO_FASTCALL", "0") not in ("", "0") else _hip.load_fastcall()
+
+    def _fast_state(self):
+        """This thread's state object of the C++ host path, None without the module or the library."""
+        fc = self._fastcall
+        if fc is None:
+            return None
+        state = getattr(self._sites, "fast", None)
+        if state is None:
+            addresses = _hip.entry_point_addresses()
+            if addresses is None:
+                return None
+            state = self._sites.fast = fc.create(*addresses)
+        return state
 
     # -- capability ---------------------------------------------------------------------
     def availability(self) -> LoRAAvailability:
@@ -332,9 +348,14 @@ class HipLoRABackend:
         site.view = memoryview(args).cast("B")
         site.k, site.rank, site.num_slots, site.dtype, site.device, site.widths = k, rank, slots, dt, dev, widths
         site.weights_vectorisable, site.num_slices = ok, len(a_list)
+        fast = self._fast_state()
         if len(table) >= 512:
             table.clear()
+            if fast is not None:
+                self._fastcall.clear_sites(fast)
         table[key] = site
+        if fast is not None:  # (it keeps the block alive itself; its key is the one above)
+            self._fastcall.register_site(fast, a_list, b_list, widths, C.addressof(args), args, ok)
         return site
 
     def _add_lora_at_site(self, outputs, target, x, a_list, b_list, indices, metadata, scaling, effective_rank) -> bool:
@@ -364,12 +385,12 @@ class HipLoRABackend:
                 return False
             eff_ptr = effective_rank.data_ptr()
         dev = site.device
-        if dev.index is not None and dev.index != torch.cuda.current_device():
+        if dev.index is not None and dev.index != _hip.current_device_index():
             return False  # another GPU of this process: the general path makes it current
         stream = _hip.current_stream_handle(dev)
         plan_ptr = ws_ptr = ws_bytes = 0
         if site.weights_vectorisable and args.form != _hip.FORM_TOKEN and not (xs % 8 or ys % 8 or x_ptr % 16 or y_ptr % 16):
-            capture = _hip.stream_capture_id(dev, stream)
+            capture = _hip.current_stream_capture_id(dev, stream)
             # every LoRA linear of a step calls with the same metadata object, slot vector, stream
             # and capture: what the last call of this thread looked up serves the next one
             try:
@@ -386,8 +407,18 @@ class HipLoRABackend:
                 plan_ptr = plan.workspace.data_ptr()
                 # (the plan object is part of the memo: its workspace stays allocated while it is remembered)
                 self._sites.step = (metadata, source, version, capture, stream, site.num_slots, rows, plan_ptr, plan)
+                fast = self._fast_state()
+                if fast is not None:
+                    if capture or version is None:
+                        self._fastcall.forget_step(fast)
+                    else:  # (the tuple above keeps metadata, slot vector and plan alive for as long as this stands)
+                        self._fastcall.set_step(fast, metadata, source, version, stream or 0, site.num_slots, rows, plan_ptr)
             scratch = self._scratch_for(x, site.num_slices, site.rank, stream, capture)
             ws_ptr, ws_bytes = scratch.data_ptr(), scratch.numel()
+            if not capture:
+                fast = self._fast_state()
+                if fast is not None:  # (held in self._scratch for as long as it is the stream's buffer)
+                    self._fastcall.set_scratch(fast, dev.index if dev.index is not None else _hip.current_device_index(), stream or 0, ws_ptr, ws_bytes)
         # the per-step fields, written in three strokes (they lie together in the block; one attribute
         # assignment per field costs several times as much)
         _STEP_HEAD.pack_into(site.view, 0, stream or 0, x_ptr, y_ptr, xs, ys, source.data_ptr(), plan_ptr, rows)
@@ -423,6 +454,14 @@ class HipLoRABackend:
         ``y_packed`` are gathered into a new packed buffer whose views are returned and the
         caller's tensors stay untouched (reference: nanovllm_voxcpm/lora.py:276-289).
         """
+        fast = getattr(self._sites, "fast", None)
+        if fast is not None:
+            # the usual call, when nothing about it is new: checked, filled in and enqueued in C++
+            rc = self._fastcall.call(fast, y_slices, x, lora_a_slices, lora_b_slices, indices, metadata, scaling, y_packed, effective_rank)
+            if rc == 0:
+                return list(y_slices)
+            if rc < 0:
+                _hip._check(rc, "mlora_add_lora")
         if not y_slices:
             return []
         if not (len(y_slices) == len(lora_a_slices) == len(lora_b_slices)):
@@ -455,9 +494,11 @@ class HipLoRABackend:
             return outputs
 
         cols, col = [], 0
-        for y in outputs:
+        for i, y in enumerate(outputs):
             cols.append(col)
             col += y.size(-1)
+            if y.numel() > 0 and lora_b_slices[i].dim() == 3 and lora_b_slices[i].size(1) != y.size(-1):  # (empty slices are skipped)
+                raise ValueError(f"y slice {i} has {y.size(-1)} columns, lora_b[{i}] {tuple(lora_b_slices[i].shape)} gives {lora_b_slices[i].size(1)}")
         live = [i for i, y in enumerate(outputs) if y.numel() > 0]
         if not live:
             return outputs

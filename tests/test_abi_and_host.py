@@ -465,3 +465,34 @@ def test_rank_masking_under_graph_capture(monkeypatch):
     assert wide._wants_rank_masking() is True
     narrow = lora_layers.LoRALinear(8, 4, bias=False, max_loras=2, max_lora_rank=16)
     assert narrow._wants_rank_masking() is False
+
+
+def test_cpp_host_path_loads_and_leaves_what_it_does_not_know_to_python():
+    """The C++ host path of the usual add_lora call is built beside the library and loads; it
+    registers nothing for tensors that are not on a GPU, and answers "not handled" for weight
+    buffers nobody registered, for a missing metadata object and for arguments that are no tensors
+    (no compute call is made here: its state object holds no entry points)."""
+    import torch
+
+    from nanovllm_voxcpm_amd import _hip
+
+    fc = _hip.load_fastcall()
+    assert fc is not None, "make -C nanovllm-voxcpm_amd/csrc fastcall"
+    for name in ("create", "register_site", "clear_sites", "set_step", "forget_step", "set_scratch", "counters", "call"):
+        assert hasattr(fc, name), name
+    state = fc.create(0, 0)
+    a, b = [torch.zeros(2, 8, 32)], [torch.zeros(2, 16, 8)]
+    x, y = torch.zeros(4, 32), torch.zeros(4, 16)
+    slots = torch.zeros(4, dtype=torch.int32)
+    args = _hip.MloraAddArgs()
+    import ctypes
+
+    assert fc.register_site(state, a, b, (16,), ctypes.addressof(args), args, True) is False  # host tensors
+    meta = type("Meta", (), {"no_lora_flag": False, "token_to_slot": slots})()
+    assert fc.call(state, [y], x, a, b, slots, meta, 1.0, None, None) == fc.NOT_HANDLED
+    assert fc.call(state, [y], x, a, b, slots, None, 1.0, None, None) == fc.NOT_HANDLED
+    assert fc.call(state, [y], "x", a, b, slots, meta, 1.0, None, None) == fc.NOT_HANDLED
+    assert fc.call(state, [], x, [], [], slots, meta, 1.0, None, None) == fc.NOT_HANDLED
+    assert fc.counters(state) == (0, 4)
+    fc.clear_sites(state)
+    fc.forget_step(state)

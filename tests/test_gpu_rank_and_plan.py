@@ -489,3 +489,95 @@ def test_config5_backbone_at_its_own_shape():
           f"mean abs error: hip {err_hip.mean().item():.5f}, reference {err_ref.mean().item():.5f}", flush=True)
     assert worst_hip <= 1.5 * worst_ref and worst_hip <= 0.15, (worst_hip, worst_ref)
     assert err_hip.mean().item() <= 1.25 * err_ref.mean().item() + 1e-4, (err_hip.mean().item(), err_ref.mean().item())
+
+
+# ---- the C++ host path of the usual call ------------------------------------------------------------
+
+
+def test_the_cpp_host_path_enqueues_what_the_python_path_would(monkeypatch):
+    """Steps of three layers x four projections, one metadata object per step as the engine installs
+    one context per step, through a backend with the C++ host path and through one without
+    (MLORA_NO_FASTCALL=1): the same bits for every output of every step.  The C++ path takes every
+    call but those that bring something new - the first call of a step (its plan), the first use of
+    a set of weight buffers - and passes on what the Python path has to answer: a slot vector
+    rewritten in place (followed, not the old plan), a packed output with the wrong slice widths
+    and an x of the wrong K (both raise the Python path's errors), a step whose flag says that no
+    token has a slot (a no-op)."""
+    from nanovllm_voxcpm_amd import _hip, synthetic
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend
+
+    if _hip.load_fastcall() is None:
+        pytest.skip("the C++ host path is not built (make -C nanovllm-voxcpm_amd/csrc fastcall)")
+    print("C++ host path against the Python path", flush=True)
+    L, rank, T = 8, 16, 96
+    names = ["qkv", "o", "gate_up", "down"]
+    layers = [{n: _make(n, L, rank, torch.bfloat16, seed=990 + 7 * i + j) for j, n in enumerate(names)} for i in range(3)]
+    acts = {n: synthetic.make_activations(T, layers[0][n].k, sum(layers[0][n].widths), torch.bfloat16, seed=995 + j, device="cuda")
+            for j, n in enumerate(names)}
+    eff = torch.tensor([16, 8, 12, 16, 0, 16, 4, 16], dtype=torch.int32, device="cuda")
+    g = torch.Generator().manual_seed(996)
+
+    monkeypatch.setenv("MLORA_NO_FASTCALL", "1")
+    plain = HipLoRABackend("auto")
+    monkeypatch.delenv("MLORA_NO_FASTCALL")
+    fast = HipLoRABackend("auto")
+    assert plain._fastcall is None and fast._fastcall is not None
+
+    def step(backend, slots, with_eff):
+        meta = _metadata(slots)
+        outs = []
+        for layer in layers:
+            for n in names:
+                proj = layer[n]
+                x, y0 = acts[n]
+                y = y0.clone()
+                blocks = list(y.split(proj.widths, dim=-1))
+                got = backend.add_lora(blocks, x, proj.a, proj.b, indices=slots, metadata=meta, scaling=0.5,
+                                       y_packed=y if len(blocks) > 1 else None, effective_rank=eff if with_eff else None)
+                assert all(a.data_ptr() == b.data_ptr() for a, b in zip(got, blocks))
+                outs.append(y)
+        return outs
+
+    calls = 0
+    for s in range(4):
+        slots = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32).cuda()
+        want = step(plain, slots, with_eff=s % 2 == 1)
+        got = step(fast, slots, with_eff=s % 2 == 1)
+        calls += len(got)
+        assert all(torch.equal(a, b) for a, b in zip(got, want)), f"step {s}"
+    state = fast._fast_state()
+    handled, passed_on = fast._fastcall.counters(state)
+    # the very first call makes the state object and is not counted; passed on: every other weight
+    # set's first call (11) and the first call of the other three steps
+    assert handled + passed_on == calls - 1
+    assert passed_on == 11 + 3 and handled == calls - 15
+
+    # one metadata object, its slot vector rewritten in place between two calls: the second call follows the new ids
+    proj = layers[0]["o"]
+    x, y0 = acts["o"]
+    slots = torch.randint(0, L, (T,), generator=g, dtype=torch.int32).cuda()
+    meta = _metadata(slots)
+    y1, y2 = y0.clone(), y0.clone()
+    fast.add_lora([y1], x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)
+    fast.add_lora([y1.clone()], x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)  # (taken in C++)
+    slots.copy_(torch.randint(0, L, (T,), generator=g, dtype=torch.int32).cuda())
+    fast.add_lora([y2], x, proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(y2, y0, exact, mag, slots, "host path/slot vector rewritten in place")
+
+    # what has to raise raises as before, whichever path saw the weights last
+    with pytest.raises(ValueError):
+        fast.add_lora([y0.clone()], x[:, :512], proj.a, proj.b, indices=slots, metadata=meta, scaling=1.0)
+    qkv = layers[0]["qkv"]
+    xq, yq = acts["qkv"]
+    with pytest.raises((ValueError, RuntimeError)):
+        fast.add_lora(list(yq.clone().split([512, 512, 512], dim=-1)), xq, qkv.a, qkv.b, indices=slots, metadata=meta, scaling=1.0,
+                      y_packed=yq.clone())
+    # a step in which no token has a slot is a no-op
+    from nanovllm_voxcpm_amd.lora import LoRAMetadata
+
+    none = LoRAMetadata(token_to_slot=slots, token_indices_sorted_by_slot=None, active_slot_ids=None, num_tokens_per_slot=None,
+                        slot_start_offsets=None, no_lora_flag=True, num_active_loras=0)
+    y3 = y0.clone()
+    fast.add_lora([y3], x, proj.a, proj.b, indices=slots, metadata=none, scaling=1.0)
+    assert torch.equal(y3, y0)
