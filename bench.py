@@ -309,9 +309,9 @@ def run_backbone(args) -> None:
 
 
 KERNELS = {
-    "decode": "slot_kernel<bf16,16> (o, gate_up, down) + decode_kernel<bf16,16> (qkv)",
-    "prefill": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
-    "mixed": "sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64>",
+    "decode": "slot_kernel3<bf16,16> (qkv) + slot_kernel<bf16,16> (o, gate_up, down)",
+    "prefill": "wide_kernel<bf16,64> (qkv, o) + sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64> (gate_up, down)",
+    "mixed": "wide_kernel<bf16,64> (qkv, o) + sgmv_shrink_kernel<bf16,64> + sgmv_expand_kernel<bf16,64> (gate_up, down)",
 }
 
 

@@ -127,14 +127,20 @@ const ApiKnobs& knobs() {
 // gate_up 900 / 1400 / 4500, down 1000 / 1500 / 4800).
 // The rank-64 limit is 1.5e7: with many adapters in the batch the small tiles lose earlier (the
 // mixed batch, 8192 tokens and 128 adapters: o 28.8 us per call on small tiles, 23.0 in two launches).
+// Where the other form would be the one-launch form over 64-token tiles (`one_launch`), which
+// pays about half as much before it moves data, the small tiles lose earlier: measured on the same
+// batches, us per call over small tiles / in one launch over 64-token tiles, by tokens of the batch:
+// rank 64, qkv: 14.8 / 14.3 at 1620, 15.4 / 14.6 at 2098, 18.0 / 15.0 at 3250, 21.2 / 15.5 at 4511;
+// o: 10.5 / 14.8 at 4511, 18.1 / 15.2 at 6648; rank 32, qkv: 11.5 / 12.3 at 3250, 14.4 / 12.8 at 4511;
+// o: 12.4 / 12.6 at 6648, 13.9 / 14.8 at 9392: the limits are 0.65 times the above there.
 // MLORA_SMALL_BATCH_TOKENS, when set, replaces the rule by a plain token count.
-static bool small_batch(const MloraAddArgs* a) {
+static bool small_batch(const MloraAddArgs* a, bool one_launch) {
   const int fixed = knobs().small_batch_tokens;
   if (fixed > 0) return a->num_tokens <= fixed;
   double cols = 0;
   for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
   const double width = static_cast<double>(a->num_slices) * a->k * (a->k > 1024 ? a->k / 1024.0 : 1.0) + cols * (cols > 4096 ? cols / 4096.0 : 1.0);
-  const double limit = a->r <= 16 ? 8.3e7 : a->r <= 32 ? 2.6e7 : 1.5e7;
+  const double limit = (a->r <= 16 ? 8.3e7 : a->r <= 32 ? 2.6e7 : 1.5e7) * (one_launch ? 0.65 : 1.0);
   return a->num_tokens * width <= limit;
 }
 
@@ -147,8 +153,12 @@ static bool small_batch(const MloraAddArgs* a) {
 // takes 967 us per decode step against 629.  With K shared out between a tile's workgroups (down) it
 // is the faster one throughout (5.2 / 5.6 at 4 tokens, 6.4 / 6.8 at 256).  So: always with K parts;
 // else while all slots together weigh at most 3 MB, or when the batch has four tokens per slot id.
+// All of this was measured on decode batches; on batches of many tiles per slot (a prefill of
+// 2098 tokens over 8 slot ids, o: 15.4 us per call against 10.1 tile-major) the grid over the slots
+// is the slower one: it is taken up to 32 tokens per slot id.
 static bool slot_major_pays(const MloraAddArgs* a) {
   if (a->num_slots > knobs().slot_max_slots) return false;
+  if (a->num_tokens > 32 * a->num_slots) return false;
   if (slot_k_parts(a) > 1) return true;
   double cols = 0;
   for (int i = 0; i < a->num_slices; ++i) cols += a->slices[i].n;
@@ -211,8 +221,8 @@ int add_lora_impl(const MloraAddArgs* a, bool trusted_workspace) {
     const bool two_launches = mfma_supported(a) && sgmv_supported(a) && sgmv_workspace_ok(a);
     const bool one_launch = mfma_supported(a) && wide_supported(a) && wide_pays(a) && !knobs().no_wide;
     if (!vec) form = MLORA_FORM_TOKEN;
-    else if (one_launch && !(small_tiles && small_batch(a))) form = MLORA_FORM_WIDE;
-    else if (two_launches && !(small_tiles && small_batch(a))) form = MLORA_FORM_SGMV;
+    else if (one_launch && !(small_tiles && small_batch(a, true))) form = MLORA_FORM_WIDE;
+    else if (!one_launch && two_launches && !(small_tiles && small_batch(a, false))) form = MLORA_FORM_SGMV;
     else if (small_tiles) form = MLORA_FORM_SPLIT;
     else form = MLORA_FORM_BGMV;
   }
