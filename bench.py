@@ -555,7 +555,7 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode", choices=sorted(WORKLOADS))
-    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | slot | split | sgmv | fused | token")
+    ap.add_argument("--form", default="auto", help="kernel family: auto | bgmv | mfma | slot | split | sgmv | wide | fused | token")
     ap.add_argument("--only", default=None, choices=ORDER, help="restrict the step to one projection (profiling)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of graph replay")
     ap.add_argument("--slot-ids", type=int, default=0,
