@@ -48,8 +48,15 @@ def set_weight_loader(param: nn.Parameter, loader) -> None:
     param.weight_loader = loader
 
 
+_stream_is_capturing = getattr(torch._C, "_cuda_isCurrentStreamCapturing", None)
+
+
 def _is_cuda_graph_capture() -> bool:
-    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+    # (asked on every forward: without an initialised GPU runtime nothing can be capturing, and
+    # torch's own binding answers in a fraction of what the wrappers around it take)
+    if not torch.cuda.is_initialized():
+        return False
+    return _stream_is_capturing() if _stream_is_capturing is not None else torch.cuda.is_current_stream_capturing()
 
 
 class _LoRALayerBase(nn.Module):
@@ -72,6 +79,8 @@ class _LoRALayerBase(nn.Module):
         self._lora_scaling_values = [0.0] * max_loras
         self._lora_base_scaling_values = [0.0] * max_loras
         self._effective_lora_rank_values = [0] * max_loras
+        self._rank_summary_of: list | None = None  # the mirror the summary below was made from
+        self._rank_summary = (False, False)
 
     # ---- subclass contract ------------------------------------------------------------------
     def _target_keys(self) -> list:
@@ -99,12 +108,23 @@ class _LoRALayerBase(nn.Module):
     def _slot_scaling(self, slot_id: int) -> float:
         return self._lora_scaling_values[slot_id]
 
+    def _residency(self) -> tuple[bool, bool]:
+        """(some slot holds an adapter, some resident adapter is below the padded rank), from the
+        host mirror; walked again only when the mirror has changed (a list comparison otherwise:
+        this runs on every forward)."""
+        values = self._effective_lora_rank_values
+        if self._rank_summary_of != values:
+            resident = [rank for rank in values if rank > 0]
+            self._rank_summary = (bool(resident), any(rank < self.max_lora_rank for rank in resident))
+            self._rank_summary_of = list(values)
+        return self._rank_summary
+
     def _batch_has_no_effective_rank(self, context) -> bool:
         """True iff no slot this batch can reference holds an adapter in this module.  Decided
         from the host mirrors only; a device-resident ``active_slot_ids`` is not read."""
         active = getattr(context, "active_slot_ids", None)
         if active is None or active.is_cuda:
-            return not any(rank > 0 for rank in self._effective_lora_rank_values)
+            return not self._residency()[0]
         return not any(s >= 0 and self._effective_lora_rank_values[int(s)] > 0 for s in active.tolist())
 
     def _resolve_token_slots(self, x_flat: torch.Tensor) -> torch.Tensor | None:
@@ -196,10 +216,10 @@ class _LoRALayerBase(nn.Module):
         zero-fills the ranks it does not use.  Decided from the host mirror only."""
         if self.max_lora_rank <= 16:
             return False
-        resident = [rank for rank in self._effective_lora_rank_values if rank > 0]
-        if _is_cuda_graph_capture() and not resident:
-            return True
-        return any(rank < self.max_lora_rank for rank in resident)
+        some_resident, some_below = self._residency()
+        if not some_resident:
+            return _is_cuda_graph_capture()
+        return some_below
 
     def prime_lora_cache(self) -> None:
         if not self.supports_lora:
