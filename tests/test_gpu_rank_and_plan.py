@@ -581,3 +581,72 @@ def test_the_cpp_host_path_enqueues_what_the_python_path_would(monkeypatch):
     y3 = y0.clone()
     fast.add_lora([y3], x, proj.a, proj.b, indices=slots, metadata=none, scaling=1.0)
     assert torch.equal(y3, y0)
+
+
+def test_the_cpp_host_path_keeps_a_state_per_thread():
+    """Two threads drive one backend, each on a stream of its own with its own batches: every
+    thread has its own state object of the C++ host path (argument blocks, step, scratch buffer),
+    so neither enqueues with what the other looked up.  Every output equals what a backend
+    without the C++ path gives for the same inputs."""
+    import threading
+
+    from nanovllm_voxcpm_amd import _hip, synthetic
+    from nanovllm_voxcpm_amd.lora import HipLoRABackend
+
+    if _hip.load_fastcall() is None:
+        pytest.skip("the C++ host path is not built (make -C nanovllm-voxcpm_amd/csrc fastcall)")
+    print("C++ host path, two threads", flush=True)
+    L, rank = 6, 32
+    names = ["o", "down", "qkv"]
+    projs = {n: _make(n, L, rank, torch.bfloat16, seed=1100 + j) for j, n in enumerate(names)}
+    fast = HipLoRABackend("auto")
+    results, errors = {}, []
+
+    def worker(tag, T, seed):
+        try:
+            stream = torch.cuda.Stream()
+            g = torch.Generator().manual_seed(seed)
+            acts = {n: synthetic.make_activations(T, projs[n].k, sum(projs[n].widths), torch.bfloat16, seed=seed + j, device="cuda")
+                    for j, n in enumerate(names)}
+            outs = []
+            torch.cuda.current_stream().synchronize()
+            with torch.cuda.stream(stream):
+                for step in range(6):
+                    slots = torch.randint(-1, L, (T,), generator=g, dtype=torch.int32).cuda()
+                    meta = _metadata(slots)
+                    for rep in range(2):  # every projection twice per step: the second call is the C++ path's
+                        for n in names:
+                            x, y0 = acts[n]
+                            y = y0.clone()
+                            blocks = list(y.split(projs[n].widths, dim=-1))
+                            fast.add_lora(blocks, x, projs[n].a, projs[n].b, indices=slots, metadata=meta, scaling=1.0,
+                                          y_packed=y if len(blocks) > 1 else None)
+                            outs.append((n, slots, y))
+                stream.synchronize()
+            results[tag] = (acts, outs)
+        except Exception as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append((tag, exc))
+
+    threads = [threading.Thread(target=worker, args=("a", 80, 1200)), threading.Thread(target=worker, args=("b", 200, 1300))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    import os
+
+    os.environ["MLORA_NO_FASTCALL"] = "1"
+    try:
+        plain = HipLoRABackend("auto")
+    finally:
+        del os.environ["MLORA_NO_FASTCALL"]
+    assert plain._fastcall is None
+    for tag, (acts, outs) in results.items():
+        for n, slots, got in outs:
+            x, y0 = acts[n]
+            want = y0.clone()
+            blocks = list(want.split(projs[n].widths, dim=-1))
+            plain.add_lora(blocks, x, projs[n].a, projs[n].b, indices=slots, metadata=_metadata(slots), scaling=1.0,
+                           y_packed=want if len(blocks) > 1 else None)
+            assert torch.equal(got, want), (tag, n)
