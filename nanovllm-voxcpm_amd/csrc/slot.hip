@@ -119,8 +119,8 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
   }
   i32x4 ast[RB][4 * ROUNDS];
   Pack8 bop[SA][4][KSTEPS];
-  // every A line of this wavefront's K range and the B rows of its spans
-  auto request_weights = [&](const int slot, const int rb_n) {
+  // every A line of this wavefront's K range
+  auto request_a = [&](const int slot, const int rb_n) {
     const T* A = static_cast<const T*>(sp.a) + static_cast<int64_t>(slot) * rbuf * K;
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
@@ -135,6 +135,9 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
         }
       }
     }
+  };
+  // the B rows of its spans
+  auto request_b = [&](const int slot) {
     const T* B = static_cast<const T*>(sp.b) + static_cast<int64_t>(slot) * sp.n * rbuf;
 #pragma unroll
     for (int s = 0; s < SA; ++s) {
@@ -171,14 +174,8 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int j = 0; j < 4 * ROUNDS; ++j) asm volatile("" ::"v"(ast[rb][j]));
-#pragma unroll
-    for (int s = 0; s < SA; ++s)
-#pragma unroll
-      for (int j = 0; j < (K16 ? 2 : 4); ++j)
-#pragma unroll
-        for (int ks = 0; ks < (K16 ? 1 : KSTEPS); ++ks) asm volatile("" ::"v"(bop[s][j][ks].raw));
   };
-  if constexpr (EARLY) request_weights(slot_early, RB);
+  if constexpr (EARLY) request_a(slot_early, RB);
   // (everything above is requested before anything below is scheduled)
   __builtin_amdgcn_sched_barrier(0);
 
@@ -250,7 +247,7 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
     }
   }
   const int rb_n = MASKED ? (eff + 15) >> 4 : RB;  // 16-rank blocks of A in use
-  if constexpr (!EARLY) request_weights(slot, rb_n);
+  if constexpr (!EARLY) request_a(slot, rb_n);
 
   // ---- the rows the record names --------------------------------------------------------------
   i32x4 xst[4 * ROUNDS];
@@ -260,6 +257,9 @@ __device__ __forceinline__ void slot_tile(const int32_t* __restrict__ rec, const
 #pragma unroll
     for (int i = 0; i < 4; ++i) xst[4 * r + i] = load128(static_cast<const T*>(xv) + static_cast<int64_t>(rows4[i]) * xs + koff);
   }
+  // (the B rows behind the x rows: they are not needed before the expand, and in front of the
+  // record's wait they would hold the x rows up for as long as it takes to hand them over)
+  request_b(slot);
   uint2 yq[SA][4];  // four columns of four tokens per lane and span
   T* const ycols = static_cast<T*>(yv_) + y_col;
   auto request_y = [&](int c0, uint2(&yy)[4]) {
