@@ -602,14 +602,15 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel(const int32_t* __restr
 }
 
 // Three slices (the stacked q | k | v projection): six pointers do not fit the fourteen preloaded
-// dwords, so the second and third slice's travel as 32-bit offsets from the first one's, in units of
-// 16 bytes (the launcher takes this kernel only when they fit), and the widths as 16-bit counts of
-// eight columns.  widths01 = n0 / 8 | n1 / 8 << 16; widths2 = n2 / 8 | ranges of slice 0 << 16 |
+// dwords, so the second and third slice's travel as 40-bit offsets from the first one's, in units of
+// 16 bytes (+-8 TiB: the slices of a projection are allocations of their own and may lie far apart;
+// the launcher takes this kernel only when they fit): their low 32 bits as four arguments, their
+// high 8 bits together in a fifth; the widths as 16-bit counts of eight columns.  widths01 = n0 / 8 | n1 / 8 << 16; widths2 = n2 / 8 | ranges of slice 0 << 16 |
 // ranges of slices 0 and 1 << 24; packed = columns per range / 64 | slots << 16.
 template <typename T, int R, bool MASKED>
 __global__ __launch_bounds__(kNW* kWave) void slot_kernel3(const int32_t* __restrict__ recs, const void* __restrict__ a0,
-                                                           const void* __restrict__ b0, int aoff1, int aoff2, int boff1, int boff2,
-                                                           uint32_t widths01, uint32_t widths2, uint32_t packed,
+                                                           const void* __restrict__ b0, uint32_t aoff1, uint32_t aoff2, uint32_t boff1, uint32_t boff2,
+                                                           uint32_t off_high, uint32_t widths01, uint32_t widths2, uint32_t packed,
                                                            const void* __restrict__ xv, void* __restrict__ yv_, int64_t xs, int64_t ys,
                                                            int y_col0, int y_col1, int y_col2, uint32_t check, float scaling,
                                                            const int32_t* __restrict__ eff_rank, int32_t* __restrict__ plan_hdr) {
@@ -628,7 +629,10 @@ __global__ __launch_bounds__(kNW* kWave) void slot_kernel3(const int32_t* __rest
   const int cum1 = static_cast<int>((widths2 >> 16) & 255u), cum2 = static_cast<int>(widths2 >> 24);
   const int ri = blockIdx.y;
   const int slice = int(ri >= cum1) + int(ri >= cum2);
-  const int64_t ao = slice == 0 ? 0 : slice == 1 ? aoff1 : aoff2, bo = slice == 0 ? 0 : slice == 1 ? boff1 : boff2;
+  // (offset i: low word off_i, bits 32..39 in byte i of off_high, sign-extended)
+  const uint32_t alo = slice == 1 ? aoff1 : aoff2, blo = slice == 1 ? boff1 : boff2;
+  const int32_t ahi = static_cast<int8_t>(off_high >> (slice == 1 ? 0 : 8)), bhi = static_cast<int8_t>(off_high >> (slice == 1 ? 16 : 24));
+  const int64_t ao = slice == 0 ? 0 : (static_cast<int64_t>(ahi) << 32) | alo, bo = slice == 0 ? 0 : (static_cast<int64_t>(bhi) << 32) | blo;
   Range sp;
   sp.a = static_cast<const char*>(a0) + ao * 16;
   sp.b = static_cast<const char*>(b0) + bo * 16;
@@ -659,36 +663,39 @@ struct Launch {
   int spin_ticks, trusted;
 };
 
-// Offsets of slice i's A and B from slice 0's, in units of 16 bytes, when they fit 32 bits.
-bool offsets16(const MloraAddArgs* a, int i, int* ao, int* bo) {
+// Offsets of slice i's A and B from slice 0's, in units of 16 bytes, when they fit 40 bits.
+bool offsets16(const MloraAddArgs* a, int i, long long* ao, long long* bo) {
   const long long da = static_cast<const char*>(a->slices[i].a) - static_cast<const char*>(a->slices[0].a);
   const long long db = static_cast<const char*>(a->slices[i].b) - static_cast<const char*>(a->slices[0].b);
   if ((da & 15) || (db & 15)) return false;
-  const long long qa = da / 16, qb = db / 16;
-  if (qa < INT32_MIN || qa > INT32_MAX || qb < INT32_MIN || qb > INT32_MAX) return false;
-  *ao = static_cast<int>(qa);
-  *bo = static_cast<int>(qb);
+  const long long qa = da / 16, qb = db / 16, lim = 1ll << 39;
+  if (qa < -lim || qa >= lim || qb < -lim || qb >= lim) return false;
+  *ao = qa;
+  *bo = qb;
   return true;
 }
 
 template <typename T, int R>
 void launch_three(const MloraAddArgs* a, dim3 grid, int nt, int cum1, int cum2) {
   const PlanLayout lay = plan_layout(a->num_tokens, a->num_slots);
-  int ao1 = 0, ao2 = 0, bo1 = 0, bo2 = 0;
-  (void)offsets16(a, 1, &ao1, &bo1);
-  (void)offsets16(a, 2, &ao2, &bo2);
+  long long o[4] = {0, 0, 0, 0};  // A of slices 1 and 2, B of slices 1 and 2
+  (void)offsets16(a, 1, &o[0], &o[2]);
+  (void)offsets16(a, 2, &o[1], &o[3]);
+  const uint32_t ao1 = static_cast<uint32_t>(o[0]), ao2 = static_cast<uint32_t>(o[1]), bo1 = static_cast<uint32_t>(o[2]), bo2 = static_cast<uint32_t>(o[3]);
+  uint32_t high = 0;
+  for (int i = 0; i < 4; ++i) high |= static_cast<uint32_t>((o[i] >> 32) & 0xff) << (8 * i);
   const uint32_t w01 = static_cast<uint32_t>(a->slices[0].n / 8) | (static_cast<uint32_t>(a->slices[1].n / 8) << 16);
   const uint32_t w2 = static_cast<uint32_t>(a->slices[2].n / 8) | (static_cast<uint32_t>(cum1) << 16) | (static_cast<uint32_t>(cum2) << 24);
   const uint32_t packed = static_cast<uint32_t>(nt / 64) | (static_cast<uint32_t>(a->num_slots) << 16);
   const uint32_t check = static_cast<uint32_t>(MLORA_PLAN_CHECK(a->num_tokens, a->num_slots));
   if (a->effective_rank)
     hipLaunchKernelGGL((slot_kernel3<T, R, true>), grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream), a->plan + lay.slotrec_off,
-                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
+                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, high, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
                        a->slices[0].y_col, a->slices[1].y_col, a->slices[2].y_col, check, a->scaling, a->effective_rank,
                        const_cast<int32_t*>(a->plan));
   else
     hipLaunchKernelGGL((slot_kernel3<T, R, false>), grid, dim3(kNW * kWave), 0, static_cast<hipStream_t>(a->stream), a->plan + lay.slotrec_off,
-                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
+                       a->slices[0].a, a->slices[0].b, ao1, ao2, bo1, bo2, high, w01, w2, packed, a->x, a->y, a->x_stride, a->y_stride,
                        a->slices[0].y_col, a->slices[1].y_col, a->slices[2].y_col, check, a->scaling, a->effective_rank,
                        const_cast<int32_t*>(a->plan));
 }
@@ -820,9 +827,9 @@ bool slot_supported(const MloraAddArgs* a) {
   if (!padded_rank(a->r)) return false;
   const int kspw = kspw_of(a);
   if (a->num_slices == 3) {
-    // q | k | v: K = 1024, an exact rank, offsets that fit 32 bits, widths that fit 16-bit counts of
+    // q | k | v: K = 1024, an exact rank, offsets that fit 40 bits, widths that fit 16-bit counts of
     // eight columns, and column ranges of at most 512 columns (one span per wavefront)
-    int ao, bo;
+    long long ao, bo;
     if (kspw != 4 || !exact_rank(a->r) || !offsets16(a, 1, &ao, &bo) || !offsets16(a, 2, &ao, &bo)) return false;
     for (int i = 0; i < 3; ++i)
       if (a->slices[i].n % 8 || a->slices[i].n / 8 > 0xffff) return false;

@@ -1264,3 +1264,56 @@ def test_graph_replays_of_the_shared_and_the_two_launch_forms(name, tokens, rank
         exact, mag = _exact(proj, x, y0, slots)
         _check(y_buf, y0, exact, mag, slots, f"graph/{name}/T{tokens}/step{step}")
         assert torch.equal(y_buf, eager), f"replay {step} differs from the eager call"
+
+
+def test_slot_major_grid_takes_three_slices_that_lie_far_apart():
+    """The three-slice kernel gets the second and third slice's weight pointers as 40-bit offsets
+    (units of 16 bytes) from the first one's.  The slices of a projection are allocations of their
+    own; here the first slice's buffers lie at the start of a 36 GiB allocation and the others' at
+    its end, so the offsets do not fit 32 bits.  The result is the oracle's and, bit for bit, the
+    tile-major grid's."""
+    from nanovllm_voxcpm_amd import synthetic
+
+    print("slot-major qkv, slices 36 GiB apart", flush=True)
+    free, _ = torch.cuda.mem_get_info()
+    if free < (48 << 30):
+        pytest.skip("needs 48 GiB of free device memory")
+    L, rank, T = 8, 16, 64
+    base = _make("qkv", L, rank, torch.bfloat16, seed=1400)
+    arena = torch.empty(36 << 30, dtype=torch.uint8, device="cuda")
+    cursor = [arena.numel()]
+
+    def at_the_end(t):  # a copy of t in the arena, carved from its end (256-byte aligned)
+        nbytes = (t.numel() * t.element_size() + 255) & ~255
+        cursor[0] -= nbytes
+        view = arena[cursor[0] : cursor[0] + t.numel() * t.element_size()].view(t.dtype).view(t.shape)
+        view.copy_(t)
+        return view
+
+    def at_the_start(t, offset):
+        view = arena[offset : offset + t.numel() * t.element_size()].view(t.dtype).view(t.shape)
+        view.copy_(t)
+        return view
+
+    a0 = at_the_start(base.a[0], 0)
+    b0 = at_the_start(base.b[0], (base.a[0].numel() * 2 + 255) & ~255)
+    proj = synthetic.ProjectionWeights("qkv", base.k, list(base.widths), [a0, at_the_end(base.a[1]), at_the_end(base.a[2])],
+                                       [b0, at_the_end(base.b[1]), at_the_end(base.b[2])])
+    gaps = [proj.a[i].data_ptr() - proj.a[0].data_ptr() for i in (1, 2)] + [proj.b[i].data_ptr() - proj.b[0].data_ptr() for i in (1, 2)]
+    assert min(gaps) > (32 << 30)
+    x, y0 = synthetic.make_activations(T, proj.k, sum(proj.widths), torch.bfloat16, seed=1401, device="cuda")
+    slots = synthetic.decode_slots(T, L, seed=1402).cuda()
+    got = _apply("slot", proj, x, y0.clone(), slots)
+    exact, mag = _exact(proj, x, y0, slots)
+    _check(got, y0, exact, mag, slots, "slot-major/qkv/far apart")
+    assert torch.equal(got, _apply("mfma", proj, x, y0.clone(), slots))
+    # and with the later slices in front of the first one (negative offsets)
+    back = synthetic.ProjectionWeights("qkv", base.k, list(base.widths), [proj.a[1], a0, proj.a[2]], [proj.b[1], b0, proj.b[2]])
+    back.widths = [base.widths[1], base.widths[0], base.widths[2]]
+    y1 = torch.randn(T, sum(back.widths), generator=torch.Generator().manual_seed(1403)).to(torch.bfloat16).cuda()
+    got = _apply("slot", back, x, y1.clone(), slots)
+    exact, mag = _exact(back, x, y1, slots)
+    _check(got, y1, exact, mag, slots, "slot-major/qkv/far apart, first slice last in memory")
+    torch.cuda.synchronize()
+    del proj, back, a0, b0, arena
+    torch.cuda.empty_cache()
