@@ -47,8 +47,8 @@ extern "C" {
                               out its shrink, seal what they wrote to the workspace, wait for each other's seals
                               and expand a column range each; needs an initialised workspace */
 #define MLORA_FORM_SLOT 7  /* MLORA_FORM_MFMA with the grid laid over the slots instead of the tiles: the workgroup of
-                              (slot, column range) requests A[slot] and B[slot] from its own index alone, before the
-                              record of the slot's first sixteen tokens has arrived; further tiles of a slot are
+                              (slot, column range) requests A[slot] from its own index alone, before the record of the
+                              slot's first sixteen tokens has arrived; further tiles of a slot are
                               taken by extra workgroups of the same launch */
 
 #define MLORA_FORM_WIDE 8  /* the tiles of MLORA_FORM_SGMV in one launch without anything passing between workgroups:

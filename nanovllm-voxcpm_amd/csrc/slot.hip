@@ -11,12 +11,15 @@
 // More than half of a decode launch's bytes are A[slot] and B[slot], and their addresses need the
 // slot id only.  Here the slot id IS the workgroup index: workgroup (x, range, z) serves slot
 // 8 z + x, so it requests the slot's record (its first sixteen tokens) and right behind it, without
-// waiting, every A and B line it will need; the record is waited for while the weights are on
-// their way, and only the x and y rows (whose addresses are token indices) hang on it.  For that
+// waiting, every A line it will need; the record is waited for while they are on their way, and
+// only the x and y rows (whose addresses are token indices) hang on it.  The B rows, which need the
+// slot id alone as well, go out behind the x rows: nothing uses them before the expand, and a
+// compute unit hands over only so many requests at a time, so in front of the record's wait they
+// held the x rows up (gate_up: 32 KB of A and 32 KB of B per workgroup).  For that
 // to be true the weight pointers must not need a fetch either: they are leading kernel arguments,
 // which arrive preloaded in scalar registers with the wavefront (14 dwords: the record list, two
 // slices' A and B, their widths, and a packed word).  A slot without tokens costs its workgroups
-// the weight lines they requested in vain; they leave as soon as the record says so.
+// the A lines they requested in vain; they leave as soon as the record says so.
 //
 // Tiles behind a slot's first sixteen tokens are taken by further workgroups of the same launch
 // (z beyond the slot layers), which learn their slot from their record like the tile-major
@@ -51,7 +54,7 @@ struct Range {
   int n, y_col, n0, n1;
 };
 
-// One tile.  EARLY: the slot is known from the workgroup index (slot_early) and the weights are
+// One tile.  EARLY: the slot is known from the workgroup index (slot_early) and A[slot] is
 // requested before the record has arrived; otherwise the record names the slot.
 // The operand path is the staged one of decode.hip: x rows and A rows of a wavefront's K range are
 // fetched row-contiguously (sixteen lanes per 256 bytes of a row), turned into MFMA operand layout
